@@ -1,0 +1,270 @@
+// extern "C" surface of the kernel manager (see include/es_km.h).  Converts the flat
+// descriptor arguments into IR values, forwards to es::kernel_manager_t and maps exceptions to
+// return codes.
+#include "../../include/es_km.h"
+
+#include "codegen.h"
+#include "kernel_manager.h"
+
+#include <cstring>
+
+struct es_km {
+    std::unique_ptr<es::kernel_manager_t> km;
+    std::string                           last_error;
+};
+
+namespace
+{
+
+thread_local std::string g_null_error;
+
+std::string& err_slot(es_km_t* h) { return h ? h->last_error : g_null_error; }
+
+// Key of the descriptor exactly as passed by the caller; cheap to build on the hot path.
+std::string raw_key(const uint64_t* join_shape, int join_rank, const int* inns_flat,
+                    const int* inns_offsets, int n_inns, int out_rank, const char* join_text,
+                    char castable)
+{
+    std::string k;
+    k.reserve(96 + std::strlen(join_text));
+    k.append(reinterpret_cast<const char*>(join_shape), sizeof(uint64_t) * size_t(join_rank));
+    k.push_back('|');
+    k.append(reinterpret_cast<const char*>(inns_offsets), sizeof(int) * size_t(n_inns + 1));
+    k.append(reinterpret_cast<const char*>(inns_flat), sizeof(int) * size_t(inns_offsets[n_inns]));
+    k.push_back('|');
+    k.push_back(char('0' + out_rank));
+    k.push_back(castable ? castable : ':');
+    k.append(join_text);
+    return k;
+}
+
+void check_descriptor(const uint64_t* join_shape, int join_rank, const int* inns_flat,
+                      const int* inns_offsets, int n_inns, int out_rank, const char* join_text)
+{
+    if (!join_shape || !inns_flat || !inns_offsets || !join_text) {
+        throw es::ir_error("einsummable descriptor: null argument");
+    }
+    if (join_rank < 1 || join_rank > 32 || n_inns < 1 || n_inns > 32 || out_rank < 1) {
+        throw es::ir_error("einsummable descriptor: bad rank or input count");
+    }
+    if (inns_offsets[0] != 0) throw es::ir_error("einsummable descriptor: inns_offsets[0] != 0");
+    for (int k = 0; k != n_inns; ++k) {
+        if (inns_offsets[k + 1] < inns_offsets[k] || inns_offsets[k + 1] > 1024) {
+            throw es::ir_error("einsummable descriptor: inns_offsets not monotone");
+        }
+    }
+}
+
+es::einsummable_t make_einsummable(const uint64_t* join_shape, int join_rank,
+                                   const int* inns_flat, const int* inns_offsets, int n_inns,
+                                   int out_rank, const char* join_text, char castable)
+{
+    std::vector<uint64_t>         shape(join_shape, join_shape + join_rank);
+    std::vector<std::vector<int>> inns;
+    for (int k = 0; k != n_inns; ++k) {
+        inns.emplace_back(inns_flat + inns_offsets[k], inns_flat + inns_offsets[k + 1]);
+    }
+    return es::einsummable_t::make(std::move(shape), std::move(inns), out_rank,
+                                   es::scalarop_t::parse(join_text),
+                                   es::castable_from_char(castable));
+}
+
+template <typename F>
+int guarded(es_km_t* h, F&& f)
+{
+    try {
+        return f();
+    } catch (es::km_error const& e) {
+        err_slot(h) = e.what();
+        return int(e.status);
+    } catch (es::ir_error const& e) {
+        err_slot(h) = e.what();
+        return ES_KM_ERR_INVALID;
+    } catch (std::exception const& e) {
+        err_slot(h) = e.what();
+        return ES_KM_ERR_DEVICE;
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+es_km_t* es_km_create(int device)
+{
+    try {
+        auto* h = new es_km;
+        h->km = std::make_unique<es::kernel_manager_t>(device);
+        return h;
+    } catch (std::exception const& e) {
+        g_null_error = e.what();
+        return nullptr;
+    }
+}
+
+void es_km_destroy(es_km_t* km) { delete km; }
+
+const char* es_km_last_error(es_km_t* km) { return err_slot(km).c_str(); }
+
+int es_km_build(es_km_t* h, const uint64_t* join_shape, int join_rank, const int* inns_flat,
+                const int* inns_offsets, int n_inns, int out_rank, const char* join_text,
+                char castable, uint64_t* workspace_bytes)
+{
+    return guarded(h, [&]() -> int {
+        if (!h) throw es::ir_error("null handle");
+        check_descriptor(join_shape, join_rank, inns_flat, inns_offsets, n_inns, out_rank,
+                         join_text);
+        es::einsummable_t e = make_einsummable(join_shape, join_rank, inns_flat, inns_offsets,
+                                               n_inns, out_rank, join_text, castable);
+        auto ws = h->km->build(e);
+        if (!ws) {
+            h->last_error = "build: no kernel for einsummable " + e.key();
+            return ES_KM_UNSUPPORTED;
+        }
+        h->km->alias_raw(raw_key(join_shape, join_rank, inns_flat, inns_offsets, n_inns, out_rank,
+                                 join_text, castable),
+                         e);
+        if (workspace_bytes) *workspace_bytes = ws.value();
+        return ES_KM_OK;
+    });
+}
+
+int es_km_workspace_size(es_km_t* h, const uint64_t* join_shape, int join_rank,
+                         const int* inns_flat, const int* inns_offsets, int n_inns, int out_rank,
+                         const char* join_text, char castable, uint64_t* workspace_bytes)
+{
+    return guarded(h, [&]() -> int {
+        if (!h) throw es::ir_error("null handle");
+        check_descriptor(join_shape, join_rank, inns_flat, inns_offsets, n_inns, out_rank,
+                         join_text);
+        es::plan_t const* p = h->km->find_raw(raw_key(join_shape, join_rank, inns_flat,
+                                                      inns_offsets, n_inns, out_rank, join_text,
+                                                      castable));
+        uint64_t ws;
+        if (p) {
+            ws = p->workspace_bytes;
+        } else {
+            ws = h->km->workspace_size(make_einsummable(join_shape, join_rank, inns_flat,
+                                                        inns_offsets, n_inns, out_rank, join_text,
+                                                        castable));
+        }
+        if (workspace_bytes) *workspace_bytes = ws;
+        return ES_KM_OK;
+    });
+}
+
+int es_km_execute(es_km_t* h, const uint64_t* join_shape, int join_rank, const int* inns_flat,
+                  const int* inns_offsets, int n_inns, int out_rank, const char* join_text,
+                  char castable, void* stream, void* out, const void* const* inns,
+                  int n_inn_ptrs, void* workspace, uint64_t workspace_bytes)
+{
+    return guarded(h, [&]() -> int {
+        if (!h) throw es::ir_error("null handle");
+        check_descriptor(join_shape, join_rank, inns_flat, inns_offsets, n_inns, out_rank,
+                         join_text);
+        if (!out || !inns) throw es::ir_error("execute: null buffer");
+        es::plan_t const* p = h->km->find_raw(raw_key(join_shape, join_rank, inns_flat,
+                                                      inns_offsets, n_inns, out_rank, join_text,
+                                                      castable));
+        if (p) {
+            h->km->run_plan(*p, static_cast<hipStream_t>(stream), out, inns, n_inn_ptrs, workspace,
+                            workspace_bytes);
+            return ES_KM_OK;
+        }
+        // Not seen under this spelling: an equal einsummable may still have been built
+        // (two descriptors that merge to the same form share a kernel).
+        es::einsummable_t e = make_einsummable(join_shape, join_rank, inns_flat, inns_offsets,
+                                               n_inns, out_rank, join_text, castable);
+        std::vector<void const*> v(inns, inns + n_inn_ptrs);
+        std::optional<std::tuple<void*, uint64_t>> ws;
+        if (workspace) ws = std::make_tuple(workspace, workspace_bytes);
+        (*h->km)(e, static_cast<hipStream_t>(stream), out, v, ws);
+        return ES_KM_OK;
+    });
+}
+
+int es_km_describe(es_km_t* h, const uint64_t* join_shape, int join_rank, const int* inns_flat,
+                   const int* inns_offsets, int n_inns, int out_rank, const char* join_text,
+                   char castable, char* out, size_t cap)
+{
+    return guarded(h, [&]() -> int {
+        if (!h) throw es::ir_error("null handle");
+        check_descriptor(join_shape, join_rank, inns_flat, inns_offsets, n_inns, out_rank,
+                         join_text);
+        std::string d = h->km->describe(make_einsummable(join_shape, join_rank, inns_flat,
+                                                         inns_offsets, n_inns, out_rank, join_text,
+                                                         castable));
+        if (!out || cap == 0) throw es::ir_error("describe: no output buffer");
+        std::strncpy(out, d.c_str(), cap - 1);
+        out[cap - 1] = 0;
+        return ES_KM_OK;
+    });
+}
+
+int es_km_touch(es_km_t* h, const uint64_t* touchdims, int rank, char castable, int dtype,
+                void* stream, void* out, const void* inn)
+{
+    return guarded(h, [&]() -> int {
+        if (!h) throw es::ir_error("null handle");
+        if (!touchdims || rank < 1 || rank > 64) throw es::ir_error("touch: bad selection");
+        if (dtype < 0 || dtype > 3) throw es::ir_error("touch: bad dtype");
+        if (!out || !inn) throw es::ir_error("touch: null buffer");
+        es::touch_t t;
+        t.dtype = es::dtype_t(dtype);
+        t.castable = es::castable_from_char(castable);
+        t.selection.resize(size_t(rank));
+        for (int i = 0; i != rank; ++i) {
+            const uint64_t* d = touchdims + 5 * i;
+            t.selection[i] = es::touchdim_t{d[0], d[1], d[2], d[3], d[4]};
+        }
+        (*h->km)(t, static_cast<hipStream_t>(stream), out, inn);
+        return ES_KM_OK;
+    });
+}
+
+int es_km_fill_constant(es_km_t* h, int dtype, uint64_t value_bits, uint64_t nelem, void* stream,
+                        void* out)
+{
+    return guarded(h, [&]() -> int {
+        if (!h) throw es::ir_error("null handle");
+        if (dtype < 0 || dtype > 3) throw es::ir_error("fill: bad dtype");
+        if (!out) throw es::ir_error("fill: null buffer");
+        h->km->constant_fill(es::dtype_t(dtype), value_bits, nelem,
+                             static_cast<hipStream_t>(stream), out);
+        return ES_KM_OK;
+    });
+}
+
+int es_km_fill_lowertri(es_km_t* h, int dtype, uint64_t lower_bits, uint64_t upper_bits,
+                        uint64_t nrow, uint64_t ncol, int64_t start, void* stream, void* out)
+{
+    return guarded(h, [&]() -> int {
+        if (!h) throw es::ir_error("null handle");
+        if (dtype < 0 || dtype > 3) throw es::ir_error("fill: bad dtype");
+        if (!out) throw es::ir_error("fill: null buffer");
+        h->km->lowerTri_fill(es::dtype_t(dtype), lower_bits, upper_bits, nrow, ncol, start,
+                             static_cast<hipStream_t>(stream), out);
+        return ES_KM_OK;
+    });
+}
+
+int es_km_codegen_source(const uint64_t* join_shape, int join_rank, const int* inns_flat,
+                         const int* inns_offsets, int n_inns, int out_rank, const char* join_text,
+                         char castable, int compile, char* out, size_t cap)
+{
+    return guarded(nullptr, [&]() -> int {
+        check_descriptor(join_shape, join_rank, inns_flat, inns_offsets, n_inns, out_rank,
+                         join_text);
+        es::einsummable_t e = make_einsummable(join_shape, join_rank, inns_flat, inns_offsets,
+                                               n_inns, out_rank, join_text, castable)
+                                  .merge_adjacent_dims();
+        es::cg_kernel_t k = es::generate_kernel(e);
+        if (compile) es::compile_hip_source(k.source, "es_generated.hip", "gfx950");
+        if (out && cap) {
+            std::strncpy(out, k.source.c_str(), cap - 1);
+            out[cap - 1] = 0;
+        }
+        return ES_KM_OK;
+    });
+}
+}

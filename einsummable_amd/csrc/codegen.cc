@@ -1,0 +1,959 @@
+#include "codegen.h"
+
+#include "kernel_manager.h"
+
+#include <hip/hip_runtime.h>
+#include <hip/hiprtc.h>
+
+#include <algorithm>
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <sstream>
+
+namespace es
+{
+
+namespace
+{
+
+// ---------------------------------------------------------------- expression emission
+
+// Arithmetic type a node is evaluated in: f16 and f32 nodes in float (f16 results are rounded
+// once, when stored or at an explicit to_f16), f64 in double, c64 as a pair of floats.
+const char* compute_type(dtype_t d)
+{
+    switch (d) {
+        case dtype_t::f16:
+        case dtype_t::f32:
+            return "float";
+        case dtype_t::f64:
+            return "double";
+        case dtype_t::c64:
+            return "c64";
+    }
+    return "float";
+}
+
+const char* storage_type(dtype_t d)
+{
+    switch (d) {
+        case dtype_t::f16:
+            return "f16";
+        case dtype_t::f32:
+            return "float";
+        case dtype_t::f64:
+            return "double";
+        case dtype_t::c64:
+            return "c64";
+    }
+    return "float";
+}
+
+bool is_double(dtype_t d) { return d == dtype_t::f64; }
+
+std::string literal(dtype_t d, double v)
+{
+    char buf[96];
+    bool dbl = is_double(d);
+    if (std::isnan(v)) return dbl ? "__builtin_nan(\"\")" : "__builtin_nanf(\"\")";
+    if (std::isinf(v)) {
+        std::string s = dbl ? "__builtin_huge_val()" : "__builtin_huge_valf()";
+        return v < 0 ? "(-" + s + ")" : s;
+    }
+    std::snprintf(buf, sizeof(buf), dbl ? "(%a)" : "(%af)", v);
+    return buf;
+}
+
+struct emitter_t {
+    std::ostringstream body;
+    int                next = 0;
+
+    std::string fresh() { return "t" + std::to_string(next++); }
+
+    std::string define(dtype_t d, std::string const& rhs)
+    {
+        std::string v = fresh();
+        body << "    const " << compute_type(d) << " " << v << " = " << rhs << ";\n";
+        return v;
+    }
+
+    std::string emit(node_t const& n)
+    {
+        std::vector<std::string> c;
+        for (auto const& ch : n.children) c.push_back(emit(ch));
+        bool const dbl = is_double(n.dtype);
+        switch (n.kind) {
+            case op_kind::constant:
+                if (n.dtype == dtype_t::c64) {
+                    return define(n.dtype, "c64{" + literal(dtype_t::f32, n.re) + ", " +
+                                               literal(dtype_t::f32, n.im) + "}");
+                }
+                return define(n.dtype, literal(n.dtype, n.re));
+            case op_kind::hole:
+                return "x" + std::to_string(n.arg);
+            case op_kind::variable:
+                throw ir_error("scalarop with variables cannot be compiled");
+            case op_kind::add:
+                if (n.dtype == dtype_t::c64) return define(n.dtype, "c_add(" + c[0] + ", " + c[1] + ")");
+                return define(n.dtype, c[0] + " + " + c[1]);
+            case op_kind::mul:
+                if (n.dtype == dtype_t::c64) return define(n.dtype, "c_mul(" + c[0] + ", " + c[1] + ")");
+                return define(n.dtype, c[0] + " * " + c[1]);
+            case op_kind::exp:
+                return define(n.dtype, std::string(dbl ? "exp(" : "expf(") + c[0] + ")");
+            case op_kind::log:
+                return define(n.dtype, std::string(dbl ? "log(" : "logf(") + c[0] + ")");
+            case op_kind::power: {
+                // The exponent is used at the precision the reference gives it
+                // (scalarop.cc:711-726): rounded to f16 / f32 for those dtypes.
+                double p = n.power;
+                if (n.dtype == dtype_t::f16) p = double(_Float16(p));
+                if (n.dtype == dtype_t::f32) p = double(float(p));
+                std::string const& x = c[0];
+                std::string one = dbl ? "1.0" : "1.0f";
+                if (p == 1.0) return define(n.dtype, x);
+                if (p == 2.0) return define(n.dtype, x + " * " + x);
+                if (p == 3.0) return define(n.dtype, x + " * " + x + " * " + x);
+                if (p == -1.0) return define(n.dtype, one + " / " + x);
+                if (p == -2.0) return define(n.dtype, one + " / (" + x + " * " + x + ")");
+                if (p == 0.5) return define(n.dtype, std::string(dbl ? "sqrt(" : "sqrtf(") + x + ")");
+                if (p == -0.5) {
+                    return define(n.dtype, one + " / " + (dbl ? "sqrt(" : "sqrtf(") + x + ")");
+                }
+                return define(n.dtype, std::string(dbl ? "pow(" : "powf(") + x + ", " +
+                                           literal(n.dtype, p) + ")");
+            }
+            case op_kind::ite: {
+                static const char* cmp[] = {"<", ">", "==", "<=", ">="};
+                return define(n.dtype, "(" + c[0] + " " + cmp[int(n.compare)] + " " + c[1] +
+                                           ") ? " + c[2] + " : " + c[3]);
+            }
+            case op_kind::convert: {
+                dtype_t from = n.children[0].dtype;
+                if (n.dtype == dtype_t::f16) return define(n.dtype, "(float)(f16)(" + c[0] + ")");
+                if (n.dtype == dtype_t::f32) {
+                    return define(n.dtype, from == dtype_t::f64 ? "(float)(" + c[0] + ")" : c[0]);
+                }
+                return define(n.dtype, "(double)(" + c[0] + ")");
+            }
+            case op_kind::conj:
+                return define(n.dtype, "c64{" + c[0] + ".re, -" + c[0] + ".im}");
+            case op_kind::real:
+                return define(n.dtype, c[0] + ".re");
+            case op_kind::imag:
+                return define(n.dtype, c[0] + ".im");
+            case op_kind::cplex:
+                return define(n.dtype, "c64{" + c[0] + ", " + c[1] + "}");
+        }
+        throw ir_error("emit: bad node");
+    }
+};
+
+const char* PRELUDE = R"(
+typedef _Float16 f16;
+struct c64 { float re, im; };
+__device__ __forceinline__ c64 c_add(c64 a, c64 b) { return c64{a.re + b.re, a.im + b.im}; }
+__device__ __forceinline__ c64 c_mul(c64 a, c64 b)
+{
+    return c64{a.re * b.re - a.im * b.im, a.re * b.im + a.im * b.re};
+}
+template <typename T, int N>
+struct __attribute__((aligned(sizeof(T) * N))) vec_t { T v[N]; };
+__device__ __forceinline__ float  cvt_in(f16 v) { return (float)v; }
+__device__ __forceinline__ float  cvt_in(float v) { return v; }
+__device__ __forceinline__ double cvt_in(double v) { return v; }
+__device__ __forceinline__ c64    cvt_in(c64 v) { return v; }
+__device__ __forceinline__ float  lane_xor(float v, int m) { return __shfl_xor(v, m); }
+__device__ __forceinline__ double lane_xor(double v, int m) { return __shfl_xor(v, m); }
+__device__ __forceinline__ c64    lane_xor(c64 v, int m)
+{
+    return c64{__shfl_xor(v.re, m), __shfl_xor(v.im, m)};
+}
+)";
+
+// how one input sees the vectorised mode
+enum class access_t { straight, vec, bcast, gather };
+
+struct layout_t {
+    int                                R = 0;  // join rank
+    int                                O = 0;  // out rank
+    int                                NI = 0;
+    std::vector<uint64_t>              shape;
+    std::vector<std::vector<uint64_t>> stride;  // [input][join mode], 0 when absent
+};
+
+layout_t make_layout(einsummable_t const& e)
+{
+    layout_t L;
+    L.R = int(e.join_shape.size());
+    L.O = e.out_rank;
+    L.NI = int(e.inns.size());
+    L.shape = e.join_shape;
+    L.stride.assign(size_t(L.NI), std::vector<uint64_t>(size_t(L.R), 0));
+    for (int k = 0; k != L.NI; ++k) {
+        uint64_t s = 1;
+        for (int i = int(e.inns[k].size()) - 1; i >= 0; --i) {
+            L.stride[k][e.inns[k][i]] = s;
+            s *= e.join_shape[e.inns[k][i]];
+        }
+    }
+    return L;
+}
+
+access_t classify(einsummable_t const& e, int k, int vmode, bool allow_straight)
+{
+    auto const& inn = e.inns[k];
+    if (allow_straight && int(inn.size()) == e.out_rank) {
+        bool straight = true;
+        for (size_t i = 0; i != inn.size(); ++i) straight = straight && inn[i] == int(i);
+        if (straight) return access_t::straight;
+    }
+    auto it = std::find(inn.begin(), inn.end(), vmode);
+    if (it == inn.end()) return access_t::bcast;
+    if (it + 1 == inn.end()) return access_t::vec;
+    return access_t::gather;
+}
+
+int pow2_divisor(uint64_t n, int cap)
+{
+    int v = 1;
+    while (v * 2 <= cap && n % uint64_t(v * 2) == 0) v *= 2;
+    return v;
+}
+
+std::string identity_of(castable_t c, dtype_t d)
+{
+    bool dbl = is_double(d);
+    if (d == dtype_t::c64) return c == castable_t::add ? "c64{0.0f, 0.0f}" : "c64{1.0f, 0.0f}";
+    switch (c) {
+        case castable_t::add:
+            return dbl ? "0.0" : "0.0f";
+        case castable_t::mul:
+            return dbl ? "1.0" : "1.0f";
+        case castable_t::min:
+            return dbl ? "__builtin_huge_val()" : "__builtin_huge_valf()";
+        case castable_t::max:
+            return dbl ? "(-__builtin_huge_val())" : "(-__builtin_huge_valf())";
+    }
+    return "0";
+}
+
+// acc <- castable(acc, v); min/max follow make_min / make_max (scalarop.cc:2267-2280)
+std::string combine_expr(castable_t c, dtype_t d, std::string const& a, std::string const& v)
+{
+    if (d == dtype_t::c64) {
+        return c == castable_t::add ? "c_add(" + a + ", " + v + ")" : "c_mul(" + a + ", " + v + ")";
+    }
+    switch (c) {
+        case castable_t::add:
+            return a + " + " + v;
+        case castable_t::mul:
+            return a + " * " + v;
+        case castable_t::min:
+            return "(" + a + " < " + v + ") ? " + a + " : " + v;
+        case castable_t::max:
+            return "(" + a + " > " + v + ") ? " + a + " : " + v;
+    }
+    return a;
+}
+
+struct gen_t {
+    einsummable_t const& e;
+    layout_t             L;
+    std::ostringstream   src;
+    cg_kernel_t          k;
+    int                  n_params = 0;
+
+    explicit gen_t(einsummable_t const& e_) : e(e_), L(make_layout(e_)) {}
+
+    int param(uint64_t v)
+    {
+        k.params.push_back(v);
+        return n_params++;
+    }
+
+    std::string P(int i) const { return "a.p[" + std::to_string(i) + "]"; }
+
+    void header()
+    {
+        src << PRELUDE;
+        src << "typedef " << (k.idx64 ? "unsigned long long" : "unsigned int") << " idx_t;\n";
+        // the join as a function of the (converted) inputs
+        emitter_t em;
+        std::string r = em.emit(e.join.root);
+        src << "__device__ __forceinline__ " << compute_type(e.out_dtype()) << " join_fn(";
+        for (int i = 0; i != L.NI; ++i) {
+            src << (i ? ", " : "") << compute_type(e.inn_dtype(i)) << " x" << i;
+        }
+        src << ")\n{\n" << em.body.str() << "    return " << r << ";\n}\n";
+    }
+
+    void args_struct()
+    {
+        src << "struct args_t {\n    " << storage_type(e.out_dtype()) << "* out;\n";
+        for (int i = 0; i != L.NI; ++i) {
+            src << "    const " << storage_type(e.inn_dtype(i)) << "* in" << i << ";\n";
+        }
+        src << "    idx_t p[" << std::max(n_params, 1) << "];\n};\n";
+    }
+
+    std::string store_cast(std::string const& v) const
+    {
+        if (e.out_dtype() == dtype_t::f16) return "(f16)(" + v + ")";
+        return v;
+    }
+};
+
+bool fits32(einsummable_t const& e)
+{
+    uint64_t const lim = (1ull << 32) - 1;
+    if (e.out_nelem() >= lim) return false;
+    for (int k = 0; k != int(e.inns.size()); ++k) {
+        if (e.inn_nelem(k) >= lim) return false;
+    }
+    uint64_t join = 1;
+    for (uint64_t d : e.join_shape) {
+        join *= d;
+        if (join >= (1ull << 62)) return false;
+    }
+    return true;
+}
+
+int min_elem_size(einsummable_t const& e)
+{
+    int m = int(dtype_size(e.out_dtype()));
+    for (int k = 0; k != int(e.inns.size()); ++k) m = std::min(m, int(dtype_size(e.inn_dtype(k))));
+    return m;
+}
+
+// ------------------------------------------------------------------------ elementwise
+//
+// One thread produces V consecutive elements of the innermost output mode; U such vectors
+// per thread, 256 lanes apart, all loads issued before the first store (so an output that
+// aliases a same-index input is safe).
+cg_kernel_t gen_elementwise(einsummable_t const& e, int max_vec)
+{
+    gen_t g(e);
+    auto& L = g.L;
+    int const R = L.R;
+    g.k.kind = cg_kind::elementwise;
+    g.k.n_inns = L.NI;
+    g.k.idx64 = !fits32(e);
+    g.k.entry = "es_kernel";
+
+    std::vector<access_t> acc(L.NI);
+    bool all_straight = true;
+    for (int k = 0; k != L.NI; ++k) {
+        acc[k] = classify(e, k, R - 1, true);
+        all_straight = all_straight && acc[k] == access_t::straight;
+    }
+    uint64_t const inner = L.shape[R - 1];
+    uint64_t const n_out = e.out_nelem();
+    int const vcap = std::min(max_vec, 16 / min_elem_size(e));
+    int V;
+    uint64_t tail = 0;
+    if (all_straight) {
+        // the whole tensor is one row: full vectors plus a scalar tail
+        V = (n_out >= uint64_t(vcap)) ? vcap : 1;
+        tail = n_out % uint64_t(V);
+    } else {
+        V = pow2_divisor(inner, vcap);
+    }
+    int const U = (L.NI <= 2) ? 4 : 2;
+    uint64_t const n_vec = all_straight ? n_out / uint64_t(V) : n_out / uint64_t(V);
+    g.k.vec = V;
+
+    int p_nvec = g.param(n_vec);
+    int p_vpr = g.param(all_straight ? n_vec : inner / uint64_t(V));
+    std::vector<int> p_shape(R);
+    for (int m = 0; m != R; ++m) p_shape[m] = g.param(L.shape[m]);
+    std::vector<std::vector<int>> p_str(L.NI, std::vector<int>(R, -1));
+    for (int k = 0; k != L.NI; ++k) {
+        if (acc[k] == access_t::straight) continue;
+        for (int m = 0; m != R; ++m) {
+            if (L.stride[k][m]) p_str[k][m] = g.param(L.stride[k][m]);
+        }
+    }
+
+    g.header();
+    g.args_struct();
+    auto& s = g.src;
+    s << "#define V " << V << "\n#define U " << U << "\n";
+    s << "extern \"C\" __global__ __launch_bounds__(256) void es_kernel(args_t a)\n{\n";
+    s << "    const idx_t n_vec = " << g.P(p_nvec) << ";\n";
+    for (int k = 0; k != L.NI; ++k) {
+        std::string T = storage_type(e.inn_dtype(k));
+        if (acc[k] == access_t::bcast) {
+            s << "    " << T << " s" << k << "[U];\n";
+        } else {
+            s << "    vec_t<" << T << ", V> r" << k << "[U];\n";
+        }
+    }
+    s << "    idx_t vid[U];\n    bool live[U];\n";
+    s << "#pragma unroll\n    for (int u = 0; u != U; ++u) {\n";
+    s << "        vid[u] = ((idx_t)blockIdx.x * U + u) * 256 + threadIdx.x;\n";
+    s << "        live[u] = vid[u] < n_vec;\n";
+    s << "        if (live[u]) {\n";
+    if (!all_straight) {
+        s << "            idx_t rem = vid[u];\n";
+        s << "            const idx_t c = (rem % " << g.P(p_vpr) << ") * V;\n";
+        s << "            rem /= " << g.P(p_vpr) << ";\n";
+        for (int m = R - 2; m >= 1; --m) {
+            s << "            const idx_t d" << m << " = rem % " << g.P(p_shape[m]) << ";\n";
+            s << "            rem /= " << g.P(p_shape[m]) << ";\n";
+        }
+        if (R >= 2) s << "            const idx_t d0 = rem;\n";
+    }
+    for (int k = 0; k != L.NI; ++k) {
+        std::string T = storage_type(e.inn_dtype(k));
+        if (acc[k] == access_t::straight) {
+            s << "            r" << k << "[u] = *reinterpret_cast<const vec_t<" << T
+              << ", V>*>(a.in" << k << " + vid[u] * V);\n";
+            continue;
+        }
+        std::string off = "0";
+        for (int m = 0; m != R - 1; ++m) {
+            if (p_str[k][m] >= 0) off += " + d" + std::to_string(m) + " * " + g.P(p_str[k][m]);
+        }
+        if (acc[k] == access_t::vec) {
+            s << "            r" << k << "[u] = *reinterpret_cast<const vec_t<" << T
+              << ", V>*>(a.in" << k << " + (" << off << " + c));\n";
+        } else if (acc[k] == access_t::bcast) {
+            s << "            s" << k << "[u] = a.in" << k << "[" << off << "];\n";
+        } else {
+            s << "            {\n                const idx_t o = " << off << " + c * "
+              << g.P(p_str[k][R - 1]) << ";\n";
+            s << "#pragma unroll\n                for (int j = 0; j != V; ++j) r" << k
+              << "[u].v[j] = a.in" << k << "[o + j * " << g.P(p_str[k][R - 1]) << "];\n";
+            s << "            }\n";
+        }
+    }
+    s << "        }\n    }\n";
+    s << "#pragma unroll\n    for (int u = 0; u != U; ++u) {\n        if (live[u]) {\n";
+    s << "            vec_t<" << storage_type(e.out_dtype()) << ", V> res;\n";
+    s << "#pragma unroll\n            for (int j = 0; j != V; ++j) {\n";
+    s << "                res.v[j] = " << g.store_cast([&] {
+        std::string call = "join_fn(";
+        for (int k = 0; k != L.NI; ++k) {
+            call += (k ? ", " : "");
+            if (acc[k] == access_t::bcast) {
+                call += "cvt_in(s" + std::to_string(k) + "[u])";
+            } else {
+                call += "cvt_in(r" + std::to_string(k) + "[u].v[j])";
+            }
+        }
+        return call + ")";
+    }()) << ";\n";
+    s << "            }\n";
+    s << "            *reinterpret_cast<vec_t<" << storage_type(e.out_dtype())
+      << ", V>*>(a.out + vid[u] * V) = res;\n";
+    s << "        }\n    }\n";
+    if (tail) {
+        s << "    if (blockIdx.x == 0 && threadIdx.x < " << tail << ") {\n";
+        s << "        const idx_t i = n_vec * V + threadIdx.x;\n";
+        s << "        a.out[i] = " << g.store_cast([&] {
+            std::string call = "join_fn(";
+            for (int k = 0; k != L.NI; ++k) {
+                call += std::string(k ? ", " : "") + "cvt_in(a.in" + std::to_string(k) + "[i])";
+            }
+            return call + ")";
+        }()) << ";\n    }\n";
+    }
+    s << "}\n";
+
+    g.k.source = s.str();
+    uint64_t per_block = 256ull * uint64_t(U);
+    g.k.grid = std::max<uint64_t>(1, (n_vec + per_block - 1) / per_block);
+    g.k.block = 256;
+    g.k.out_inn_align.push_back(V * int(dtype_size(e.out_dtype())));
+    for (int k = 0; k != L.NI; ++k) {
+        bool wide = acc[k] == access_t::straight || acc[k] == access_t::vec;
+        g.k.out_inn_align.push_back((wide ? V : 1) * int(dtype_size(e.inn_dtype(k))));
+    }
+    return std::move(g.k);
+}
+
+// --------------------------------------------------------------- reduce, aggregated modes
+// innermost: a team of TEAM lanes (one wavefront, or a 256-thread workgroup for long rows)
+// owns one output element, strides over the flattened aggregated index space in V-element
+// vectors, accumulates in float / double, then reduces across lanes with DPP shuffles and
+// across wavefronts through LDS.
+cg_kernel_t gen_reduce_row(einsummable_t const& e, int max_vec)
+{
+    gen_t g(e);
+    auto& L = g.L;
+    int const R = L.R, O = L.O;
+    g.k.kind = cg_kind::reduce_row;
+    g.k.n_inns = L.NI;
+    g.k.idx64 = !fits32(e);
+    g.k.entry = "es_kernel";
+    castable_t const cast = e.castable.value();
+    dtype_t const od = e.out_dtype();
+
+    std::vector<access_t> acc(L.NI);
+    for (int k = 0; k != L.NI; ++k) acc[k] = classify(e, k, R - 1, false);
+    uint64_t nA = 1;
+    for (int m = O; m != R; ++m) nA *= L.shape[m];
+    uint64_t const n_out = e.out_nelem();
+    int const vcap = std::min(max_vec, 16 / min_elem_size(e));
+    int const V = pow2_divisor(L.shape[R - 1], vcap);
+    uint64_t const nvecA = nA / uint64_t(V);
+    int const TEAM = (nvecA >= 512) ? 256 : 64;
+    int const BLOCK = 256;
+    int const U = (nvecA >= uint64_t(TEAM) * 4) ? 4 : ((nvecA >= uint64_t(TEAM) * 2) ? 2 : 1);
+    g.k.vec = V;
+
+    int p_nout = g.param(n_out);
+    int p_nvec = g.param(nvecA);
+    std::vector<int> p_shape(R);
+    for (int m = 0; m != R; ++m) p_shape[m] = g.param(L.shape[m]);
+    std::vector<std::vector<int>> p_str(L.NI, std::vector<int>(R, -1));
+    for (int k = 0; k != L.NI; ++k) {
+        for (int m = 0; m != R; ++m) {
+            if (L.stride[k][m]) p_str[k][m] = g.param(L.stride[k][m]);
+        }
+    }
+
+    g.header();
+    g.args_struct();
+    auto& s = g.src;
+    std::string ACC = compute_type(od);
+    s << "#define V " << V << "\n#define U " << U << "\n#define TEAM " << TEAM << "\n";
+    s << "__device__ __forceinline__ " << ACC << " comb(" << ACC << " x, " << ACC
+      << " y) { return " << combine_expr(cast, od, "x", "y") << "; }\n";
+    s << "extern \"C\" __global__ __launch_bounds__(" << BLOCK << ") void es_kernel(args_t a)\n{\n";
+    s << "    const idx_t n_out = " << g.P(p_nout) << ";\n";
+    s << "    const idx_t nvec = " << g.P(p_nvec) << ";\n";
+    s << "    const unsigned lane = threadIdx.x % TEAM;\n";
+    s << "    const idx_t row = (idx_t)blockIdx.x * (" << BLOCK << " / TEAM) + threadIdx.x / TEAM;\n";
+    s << "    " << ACC << " acc = " << identity_of(cast, od) << ";\n";
+    s << "    if (row < n_out) {\n";
+    s << "        idx_t rem = row;\n";
+    for (int m = O - 1; m >= 1; --m) {
+        s << "        const idx_t d" << m << " = rem % " << g.P(p_shape[m]) << ";\n";
+        s << "        rem /= " << g.P(p_shape[m]) << ";\n";
+    }
+    s << "        const idx_t d0 = rem;\n";
+    for (int k = 0; k != L.NI; ++k) {
+        std::string off = "0";
+        for (int m = 0; m != O; ++m) {
+            if (p_str[k][m] >= 0) off += " + d" + std::to_string(m) + " * " + g.P(p_str[k][m]);
+        }
+        s << "        const idx_t b" << k << " = " << off << ";\n";
+    }
+    // inputs without any aggregated mode are loaded once per row
+    std::vector<bool> row_const(L.NI, true);
+    for (int k = 0; k != L.NI; ++k) {
+        for (int m = O; m != R; ++m) row_const[k] = row_const[k] && p_str[k][m] < 0;
+        if (row_const[k]) {
+            s << "        const " << compute_type(e.inn_dtype(k)) << " c" << k << " = cvt_in(a.in"
+              << k << "[b" << k << "]);\n";
+        }
+    }
+    s << "        for (idx_t v0 = lane; v0 < nvec; v0 += (idx_t)TEAM * U) {\n";
+    for (int k = 0; k != L.NI; ++k) {
+        if (row_const[k]) continue;
+        std::string T = storage_type(e.inn_dtype(k));
+        if (acc[k] == access_t::bcast) {
+            s << "            " << T << " s" << k << "[U];\n";
+        } else {
+            s << "            vec_t<" << T << ", V> r" << k << "[U];\n";
+        }
+    }
+    s << "#pragma unroll\n            for (int u = 0; u != U; ++u) {\n";
+    s << "                const idx_t vv = v0 + (idx_t)u * TEAM;\n";
+    s << "                if (vv < nvec) {\n";
+    s << "                    idx_t ar = vv * V;\n";
+    s << "                    const idx_t g" << (R - 1) << " = ar % " << g.P(p_shape[R - 1]) << ";\n";
+    if (R - 1 > O) s << "                    ar /= " << g.P(p_shape[R - 1]) << ";\n";
+    for (int m = R - 2; m > O; --m) {
+        s << "                    const idx_t g" << m << " = ar % " << g.P(p_shape[m]) << ";\n";
+        s << "                    ar /= " << g.P(p_shape[m]) << ";\n";
+    }
+    if (R - 1 > O) s << "                    const idx_t g" << O << " = ar;\n";
+    for (int k = 0; k != L.NI; ++k) {
+        if (row_const[k]) continue;
+        std::string T = storage_type(e.inn_dtype(k));
+        std::string off = "b" + std::to_string(k);
+        for (int m = O; m != R - 1; ++m) {
+            if (p_str[k][m] >= 0) off += " + g" + std::to_string(m) + " * " + g.P(p_str[k][m]);
+        }
+        if (acc[k] == access_t::vec) {
+            s << "                    r" << k << "[u] = *reinterpret_cast<const vec_t<" << T
+              << ", V>*>(a.in" << k << " + (" << off << " + g" << (R - 1) << "));\n";
+        } else if (acc[k] == access_t::bcast) {
+            s << "                    s" << k << "[u] = a.in" << k << "[" << off << "];\n";
+        } else {
+            s << "#pragma unroll\n                    for (int j = 0; j != V; ++j) r" << k
+              << "[u].v[j] = a.in" << k << "[" << off << " + (g" << (R - 1) << " + j) * "
+              << g.P(p_str[k][R - 1]) << "];\n";
+        }
+    }
+    s << "                }\n            }\n";
+    s << "#pragma unroll\n            for (int u = 0; u != U; ++u) {\n";
+    s << "                if (v0 + (idx_t)u * TEAM < nvec) {\n";
+    s << "#pragma unroll\n                    for (int j = 0; j != V; ++j) {\n";
+    s << "                        acc = comb(acc, join_fn(";
+    for (int k = 0; k != L.NI; ++k) {
+        s << (k ? ", " : "");
+        if (row_const[k]) {
+            s << "c" << k;
+        } else if (acc[k] == access_t::bcast) {
+            s << "cvt_in(s" << k << "[u])";
+        } else {
+            s << "cvt_in(r" << k << "[u].v[j])";
+        }
+    }
+    s << "));\n                    }\n                }\n            }\n";
+    s << "        }\n    }\n";
+    s << "#pragma unroll\n    for (int m = 32; m >= 1; m >>= 1) acc = comb(acc, lane_xor(acc, m));\n";
+    if (TEAM == 256) {
+        s << "    __shared__ " << ACC << " part[4];\n";
+        s << "    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = acc;\n";
+        s << "    __syncthreads();\n";
+        s << "    if (threadIdx.x == 0 && row < n_out) {\n";
+        s << "        acc = comb(comb(part[0], part[1]), comb(part[2], part[3]));\n";
+        s << "        a.out[row] = " << g.store_cast("acc") << ";\n    }\n";
+    } else {
+        s << "    if (lane == 0 && row < n_out) a.out[row] = " << g.store_cast("acc") << ";\n";
+    }
+    s << "}\n";
+
+    g.k.source = s.str();
+    uint64_t rows_per_block = uint64_t(BLOCK / TEAM);
+    g.k.grid = (n_out + rows_per_block - 1) / rows_per_block;
+    g.k.block = unsigned(BLOCK);
+    g.k.out_inn_align.push_back(int(dtype_size(od)));
+    for (int k = 0; k != L.NI; ++k) {
+        bool wide = acc[k] == access_t::vec && !row_const[k];
+        g.k.out_inn_align.push_back((wide ? V : 1) * int(dtype_size(e.inn_dtype(k))));
+    }
+    return std::move(g.k);
+}
+
+// ------------------------------------------------------------- reduce, any other layout:
+// one thread owns V consecutive elements of the innermost output mode and walks the
+// aggregated modes serially (nested loops, one per aggregated mode).  Lanes stay coalesced
+// along the output's innermost mode.
+cg_kernel_t gen_reduce_col(einsummable_t const& e, int max_vec)
+{
+    gen_t g(e);
+    auto& L = g.L;
+    int const R = L.R, O = L.O;
+    g.k.kind = cg_kind::reduce_col;
+    g.k.n_inns = L.NI;
+    g.k.idx64 = !fits32(e);
+    g.k.entry = "es_kernel";
+    castable_t const cast = e.castable.value();
+    dtype_t const od = e.out_dtype();
+
+    std::vector<access_t> acc(L.NI);
+    bool any_vec = false;
+    for (int k = 0; k != L.NI; ++k) {
+        acc[k] = classify(e, k, O - 1, false);
+        any_vec = any_vec || acc[k] == access_t::vec;
+    }
+    uint64_t const n_out = e.out_nelem();
+    int const vcap = std::min(max_vec, 16 / min_elem_size(e));
+    // vectors only pay when some input is contiguous along the output's inner mode
+    int const V = any_vec ? pow2_divisor(L.shape[O - 1], vcap) : 1;
+    uint64_t const n_vec = n_out / uint64_t(V);
+    g.k.vec = V;
+
+    int p_nvec = g.param(n_vec);
+    int p_vpr = g.param(L.shape[O - 1] / uint64_t(V));
+    std::vector<int> p_shape(R);
+    for (int m = 0; m != R; ++m) p_shape[m] = g.param(L.shape[m]);
+    std::vector<std::vector<int>> p_str(L.NI, std::vector<int>(R, -1));
+    for (int k = 0; k != L.NI; ++k) {
+        for (int m = 0; m != R; ++m) {
+            if (L.stride[k][m]) p_str[k][m] = g.param(L.stride[k][m]);
+        }
+    }
+
+    g.header();
+    g.args_struct();
+    auto& s = g.src;
+    std::string ACC = compute_type(od);
+    s << "#define V " << V << "\n";
+    s << "__device__ __forceinline__ " << ACC << " comb(" << ACC << " x, " << ACC
+      << " y) { return " << combine_expr(cast, od, "x", "y") << "; }\n";
+    s << "extern \"C\" __global__ __launch_bounds__(256) void es_kernel(args_t a)\n{\n";
+    s << "    const idx_t vid = (idx_t)blockIdx.x * 256 + threadIdx.x;\n";
+    s << "    if (vid >= " << g.P(p_nvec) << ") return;\n";
+    s << "    idx_t rem = vid;\n";
+    s << "    const idx_t c = (rem % " << g.P(p_vpr) << ") * V;\n";
+    s << "    rem /= " << g.P(p_vpr) << ";\n";
+    for (int m = O - 2; m >= 1; --m) {
+        s << "    const idx_t d" << m << " = rem % " << g.P(p_shape[m]) << ";\n";
+        s << "    rem /= " << g.P(p_shape[m]) << ";\n";
+    }
+    if (O >= 2) s << "    const idx_t d0 = rem;\n";
+    for (int k = 0; k != L.NI; ++k) {
+        std::string off = "0";
+        for (int m = 0; m != O - 1; ++m) {
+            if (p_str[k][m] >= 0) off += " + d" + std::to_string(m) + " * " + g.P(p_str[k][m]);
+        }
+        if (p_str[k][O - 1] >= 0) off += " + c * " + g.P(p_str[k][O - 1]);
+        s << "    const idx_t b" << k << " = " << off << ";\n";
+    }
+    s << "    " << ACC << " acc[V];\n";
+    s << "#pragma unroll\n    for (int j = 0; j != V; ++j) acc[j] = " << identity_of(cast, od)
+      << ";\n";
+    std::string indent = "    ";
+    for (int m = O; m != R; ++m) {
+        s << indent << "for (idx_t g" << m << " = 0; g" << m << " != " << g.P(p_shape[m]) << "; ++g"
+          << m << ") {\n";
+        indent += "    ";
+    }
+    for (int k = 0; k != L.NI; ++k) {
+        std::string T = storage_type(e.inn_dtype(k));
+        std::string off = "b" + std::to_string(k);
+        for (int m = O; m != R; ++m) {
+            if (p_str[k][m] >= 0) off += " + g" + std::to_string(m) + " * " + g.P(p_str[k][m]);
+        }
+        if (acc[k] == access_t::vec) {
+            s << indent << "const vec_t<" << T << ", V> r" << k
+              << " = *reinterpret_cast<const vec_t<" << T << ", V>*>(a.in" << k << " + (" << off
+              << "));\n";
+        } else if (acc[k] == access_t::bcast) {
+            s << indent << "const " << T << " s" << k << " = a.in" << k << "[" << off << "];\n";
+        } else {
+            s << indent << "vec_t<" << T << ", V> r" << k << ";\n";
+            s << "#pragma unroll\n" << indent << "for (int j = 0; j != V; ++j) r" << k
+              << ".v[j] = a.in" << k << "[" << off << " + j * " << g.P(p_str[k][O - 1]) << "];\n";
+        }
+    }
+    s << "#pragma unroll\n" << indent << "for (int j = 0; j != V; ++j) acc[j] = comb(acc[j], join_fn(";
+    for (int k = 0; k != L.NI; ++k) {
+        s << (k ? ", " : "");
+        if (acc[k] == access_t::bcast) {
+            s << "cvt_in(s" << k << ")";
+        } else {
+            s << "cvt_in(r" << k << ".v[j])";
+        }
+    }
+    s << "));\n";
+    for (int m = O; m != R; ++m) {
+        indent.resize(indent.size() - 4);
+        s << indent << "}\n";
+    }
+    s << "    vec_t<" << storage_type(od) << ", V> res;\n";
+    s << "#pragma unroll\n    for (int j = 0; j != V; ++j) res.v[j] = " << g.store_cast("acc[j]")
+      << ";\n";
+    s << "    *reinterpret_cast<vec_t<" << storage_type(od) << ", V>*>(a.out + vid * V) = res;\n";
+    s << "}\n";
+
+    g.k.source = s.str();
+    g.k.grid = std::max<uint64_t>(1, (n_vec + 255) / 256);
+    g.k.block = 256;
+    g.k.out_inn_align.push_back(V * int(dtype_size(od)));
+    for (int k = 0; k != L.NI; ++k) {
+        bool wide = acc[k] == access_t::vec;
+        g.k.out_inn_align.push_back((wide ? V : 1) * int(dtype_size(e.inn_dtype(k))));
+    }
+    return std::move(g.k);
+}
+
+}  // namespace
+
+cg_kernel_t generate_kernel(einsummable_t const& e, int max_vec)
+{
+    if (e.join_shape.size() > 12 || e.inns.size() > 8) {
+        throw ir_error("generate_kernel: too many modes or inputs");
+    }
+    if (!e.has_aggregation()) return gen_elementwise(e, max_vec);
+    if (e.out_dtype() == dtype_t::c64 &&
+        (e.castable.value() == castable_t::min || e.castable.value() == castable_t::max)) {
+        throw ir_error("generate_kernel: min/max aggregation of complex values");
+    }
+    int const R = int(e.join_shape.size());
+    bool      row = false;
+    for (int k = 0; k != int(e.inns.size()); ++k) {
+        row = row || (!e.inns[k].empty() && e.inns[k].back() == R - 1);
+    }
+    return row ? gen_reduce_row(e, max_vec) : gen_reduce_col(e, max_vec);
+}
+
+std::vector<char> compile_hip_source(std::string const& source, std::string const& name,
+                                     std::string const& arch)
+{
+    hiprtcProgram prog;
+    if (hiprtcCreateProgram(&prog, source.c_str(), name.c_str(), 0, nullptr, nullptr) !=
+        HIPRTC_SUCCESS) {
+        throw km_error(km_status::device, "hiprtcCreateProgram failed");
+    }
+    std::string arch_opt = "--offload-arch=" + arch;
+    // packed-fp32 instruction selection is switched off for all device code of this library
+    const char* opts[] = {arch_opt.c_str(), "-O3",      "-std=c++17",       "-Xclang",
+                          "-target-feature", "-Xclang", "-packed-fp32-ops"};
+    int         n_opts = 7;
+    hiprtcResult rc = hiprtcCompileProgram(prog, n_opts, opts);
+    if (rc != HIPRTC_SUCCESS) {
+        size_t n = 0;
+        hiprtcGetProgramLogSize(prog, &n);
+        std::string log(n, 0);
+        if (n) hiprtcGetProgramLog(prog, &log[0]);
+        hiprtcDestroyProgram(&prog);
+        throw km_error(km_status::device, "runtime compile of " + name + " failed:\n" + log +
+                                              "\n---- source ----\n" + source);
+    }
+    size_t n = 0;
+    hiprtcGetCodeSize(prog, &n);
+    std::vector<char> code(n);
+    hiprtcGetCode(prog, code.data());
+    hiprtcDestroyProgram(&prog);
+    return code;
+}
+
+// ---------------------------------------------------------------------------- the plan
+
+namespace
+{
+
+struct module_cache_t {
+    std::mutex                                                    mu;
+    std::unordered_map<std::string, std::pair<hipModule_t, hipFunction_t>> by_source;
+};
+
+module_cache_t& module_cache()
+{
+    static module_cache_t c;
+    return c;
+}
+
+hipFunction_t load_kernel(cg_kernel_t const& k)
+{
+    auto&                       cache = module_cache();
+    std::lock_guard<std::mutex> lock(cache.mu);
+    auto                        it = cache.by_source.find(k.source);
+    if (it != cache.by_source.end()) return it->second.second;
+    std::vector<char> code = compile_hip_source(k.source, "es_generated.hip", "gfx950");
+    hipModule_t       mod;
+    hipError_t        err = hipModuleLoadData(&mod, code.data());
+    if (err != hipSuccess) {
+        throw km_error(km_status::device,
+                       std::string("hipModuleLoadData: ") + hipGetErrorString(err));
+    }
+    hipFunction_t fn;
+    err = hipModuleGetFunction(&fn, mod, k.entry.c_str());
+    if (err != hipSuccess) {
+        throw km_error(km_status::device,
+                       std::string("hipModuleGetFunction: ") + hipGetErrorString(err));
+    }
+    cache.by_source.emplace(k.source, std::make_pair(mod, fn));
+    return fn;
+}
+
+struct variant_t {
+    cg_kernel_t   k;
+    hipFunction_t fn = nullptr;
+};
+
+struct codegen_plan_t : plan_t {
+    einsummable_t     e;
+    variant_t         wide;
+    mutable variant_t narrow;  // compiled on first use with a misaligned buffer
+    mutable std::mutex mu;
+
+    explicit codegen_plan_t(einsummable_t const& e_) : e(e_) {}
+
+    static void launch(variant_t const& v, hipStream_t stream, void* out, void const* const* inns)
+    {
+        // argument block: out pointer, input pointers, then idx_t parameters
+        unsigned char buf[1024];
+        size_t        n = 0;
+        std::memcpy(buf + n, &out, 8);
+        n += 8;
+        for (int i = 0; i != v.k.n_inns; ++i) {
+            std::memcpy(buf + n, &inns[i], 8);
+            n += 8;
+        }
+        if (v.k.idx64) {
+            for (uint64_t p : v.k.params) {
+                std::memcpy(buf + n, &p, 8);
+                n += 8;
+            }
+        } else {
+            for (uint64_t p : v.k.params) {
+                uint32_t q = uint32_t(p);
+                std::memcpy(buf + n, &q, 4);
+                n += 4;
+            }
+            n = (n + 7) & ~size_t(7);
+        }
+        void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, buf, HIP_LAUNCH_PARAM_BUFFER_SIZE, &n,
+                          HIP_LAUNCH_PARAM_END};
+        hipError_t err = hipModuleLaunchKernel(v.fn, unsigned(v.k.grid), 1, 1, v.k.block, 1, 1, 0,
+                                               stream, nullptr, config);
+        if (err != hipSuccess) {
+            throw km_error(km_status::device,
+                           std::string("hipModuleLaunchKernel: ") + hipGetErrorString(err));
+        }
+    }
+
+    static bool aligned(variant_t const& v, void* out, void const* const* inns)
+    {
+        if (reinterpret_cast<uintptr_t>(out) % uintptr_t(std::min(v.k.out_inn_align[0], 16))) {
+            return false;
+        }
+        for (int i = 0; i != v.k.n_inns; ++i) {
+            if (reinterpret_cast<uintptr_t>(inns[i]) %
+                uintptr_t(std::min(v.k.out_inn_align[1 + i], 16))) {
+                return false;
+            }
+        }
+        return true;
+    }
+
+    void run(hipStream_t stream, void* out, void const* const* inns, void*, uint64_t) const override
+    {
+        if (aligned(wide, out, inns)) {
+            launch(wide, stream, out, inns);
+            return;
+        }
+        {
+            std::lock_guard<std::mutex> lock(mu);
+            if (!narrow.fn) {
+                narrow.k = generate_kernel(e, 1);
+                narrow.fn = load_kernel(narrow.k);
+            }
+        }
+        launch(narrow, stream, out, inns);
+    }
+};
+
+}  // namespace
+
+std::shared_ptr<plan_t> plan_codegen(einsummable_t const& e, int)
+{
+    cg_kernel_t k;
+    try {
+        k = generate_kernel(e);
+    } catch (ir_error const&) {
+        return nullptr;
+    }
+    if (k.grid >= (1ull << 31)) return nullptr;
+    if (8 * (1 + k.n_inns) + 8 * k.params.size() > 1000) return nullptr;
+    auto p = std::make_shared<codegen_plan_t>(e);
+    p->wide.k = std::move(k);
+    p->wide.fn = load_kernel(p->wide.k);
+    switch (p->wide.k.kind) {
+        case cg_kind::elementwise:
+            p->description = "elementwise";
+            break;
+        case cg_kind::reduce_row:
+            p->description = "reduce_row";
+            break;
+        case cg_kind::reduce_col:
+            p->description = "reduce_col";
+            break;
+    }
+    p->description += " vec=" + std::to_string(p->wide.k.vec);
+    p->workspace_bytes = 0;
+    return p;
+}
+
+}  // namespace es

@@ -1,0 +1,127 @@
+// Host-side IR of the apply-node path: dtype / castable / scalarop expression trees,
+// einsummable descriptors and touch selections.  Mirrors the data model of
+// dcbdan/einsummable (src/einsummable/scalarop.h:4-521, einsummable.h:8-288, touch.h:8-46)
+// at the level the kernel manager needs: parse the reference's text forms, type-check,
+// normalise (aggregation renumbering, merge_adjacent_dims, touch simplify) and classify.
+#pragma once
+#include <cstdint>
+#include <memory>
+#include <optional>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+namespace es
+{
+
+enum class dtype_t : int { f16 = 0, f32 = 1, f64 = 2, c64 = 3 };
+enum class castable_t : int { add = 0, mul = 1, min = 2, max = 3 };
+enum class compare_t : int { lt = 0, gt = 1, eq = 2, le = 3, ge = 4 };
+
+uint64_t    dtype_size(dtype_t);
+const char* dtype_name(dtype_t);
+// '+' 'x' 'v' '^' (scalarop.cc:3078-3093); 0 means "no castable"
+std::optional<castable_t> castable_from_char(char c);
+char                      castable_to_char(std::optional<castable_t> const&);
+
+struct ir_error : std::runtime_error {
+    using std::runtime_error::runtime_error;
+};
+
+enum class op_kind {
+    constant,
+    hole,
+    variable,
+    add,
+    mul,
+    exp,
+    log,
+    power,
+    ite,
+    convert,
+    conj,
+    real,
+    imag,
+    cplex
+};
+
+// One node of a scalarop expression tree (scalar_ns::node_t, scalarop.h:227-276).
+struct node_t {
+    op_kind             kind;
+    dtype_t             dtype;     // result dtype of this node
+    double              re = 0.0;  // constant value, already rounded to `dtype`
+    double              im = 0.0;
+    int                 arg = -1;  // hole index
+    double              power = 0.0;
+    compare_t           compare = compare_t::lt;
+    std::string         name;  // variable name
+    std::vector<node_t> children;
+};
+
+struct scalarop_t {
+    node_t root;
+    // dtype of hole k; nullopt when the expression does not use hole k
+    std::vector<std::optional<dtype_t>> hole_dtypes;
+
+    // Parses the reference's operator<< text, e.g.
+    //   *[hole|f16@0,power{-1}[+[constant{f16|1},exp[*[constant{f16|-1},hole|f16@0]]]]]
+    // (grammar: scalarop.cc:2881-3011).  Throws ir_error on malformed or ill-typed text.
+    static scalarop_t parse(std::string const& text);
+
+    std::string str() const;
+    dtype_t     out_dtype() const { return root.dtype; }
+    int         num_inputs() const { return int(hole_dtypes.size()); }
+    bool        has_variables() const;
+    bool        is_identity() const;  // exactly hole@0
+    bool        is_mul() const;       // exactly *[hole@0,hole@1]
+    bool        is_add() const;       // exactly +[hole@0,hole@1]
+};
+
+// einsummable_t (einsummable.h:8-288): out modes are 0..out_rank-1, aggregated modes follow.
+struct einsummable_t {
+    std::vector<uint64_t>         join_shape;
+    std::vector<std::vector<int>> inns;
+    int                           out_rank = 0;
+    scalarop_t                    join;
+    std::optional<castable_t>     castable;
+
+    // Runs the checks and the aggregation-mode renumbering of the reference constructor
+    // (einsummable.cc:32-93).  Throws ir_error when invalid.
+    static einsummable_t make(std::vector<uint64_t> join_shape, std::vector<std::vector<int>> inns,
+                              int out_rank, scalarop_t join, std::optional<castable_t> castable);
+
+    // Fuse modes that are adjacent in every term (einsummable.cc:166-218).
+    einsummable_t merge_adjacent_dims() const;
+
+    std::string str() const;  // "ab,bc->ac"
+    // canonical lookup key: shape, modes, join text and castable
+    std::string key() const;
+
+    bool     has_aggregation() const { return out_rank < int(join_shape.size()); }
+    bool     has_broadcast() const;
+    bool     is_straight_elementwise() const;
+    bool     is_permutation() const;
+    bool     is_contraction() const;
+    dtype_t  out_dtype() const { return join.out_dtype(); }
+    dtype_t  inn_dtype(int k) const { return join.hole_dtypes[k].value(); }
+    uint64_t out_nelem() const;
+    uint64_t inn_nelem(int k) const;
+};
+
+struct touchdim_t {
+    uint64_t d_inn, d_out, offset_inn, offset_out, size;
+};
+
+struct touch_t {
+    std::vector<touchdim_t>   selection;
+    std::optional<castable_t> castable;
+    dtype_t                   dtype;
+
+    // Merge trailing dimensions that are copied in full into their predecessor
+    // (touch.cc:3-28).
+    touch_t simplify() const;
+    // throws ir_error if a window leaves its tensor or the selection is empty
+    void validate() const;
+};
+
+}  // namespace es

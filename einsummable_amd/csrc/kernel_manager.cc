@@ -1,0 +1,194 @@
+#include "kernel_manager.h"
+
+#include "launch.h"
+
+#include <hip/hip_runtime.h>
+
+namespace es
+{
+
+namespace
+{
+
+void hip_check(hipError_t err, const char* what)
+{
+    if (err != hipSuccess) {
+        throw km_error(km_status::device, std::string(what) + ": " + hipGetErrorString(err));
+    }
+}
+
+}  // namespace
+
+kernel_manager_t::kernel_manager_t(int device) : device_(device)
+{
+    int count = 0;
+    hip_check(hipGetDeviceCount(&count), "hipGetDeviceCount");
+    if (device < 0 || device >= count) {
+        throw km_error(km_status::device, "kernel_manager_t: no such device " +
+                                              std::to_string(device) + " (" +
+                                              std::to_string(count) + " visible)");
+    }
+    hip_check(hipSetDevice(device), "hipSetDevice");
+}
+
+kernel_manager_t::~kernel_manager_t() = default;
+
+plan_t const* kernel_manager_t::find(einsummable_t const& merged) const
+{
+    auto it = plans_.find(merged.key());
+    return it == plans_.end() ? nullptr : it->second.get();
+}
+
+std::optional<uint64_t> kernel_manager_t::build(einsummable_t const& e_)
+{
+    if (e_.join.has_variables()) {
+        // the caller substitutes scalar variables before building
+        // (src/engine/gpu/exec_graph.cc:106-108, kernel_executor.cc:64-66)
+        return std::nullopt;
+    }
+    einsummable_t e = e_.merge_adjacent_dims();
+    std::string   key = e.key();
+    auto          it = plans_.find(key);
+    if (it != plans_.end()) return it->second->workspace_bytes;
+
+    std::shared_ptr<plan_t> p = plan_contraction(e, device_);
+    if (!p) p = plan_transpose(e, device_);
+    if (!p) p = plan_codegen(e, device_);
+    if (!p) return std::nullopt;
+    p->n_inns = int(e.inns.size());
+    plans_.emplace(key, p);
+    return p->workspace_bytes;
+}
+
+uint64_t kernel_manager_t::workspace_size(einsummable_t const& e) const
+{
+    plan_t const* p = find(e.merge_adjacent_dims());
+    if (!p) throw km_error(km_status::not_built, "workspace_size: einsummable was not built");
+    return p->workspace_bytes;
+}
+
+std::string kernel_manager_t::describe(einsummable_t const& e) const
+{
+    plan_t const* p = find(e.merge_adjacent_dims());
+    if (!p) throw km_error(km_status::not_built, "describe: einsummable was not built");
+    return p->description;
+}
+
+plan_t const* kernel_manager_t::find_raw(std::string const& raw_key) const
+{
+    auto it = raw_plans_.find(raw_key);
+    return it == raw_plans_.end() ? nullptr : it->second.get();
+}
+
+void kernel_manager_t::alias_raw(std::string const& raw_key, einsummable_t const& e)
+{
+    auto it = plans_.find(e.merge_adjacent_dims().key());
+    if (it != plans_.end()) raw_plans_[raw_key] = it->second;
+}
+
+void kernel_manager_t::run_plan(plan_t const& p, hipStream_t stream, void* out,
+                                void const* const* inns, int n_inns, void* workspace,
+                                uint64_t workspace_bytes) const
+{
+    if (n_inns != p.n_inns) {
+        throw km_error(km_status::inputs, "execute: " + std::to_string(n_inns) +
+                                              " inputs given, einsummable has " +
+                                              std::to_string(p.n_inns));
+    }
+    if (p.workspace_bytes > 0 && (!workspace || workspace_bytes < p.workspace_bytes)) {
+        throw km_error(km_status::workspace,
+                       "execute: workspace of " + std::to_string(p.workspace_bytes) +
+                           " bytes required, " + std::to_string(workspace ? workspace_bytes : 0) +
+                           " given");
+    }
+    p.run(stream, out, inns, workspace, workspace_bytes);
+}
+
+void kernel_manager_t::operator()(einsummable_t const& e, hipStream_t stream, void* out,
+                                  std::vector<void const*> const&             inns,
+                                  std::optional<std::tuple<void*, uint64_t>> workspace) const
+{
+    plan_t const* p = find(e.merge_adjacent_dims());
+    if (!p) throw km_error(km_status::not_built, "execute: einsummable was not built");
+    void*    ws = workspace ? std::get<0>(workspace.value()) : nullptr;
+    uint64_t wsz = workspace ? std::get<1>(workspace.value()) : 0;
+    run_plan(*p, stream, out, inns.data(), int(inns.size()), ws, wsz);
+}
+
+void kernel_manager_t::operator()(touch_t const& touch_, hipStream_t stream, void* out,
+                                  void const* inn) const
+{
+    touch_.validate();
+    touch_t t = touch_.simplify();
+    int     r = int(t.selection.size());
+    if (r > 4) {
+        throw km_error(km_status::invalid, "touch: more than four dimensions after simplify");
+    }
+    int const esz = int(dtype_size(t.dtype));
+    int const vmax = 16 / esz;
+
+    touchdim_t const& last = t.selection[r - 1];
+    bool              wide = (last.size % vmax == 0) && (last.offset_inn % vmax == 0) &&
+                (last.offset_out % vmax == 0) &&
+                (reinterpret_cast<uintptr_t>(out) % 16 == 0) &&
+                (reinterpret_cast<uintptr_t>(inn) % 16 == 0);
+    if (r > 1) wide = wide && (last.d_inn % vmax == 0) && (last.d_out % vmax == 0);
+
+    touch_launch_t a;
+    a.vec = wide ? vmax : 1;
+    a.vec_per_row = last.size / uint64_t(a.vec);
+    a.base_inn = 0;
+    a.base_out = 0;
+    // element strides of every dimension
+    uint64_t si = 1, so = 1;
+    uint64_t str_i[4], str_o[4];
+    for (int d = r - 1; d >= 0; --d) {
+        str_i[d] = si;
+        str_o[d] = so;
+        a.base_inn += t.selection[d].offset_inn * si;
+        a.base_out += t.selection[d].offset_out * so;
+        si *= t.selection[d].d_inn;
+        so *= t.selection[d].d_out;
+    }
+    // outer dimensions right-aligned into the three slots
+    a.n_vec = a.vec_per_row;
+    bool small = a.vec_per_row < (1ull << 32);
+    for (int s = 0; s != 3; ++s) {
+        int d = (r - 1) - 3 + s;  // dimension feeding slot s
+        if (d >= 0) {
+            a.size[s] = t.selection[d].size;
+            a.str_inn[s] = str_i[d];
+            a.str_out[s] = str_o[d];
+        } else {
+            a.size[s] = 1;
+            a.str_inn[s] = 0;
+            a.str_out[s] = 0;
+        }
+        a.n_vec *= a.size[s];
+        small = small && a.size[s] < (1ull << 32);
+    }
+    a.small = small && a.n_vec < (1ull << 32);
+
+    int op = 0;
+    if (t.castable) op = 1 + int(t.castable.value());
+    launch_touch(a, esz, int(t.dtype), op, stream, out, inn);
+    hip_check(hipGetLastError(), "touch launch");
+}
+
+void kernel_manager_t::constant_fill(dtype_t dtype, uint64_t value_bits, uint64_t nelem,
+                                     hipStream_t stream, void* out) const
+{
+    launch_fill_constant(int(dtype_size(dtype)), value_bits, nelem, stream, out);
+    hip_check(hipGetLastError(), "constant_fill launch");
+}
+
+void kernel_manager_t::lowerTri_fill(dtype_t dtype, uint64_t lower_bits, uint64_t upper_bits,
+                                     uint64_t nrow, uint64_t ncol, int64_t start,
+                                     hipStream_t stream, void* out) const
+{
+    launch_fill_lowertri(int(dtype_size(dtype)), lower_bits, upper_bits, nrow, ncol, start, stream,
+                         out);
+    hip_check(hipGetLastError(), "lowerTri_fill launch");
+}
+
+}  // namespace es

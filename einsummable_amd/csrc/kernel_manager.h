@@ -1,0 +1,90 @@
+// The kernel manager: plans one kernel per (merged) einsummable at build() and launches it on
+// raw device buffers at operator().  Same surface and error behaviour as the reference's
+// kernel_manager_t (src/engine/gpu/gpu_kernel_manager.h:274-321): build returns nullopt for
+// an unsupported einsummable and never throws for that reason; calling an un-built
+// einsummable, passing the wrong number of inputs or an undersized workspace throws
+// (gpu_kernel_manager.cc:1103-1107, 1126, 1260, 1586, 1968).
+#pragma once
+#include "ir.h"
+
+#include <hip/hip_runtime_api.h>
+
+#include <memory>
+#include <optional>
+#include <string>
+#include <tuple>
+#include <unordered_map>
+#include <vector>
+
+namespace es
+{
+
+enum class km_status : int {
+    invalid = -1,
+    not_built = -2,
+    workspace = -3,
+    inputs = -4,
+    device = -5
+};
+
+struct km_error : std::runtime_error {
+    km_error(km_status s, std::string const& what) : std::runtime_error(what), status(s) {}
+    km_status status;
+};
+
+// One planned kernel.  run() only enqueues work on `stream`.
+struct plan_t {
+    virtual ~plan_t() = default;
+    virtual void run(hipStream_t stream, void* out, void const* const* inns, void* workspace,
+                     uint64_t workspace_bytes) const = 0;
+    uint64_t    workspace_bytes = 0;
+    int         n_inns = 0;
+    std::string description;
+};
+
+class kernel_manager_t
+{
+public:
+    explicit kernel_manager_t(int device);
+    ~kernel_manager_t();
+
+    std::optional<uint64_t> build(einsummable_t const& e);
+    uint64_t                workspace_size(einsummable_t const& e) const;
+    std::string             describe(einsummable_t const& e) const;
+
+    void operator()(einsummable_t const& e, hipStream_t stream, void* out,
+                    std::vector<void const*> const&             inns,
+                    std::optional<std::tuple<void*, uint64_t>> workspace = std::nullopt) const;
+
+    void operator()(touch_t const& touch, hipStream_t stream, void* out, void const* inn) const;
+
+    void constant_fill(dtype_t dtype, uint64_t value_bits, uint64_t nelem, hipStream_t stream,
+                       void* out) const;
+    void lowerTri_fill(dtype_t dtype, uint64_t lower_bits, uint64_t upper_bits, uint64_t nrow,
+                       uint64_t ncol, int64_t start, hipStream_t stream, void* out) const;
+
+    // Lookup by a caller-made key (the C ABI keys on the raw descriptor text so that the hot
+    // path does not re-parse the scalarop).
+    plan_t const* find_raw(std::string const& raw_key) const;
+    void          alias_raw(std::string const& raw_key, einsummable_t const& e);
+    void          run_plan(plan_t const& p, hipStream_t stream, void* out,
+                           void const* const* inns, int n_inns, void* workspace,
+                           uint64_t workspace_bytes) const;
+
+    int device() const { return device_; }
+
+private:
+    plan_t const* find(einsummable_t const& merged) const;
+
+    int                                                      device_;
+    std::unordered_map<std::string, std::shared_ptr<plan_t>> plans_;      // by merged key
+    std::unordered_map<std::string, std::shared_ptr<plan_t>> raw_plans_;  // by caller key
+};
+
+// Planners (one translation unit each).  Each returns nullptr when the einsummable is not
+// of its kind; `e` has already been through merge_adjacent_dims.
+std::shared_ptr<plan_t> plan_contraction(einsummable_t const& e, int device);
+std::shared_ptr<plan_t> plan_transpose(einsummable_t const& e, int device);
+std::shared_ptr<plan_t> plan_codegen(einsummable_t const& e, int device);
+
+}  // namespace es

@@ -1,0 +1,327 @@
+// touch_t kernels for gfx950: N-D copy-region / accumulate (rank <= 4 after simplify) and the
+// constant / lower-triangular fills.  These replace touch1..touch4, fill_constant and
+// fill_lowerTri of the reference (src/engine/gpu/cuda_kernels.cu:99-515, 579-647) and follow
+// the value semantics of the CPU kernels (src/engine/touch.cc:119-135): `+=`, `*=`,
+// std::min, std::max in the tensor's own dtype, so results are bit-identical to the CPU path.
+//
+// Layout: one thread moves one 16-byte vector (or one element when the windows are not
+// 16-byte aligned) of the innermost dimension; consecutive lanes take consecutive vectors of
+// a row, so every wavefront reads and writes whole 1 KiB row segments.  Each thread handles
+// UNROLL vectors 256 lanes apart, all loads issued before the first store.
+#include "launch.h"
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstring>
+
+namespace es
+{
+namespace
+{
+
+constexpr int TOUCH_BLOCK = 256;
+constexpr int TOUCH_UNROLL = 4;
+
+struct c64_t {
+    float re, im;
+};
+
+template <typename T, int N>
+struct alignas(sizeof(T) * N) vec_t {
+    T v[N];
+};
+
+enum : int { OP_COPY = 0, OP_ADD = 1, OP_MUL = 2, OP_MIN = 3, OP_MAX = 4 };
+
+template <int OP, typename T>
+__device__ __forceinline__ T touch_op(T out, T inn)
+{
+#pragma clang fp contract(off)
+    if constexpr (OP == OP_COPY) {
+        return inn;
+    } else if constexpr (OP == OP_ADD) {
+        return out + inn;
+    } else if constexpr (OP == OP_MUL) {
+        return out * inn;
+    } else if constexpr (OP == OP_MIN) {
+        return (inn < out) ? inn : out;  // std::min(out, inn)
+    } else {
+        return (out < inn) ? inn : out;  // std::max(out, inn)
+    }
+}
+
+template <int OP>
+__device__ __forceinline__ c64_t touch_op_c64(c64_t out, c64_t inn)
+{
+#pragma clang fp contract(off)
+    if constexpr (OP == OP_ADD) {
+        return c64_t{out.re + inn.re, out.im + inn.im};
+    } else if constexpr (OP == OP_MUL) {
+        float ac = out.re * inn.re, bd = out.im * inn.im;
+        float ad = out.re * inn.im, bc = out.im * inn.re;
+        return c64_t{ac - bd, ad + bc};
+    } else {
+        return inn;
+    }
+}
+
+template <int OP, typename T>
+__device__ __forceinline__ T apply(T out, T inn)
+{
+    if constexpr (sizeof(T) == 8 && alignof(T) == 4) {
+        return touch_op_c64<OP>(out, inn);
+    } else {
+        return touch_op<OP>(out, inn);
+    }
+}
+
+// T: element type, V: elements per thread-vector
+template <typename T, int V, int OP>
+__global__ __launch_bounds__(TOUCH_BLOCK) void touch_kernel(touch_launch_t a, T* __restrict__ out,
+                                                            T const* __restrict__ inn)
+{
+    using vt = vec_t<T, V>;
+    uint64_t const first = (uint64_t(blockIdx.x) * TOUCH_UNROLL) * TOUCH_BLOCK + threadIdx.x;
+    vt             x[TOUCH_UNROLL];
+    vt             y[TOUCH_UNROLL];
+    uint64_t       oo[TOUCH_UNROLL];
+    bool           live[TOUCH_UNROLL];
+#pragma unroll
+    for (int u = 0; u != TOUCH_UNROLL; ++u) {
+        uint64_t idx = first + uint64_t(u) * TOUCH_BLOCK;
+        live[u] = idx < a.n_vec;
+        if (live[u]) {
+            uint64_t oi, ii;
+            if (a.small) {
+                uint32_t r = uint32_t(idx);
+                uint32_t c = r % uint32_t(a.vec_per_row);
+                r /= uint32_t(a.vec_per_row);
+                uint32_t i2 = r % uint32_t(a.size[2]);
+                r /= uint32_t(a.size[2]);
+                uint32_t i1 = r % uint32_t(a.size[1]);
+                uint32_t i0 = r / uint32_t(a.size[1]);
+                ii = a.base_inn + i0 * a.str_inn[0] + i1 * a.str_inn[1] + i2 * a.str_inn[2] +
+                     uint64_t(c) * V;
+                oi = a.base_out + i0 * a.str_out[0] + i1 * a.str_out[1] + i2 * a.str_out[2] +
+                     uint64_t(c) * V;
+            } else {
+                uint64_t r = idx;
+                uint64_t c = r % a.vec_per_row;
+                r /= a.vec_per_row;
+                uint64_t i2 = r % a.size[2];
+                r /= a.size[2];
+                uint64_t i1 = r % a.size[1];
+                uint64_t i0 = r / a.size[1];
+                ii = a.base_inn + i0 * a.str_inn[0] + i1 * a.str_inn[1] + i2 * a.str_inn[2] +
+                     c * V;
+                oi = a.base_out + i0 * a.str_out[0] + i1 * a.str_out[1] + i2 * a.str_out[2] +
+                     c * V;
+            }
+            oo[u] = oi;
+            x[u] = *reinterpret_cast<vt const*>(inn + ii);
+            if constexpr (OP != OP_COPY) {
+                y[u] = *reinterpret_cast<vt const*>(out + oi);
+            }
+        }
+    }
+#pragma unroll
+    for (int u = 0; u != TOUCH_UNROLL; ++u) {
+        if (live[u]) {
+            vt r;
+            if constexpr (OP == OP_COPY) {
+                r = x[u];
+            } else {
+#pragma unroll
+                for (int j = 0; j != V; ++j) r.v[j] = apply<OP, T>(y[u].v[j], x[u].v[j]);
+            }
+            *reinterpret_cast<vt*>(out + oo[u]) = r;
+        }
+    }
+}
+
+template <typename T, int V, int OP>
+void launch_touch_v(touch_launch_t const& a, hipStream_t stream, void* out, void const* inn)
+{
+    uint64_t per_block = uint64_t(TOUCH_BLOCK) * TOUCH_UNROLL;
+    uint64_t blocks = (a.n_vec + per_block - 1) / per_block;
+    hipLaunchKernelGGL((touch_kernel<T, V, OP>), dim3((unsigned)blocks), dim3(TOUCH_BLOCK), 0,
+                       stream, a, static_cast<T*>(out), static_cast<T const*>(inn));
+}
+
+template <typename T, int OP>
+void launch_touch_t(touch_launch_t const& a, hipStream_t stream, void* out, void const* inn)
+{
+    constexpr int VMAX = 16 / sizeof(T);
+    if (a.vec == VMAX) {
+        launch_touch_v<T, VMAX, OP>(a, stream, out, inn);
+    } else {
+        launch_touch_v<T, 1, OP>(a, stream, out, inn);
+    }
+}
+
+template <typename T>
+void launch_touch_op(touch_launch_t const& a, int op, hipStream_t stream, void* out,
+                     void const* inn)
+{
+    switch (op) {
+        case OP_ADD:
+            return launch_touch_t<T, OP_ADD>(a, stream, out, inn);
+        case OP_MUL:
+            return launch_touch_t<T, OP_MUL>(a, stream, out, inn);
+        case OP_MIN:
+            return launch_touch_t<T, OP_MIN>(a, stream, out, inn);
+        case OP_MAX:
+            return launch_touch_t<T, OP_MAX>(a, stream, out, inn);
+    }
+}
+
+// ---- fills
+
+template <int V>
+__global__ __launch_bounds__(256) void fill_constant_kernel(uint64_t n_vec, vec_t<uint32_t, V> pat,
+                                                            vec_t<uint32_t, V>* __restrict__ out)
+{
+    uint64_t i = uint64_t(blockIdx.x) * 256 + threadIdx.x;
+    uint64_t stride = uint64_t(gridDim.x) * 256;
+    for (; i < n_vec; i += stride) out[i] = pat;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void fill_tail_kernel(uint64_t begin, uint64_t end, T value,
+                                                        T* __restrict__ out)
+{
+    uint64_t i = begin + uint64_t(blockIdx.x) * 256 + threadIdx.x;
+    if (i < end) out[i] = value;
+}
+
+// out[r, c] = (r - start >= c) ? lower : upper, signed r - start
+// (src/einsummable/fill.h:17-19); one thread writes V consecutive columns.
+template <typename T, int V>
+__global__ __launch_bounds__(256) void fill_lowertri_kernel(uint64_t nrow, uint64_t ncol,
+                                                            int64_t start, T lower, T upper,
+                                                            T* __restrict__ out)
+{
+    uint64_t vec_per_row = ncol / V;
+    uint64_t n_vec = nrow * vec_per_row;
+    uint64_t i = uint64_t(blockIdx.x) * 256 + threadIdx.x;
+    uint64_t stride = uint64_t(gridDim.x) * 256;
+    for (; i < n_vec; i += stride) {
+        uint64_t  r = i / vec_per_row;
+        uint64_t  c0 = (i % vec_per_row) * V;
+        int64_t   edge = int64_t(r) - start;  // columns <= edge take `lower`
+        vec_t<T, V> v;
+#pragma unroll
+        for (int j = 0; j != V; ++j) v.v[j] = (edge >= int64_t(c0 + j)) ? lower : upper;
+        *reinterpret_cast<vec_t<T, V>*>(out + r * ncol + c0) = v;
+    }
+}
+
+template <typename T>
+void launch_lowertri(uint64_t nrow, uint64_t ncol, int64_t start, uint64_t lower_bits,
+                     uint64_t upper_bits, hipStream_t stream, void* out)
+{
+    T lower, upper;
+    std::memcpy(&lower, &lower_bits, sizeof(T));
+    std::memcpy(&upper, &upper_bits, sizeof(T));
+    constexpr int VMAX = 16 / sizeof(T);
+    bool          wide = (ncol % VMAX == 0) && (reinterpret_cast<uintptr_t>(out) % 16 == 0);
+    uint64_t      n_vec = wide ? nrow * (ncol / VMAX) : nrow * ncol;
+    unsigned      blocks = (unsigned)std::min<uint64_t>((n_vec + 255) / 256, 65536);
+    if (blocks == 0) return;
+    if (wide) {
+        hipLaunchKernelGGL((fill_lowertri_kernel<T, VMAX>), dim3(blocks), dim3(256), 0, stream,
+                           nrow, ncol, start, lower, upper, static_cast<T*>(out));
+    } else {
+        hipLaunchKernelGGL((fill_lowertri_kernel<T, 1>), dim3(blocks), dim3(256), 0, stream, nrow,
+                           ncol, start, lower, upper, static_cast<T*>(out));
+    }
+}
+
+}  // namespace
+
+void launch_touch(touch_launch_t const& a, int elem_size, int dtype_code, int op,
+                  hipStream_t stream, void* out, void const* inn)
+{
+    if (a.n_vec == 0) return;
+    if (op == OP_COPY) {
+        // copies only depend on the element width
+        switch (elem_size) {
+            case 2:
+                return launch_touch_t<uint16_t, OP_COPY>(a, stream, out, inn);
+            case 4:
+                return launch_touch_t<uint32_t, OP_COPY>(a, stream, out, inn);
+            default:
+                return launch_touch_t<uint64_t, OP_COPY>(a, stream, out, inn);
+        }
+    }
+    switch (dtype_code) {
+        case 0:
+            return launch_touch_op<_Float16>(a, op, stream, out, inn);
+        case 1:
+            return launch_touch_op<float>(a, op, stream, out, inn);
+        case 2:
+            return launch_touch_op<double>(a, op, stream, out, inn);
+        default:
+            if (op == OP_ADD) return launch_touch_t<c64_t, OP_ADD>(a, stream, out, inn);
+            return launch_touch_t<c64_t, OP_MUL>(a, stream, out, inn);
+    }
+}
+
+void launch_fill_constant(int elem_size, uint64_t bits, uint64_t nelem, hipStream_t stream,
+                          void* out)
+{
+    if (nelem == 0) return;
+    // replicate the element into a 16-byte pattern
+    vec_t<uint32_t, 4> pat;
+    unsigned char      raw[16];
+    for (int i = 0; i < 16; i += elem_size) std::memcpy(raw + i, &bits, size_t(elem_size));
+    std::memcpy(&pat, raw, 16);
+    uint64_t  bytes = nelem * uint64_t(elem_size);
+    uintptr_t p = reinterpret_cast<uintptr_t>(out);
+    uint64_t  head_bytes = (16 - (p % 16)) % 16;  // multiple of elem_size: out is element aligned
+    if (head_bytes > bytes) head_bytes = bytes;
+    uint64_t body_vec = (bytes - head_bytes) / 16;
+    uint64_t tail_begin = (head_bytes + body_vec * 16) / uint64_t(elem_size);
+    auto     edge = [&](uint64_t b, uint64_t e) {
+        if (b == e) return;
+        unsigned blocks = unsigned((e - b + 255) / 256);
+        if (elem_size == 2) {
+            hipLaunchKernelGGL((fill_tail_kernel<uint16_t>), dim3(blocks), dim3(256), 0, stream, b,
+                               e, uint16_t(bits), static_cast<uint16_t*>(out));
+        } else if (elem_size == 4) {
+            hipLaunchKernelGGL((fill_tail_kernel<uint32_t>), dim3(blocks), dim3(256), 0, stream, b,
+                               e, uint32_t(bits), static_cast<uint32_t*>(out));
+        } else {
+            hipLaunchKernelGGL((fill_tail_kernel<uint64_t>), dim3(blocks), dim3(256), 0, stream, b,
+                               e, bits, static_cast<uint64_t*>(out));
+        }
+    };
+    edge(0, head_bytes / uint64_t(elem_size));
+    if (body_vec) {
+        unsigned blocks = (unsigned)std::min<uint64_t>((body_vec + 255) / 256, 16384);
+        hipLaunchKernelGGL((fill_constant_kernel<4>), dim3(blocks), dim3(256), 0, stream, body_vec,
+                           pat,
+                           reinterpret_cast<vec_t<uint32_t, 4>*>(static_cast<char*>(out) +
+                                                                  head_bytes));
+    }
+    edge(tail_begin, nelem);
+}
+
+void launch_fill_lowertri(int elem_size, uint64_t lower_bits, uint64_t upper_bits, uint64_t nrow,
+                          uint64_t ncol, int64_t start, hipStream_t stream, void* out)
+{
+    switch (elem_size) {
+        case 2:
+            return launch_lowertri<uint16_t>(nrow, ncol, start, lower_bits, upper_bits, stream,
+                                             out);
+        case 4:
+            return launch_lowertri<uint32_t>(nrow, ncol, start, lower_bits, upper_bits, stream,
+                                             out);
+        default:
+            return launch_lowertri<uint64_t>(nrow, ncol, start, lower_bits, upper_bits, stream,
+                                             out);
+    }
+}
+
+}  // namespace es

@@ -1,0 +1,5 @@
+#include "kernel_manager.h"
+namespace es
+{
+std::shared_ptr<plan_t> plan_transpose(einsummable_t const&, int) { return nullptr; }
+}  // namespace es

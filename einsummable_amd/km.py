@@ -1,0 +1,269 @@
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+
+F16, F32, F64, C64 = 0, 1, 2, 3
+DTYPE_SIZE = {F16: 2, F32: 4, F64: 8, C64: 8}
+
+OK, UNSUPPORTED = 0, 1
+ERR_INVALID, ERR_NOT_BUILT, ERR_WORKSPACE, ERR_INPUTS, ERR_DEVICE = -1, -2, -3, -4, -5
+
+EXPORTS = [
+    "es_km_create",
+    "es_km_destroy",
+    "es_km_last_error",
+    "es_km_build",
+    "es_km_workspace_size",
+    "es_km_execute",
+    "es_km_describe",
+    "es_km_touch",
+    "es_km_fill_constant",
+    "es_km_fill_lowertri",
+    "es_km_codegen_source",
+]
+
+
+class KmError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__("es_km error %d: %s" % (code, message))
+        self.code = code
+
+
+def lib_path():
+    return os.path.join(_HERE, "libes_km.so")
+
+
+_lib = None
+
+
+def load_library():
+    """Load libes_km.so.  There is no fallback: a missing library is an error."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = lib_path()
+    if not os.path.exists(path):
+        raise ImportError(
+            "%s is missing: build it with `python -m einsummable_amd.build`" % path
+        )
+    lib = ctypes.CDLL(path)
+    lib.es_km_create.restype = ctypes.c_void_p
+    lib.es_km_create.argtypes = [ctypes.c_int]
+    lib.es_km_destroy.argtypes = [ctypes.c_void_p]
+    lib.es_km_last_error.restype = ctypes.c_char_p
+    lib.es_km_last_error.argtypes = [ctypes.c_void_p]
+    desc = [
+        ctypes.c_void_p,  # join_shape
+        ctypes.c_int,
+        ctypes.c_void_p,  # inns_flat
+        ctypes.c_void_p,  # inns_offsets
+        ctypes.c_int,
+        ctypes.c_int,
+        ctypes.c_char_p,
+        ctypes.c_char,
+    ]
+    lib.es_km_build.argtypes = [ctypes.c_void_p] + desc + [ctypes.c_void_p]
+    lib.es_km_workspace_size.argtypes = [ctypes.c_void_p] + desc + [ctypes.c_void_p]
+    lib.es_km_execute.argtypes = [ctypes.c_void_p] + desc + [
+        ctypes.c_void_p,
+        ctypes.c_void_p,
+        ctypes.c_void_p,
+        ctypes.c_int,
+        ctypes.c_void_p,
+        ctypes.c_uint64,
+    ]
+    lib.es_km_describe.argtypes = [ctypes.c_void_p] + desc + [ctypes.c_void_p, ctypes.c_size_t]
+    lib.es_km_touch.argtypes = [
+        ctypes.c_void_p,
+        ctypes.c_void_p,
+        ctypes.c_int,
+        ctypes.c_char,
+        ctypes.c_int,
+        ctypes.c_void_p,
+        ctypes.c_void_p,
+        ctypes.c_void_p,
+    ]
+    lib.es_km_fill_constant.argtypes = [
+        ctypes.c_void_p,
+        ctypes.c_int,
+        ctypes.c_uint64,
+        ctypes.c_uint64,
+        ctypes.c_void_p,
+        ctypes.c_void_p,
+    ]
+    lib.es_km_fill_lowertri.argtypes = [
+        ctypes.c_void_p,
+        ctypes.c_int,
+        ctypes.c_uint64,
+        ctypes.c_uint64,
+        ctypes.c_uint64,
+        ctypes.c_uint64,
+        ctypes.c_int64,
+        ctypes.c_void_p,
+        ctypes.c_void_p,
+    ]
+    lib.es_km_codegen_source.argtypes = desc + [ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t]
+    _lib = lib
+    return lib
+
+
+def _castable_char(c):
+    return (c.encode() if c else b"\0")
+
+
+class Einsummable:
+    """The fields of einsummable_t (src/einsummable/einsummable.h:8-20); `join` is the
+    scalarop text, `castable` one of '+', 'x', 'v', '^' or None."""
+
+    def __init__(self, join_shape, inns, out_rank, join, castable=None):
+        self.join_shape = [int(x) for x in join_shape]
+        self.inns = [list(map(int, inn)) for inn in inns]
+        self.out_rank = int(out_rank)
+        self.join = join
+        self.castable = castable
+        flat, offs = [], [0]
+        for inn in self.inns:
+            flat.extend(inn)
+            offs.append(len(flat))
+        self._shape = (ctypes.c_uint64 * len(self.join_shape))(*self.join_shape)
+        self._flat = (ctypes.c_int * max(len(flat), 1))(*flat)
+        self._offs = (ctypes.c_int * len(offs))(*offs)
+        self._join = join.encode()
+        self._args = (
+            ctypes.cast(self._shape, ctypes.c_void_p),
+            len(self.join_shape),
+            ctypes.cast(self._flat, ctypes.c_void_p),
+            ctypes.cast(self._offs, ctypes.c_void_p),
+            len(self.inns),
+            self.out_rank,
+            self._join,
+            _castable_char(castable),
+        )
+
+    @staticmethod
+    def from_str(s, sizes, join, castable=None):
+        """'ij,jk->ik' with sizes {'i': .., 'j': .., 'k': ..} (parse_str,
+        src/einsummable/einsummable.cc:364-441)."""
+        lhs, out = s.split("->")
+        ids = {}
+        for ch in out:
+            ids[ch] = len(ids)
+        inns = []
+        for word in lhs.split(","):
+            inn = []
+            for ch in word:
+                if ch not in ids:
+                    ids[ch] = len(ids)
+                inn.append(ids[ch])
+            inns.append(inn)
+        shape = [0] * len(ids)
+        for ch, i in ids.items():
+            shape[i] = sizes[ch]
+        return Einsummable(shape, inns, len(out), join, castable)
+
+    def out_nelem(self):
+        n = 1
+        for d in self.join_shape[: self.out_rank]:
+            n *= d
+        return n
+
+    def inn_shape(self, k):
+        return [self.join_shape[m] for m in self.inns[k]]
+
+
+class Touch:
+    """touch_t (src/einsummable/touch.h:25-29): selection of
+    (d_inn, d_out, offset_inn, offset_out, size), optional castable, dtype."""
+
+    def __init__(self, selection, castable, dtype):
+        self.selection = [tuple(int(v) for v in d) for d in selection]
+        self.castable = castable
+        self.dtype = dtype
+        flat = [v for d in self.selection for v in d]
+        self._dims = (ctypes.c_uint64 * len(flat))(*flat)
+
+
+def codegen_source(e, compile=False):
+    lib = load_library()
+    buf = ctypes.create_string_buffer(1 << 16)
+    rc = lib.es_km_codegen_source(*e._args, int(compile), ctypes.cast(buf, ctypes.c_void_p),
+                                  1 << 16)
+    if rc != OK:
+        raise KmError(rc, lib.es_km_last_error(None).decode())
+    return buf.value.decode()
+
+
+class KernelManager:
+    """kernel_manager_t(device): build / workspace_size / __call__ / touch / fills on raw
+    device addresses (ints) and a raw hipStream_t (int, 0 = default stream)."""
+
+    def __init__(self, device=0):
+        self._lib = load_library()
+        self._h = self._lib.es_km_create(int(device))
+        if not self._h:
+            raise KmError(ERR_DEVICE, self._lib.es_km_last_error(None).decode())
+
+    def close(self):
+        if self._h:
+            self._lib.es_km_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def _fail(self, rc):
+        raise KmError(rc, self._lib.es_km_last_error(self._h).decode())
+
+    def build(self, e):
+        """Workspace bytes, or None when unsupported (the reference returns nullopt)."""
+        ws = ctypes.c_uint64(0)
+        rc = self._lib.es_km_build(self._h, *e._args, ctypes.byref(ws))
+        if rc == UNSUPPORTED:
+            return None
+        if rc != OK:
+            self._fail(rc)
+        return ws.value
+
+    def workspace_size(self, e):
+        ws = ctypes.c_uint64(0)
+        rc = self._lib.es_km_workspace_size(self._h, *e._args, ctypes.byref(ws))
+        if rc != OK:
+            self._fail(rc)
+        return ws.value
+
+    def describe(self, e):
+        buf = ctypes.create_string_buffer(256)
+        rc = self._lib.es_km_describe(self._h, *e._args, ctypes.cast(buf, ctypes.c_void_p), 256)
+        if rc != OK:
+            self._fail(rc)
+        return buf.value.decode()
+
+    def __call__(self, e, stream, out, inns, workspace=None):
+        ptrs = (ctypes.c_void_p * max(len(inns), 1))(*inns)
+        ws_ptr, ws_size = workspace if workspace else (None, 0)
+        rc = self._lib.es_km_execute(self._h, *e._args, stream, out, ptrs, len(inns), ws_ptr,
+                                     ws_size)
+        if rc != OK:
+            self._fail(rc)
+
+    def touch(self, t, stream, out, inn):
+        rc = self._lib.es_km_touch(self._h, ctypes.cast(t._dims, ctypes.c_void_p),
+                                   len(t.selection), _castable_char(t.castable), t.dtype, stream,
+                                   out, inn)
+        if rc != OK:
+            self._fail(rc)
+
+    def constant_fill(self, dtype, value_bits, nelem, stream, out):
+        rc = self._lib.es_km_fill_constant(self._h, dtype, value_bits, nelem, stream, out)
+        if rc != OK:
+            self._fail(rc)
+
+    def lowerTri_fill(self, dtype, lower_bits, upper_bits, nrow, ncol, start, stream, out):
+        rc = self._lib.es_km_fill_lowertri(self._h, dtype, lower_bits, upper_bits, nrow, ncol,
+                                           start, stream, out)
+        if rc != OK:
+            self._fail(rc)

@@ -1,0 +1,120 @@
+/*
+ * es_km.h -- C ABI of the MI355X (gfx950) kernel manager for einsummable apply nodes.
+ *
+ * This is the drop-in boundary for the GPU apply path of dcbdan/einsummable: every entry
+ * point replaces one member of the reference's `kernel_manager_t`
+ * (src/engine/gpu/gpu_kernel_manager.h:274-321).  The reference has no FFI layer; its exec
+ * nodes call the C++ class directly (src/engine/gpu/exec_graph.cc:135, 316, 384, 623, 675).
+ * A maintainer binds this library by giving `kernel_manager_t` the members shown in
+ * `es_km.hpp` (a header-only C++ class over this ABI with the reference's member names).
+ *
+ * Conventions
+ *  - Descriptors travel in the reference's own text forms: a scalarop is the text written by
+ *    `operator<<(ostream&, scalarop_t)` (src/einsummable/scalarop.cc:2881-3011), e.g.
+ *    "*[hole|f16@0,hole|f16@1]"; a castable is one of '+' 'x' 'v' '^'
+ *    (scalarop.cc:3078-3093) or 0 for none; dtypes are the enum values below
+ *    (scalarop.h:10).
+ *  - An einsummable is (join_shape[join_rank], inns, out_rank, join text, castable) exactly
+ *    as the fields of `einsummable_t` (src/einsummable/einsummable.h:8-20).  `inns` is
+ *    flattened: input k holds modes inns_flat[inns_offsets[k] .. inns_offsets[k+1]).
+ *  - All device pointers are owned by the caller (sub-ranges of its arena); the library
+ *    never allocates or frees tensor memory.  Every launch is asynchronous on the given
+ *    stream (`hipStream_t` passed as void*); nothing synchronises.
+ *  - Return codes: 0 success, ES_KM_UNSUPPORTED (1) where the reference returns nullopt,
+ *    negative where the reference throws std::runtime_error.  The message of the last
+ *    failure on a handle is available from es_km_last_error.
+ */
+#ifndef ES_KM_H
+#define ES_KM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { ES_KM_F16 = 0, ES_KM_F32 = 1, ES_KM_F64 = 2, ES_KM_C64 = 3 };
+
+enum {
+    ES_KM_OK = 0,
+    ES_KM_UNSUPPORTED = 1,       /* build: no kernel for this einsummable (reference: nullopt)  */
+    ES_KM_ERR_INVALID = -1,      /* malformed descriptor (reference: constructor throws)        */
+    ES_KM_ERR_NOT_BUILT = -2,    /* execute / workspace_size before build                       */
+    ES_KM_ERR_WORKSPACE = -3,    /* workspace missing or smaller than build() reported          */
+    ES_KM_ERR_INPUTS = -4,       /* wrong number of input pointers                              */
+    ES_KM_ERR_DEVICE = -5        /* HIP runtime or runtime-compiler failure                     */
+};
+
+typedef struct es_km es_km_t;
+
+/* kernel_manager_t(int device)                          gpu_kernel_manager.h:275
+ * Returns NULL when the device cannot be selected (see es_km_last_error(NULL)). */
+es_km_t* es_km_create(int device);
+void     es_km_destroy(es_km_t* km);
+
+/* Message of the most recent failure on this handle (on this thread for km == NULL). */
+const char* es_km_last_error(es_km_t* km);
+
+/* optional<workspace_info_t> build(einsummable_t const&)        gpu_kernel_manager.h:302
+ * Plans (and, for elementwise / reduction forms, runtime-compiles) the kernel for one
+ * einsummable and memoises it under the einsummable's value, after merge_adjacent_dims
+ * (gpu_kernel_manager.cc:590-600).  *workspace_bytes receives the scratch size execute needs. */
+int es_km_build(es_km_t* km, const uint64_t* join_shape, int join_rank, const int* inns_flat,
+                const int* inns_offsets, int n_inns, int out_rank, const char* join_text,
+                char castable, uint64_t* workspace_bytes);
+
+/* workspace_info_t workspace_size(einsummable_t const&) const   gpu_kernel_manager.h:304 */
+int es_km_workspace_size(es_km_t* km, const uint64_t* join_shape, int join_rank,
+                         const int* inns_flat, const int* inns_offsets, int n_inns, int out_rank,
+                         const char* join_text, char castable, uint64_t* workspace_bytes);
+
+/* void operator()(einsummable_t const&, cudaStream_t, void* out, vector<void const*> inns,
+ *                 optional<tuple<void*, uint64_t>> workspace) const
+ *                                                               gpu_kernel_manager.h:308-312
+ * workspace may be NULL when build reported 0 bytes. */
+int es_km_execute(es_km_t* km, const uint64_t* join_shape, int join_rank, const int* inns_flat,
+                  const int* inns_offsets, int n_inns, int out_rank, const char* join_text,
+                  char castable, void* stream, void* out, const void* const* inns,
+                  int n_inn_ptrs, void* workspace, uint64_t workspace_bytes);
+
+/* Name of the kernel family chosen by build for this einsummable, e.g. "elementwise",
+ * "reduce_row", "contraction_mfma_f16" (diagnostics; no counterpart in the reference apart
+ * from its force_debug printouts, gpu_kernel_manager.cc:1008-1034). */
+int es_km_describe(es_km_t* km, const uint64_t* join_shape, int join_rank, const int* inns_flat,
+                   const int* inns_offsets, int n_inns, int out_rank, const char* join_text,
+                   char castable, char* out, size_t cap);
+
+/* void operator()(touch_t const&, cudaStream_t, void* out, void const* inn) const
+ *                                                               gpu_kernel_manager.h:306
+ * touchdims = rank x {d_inn, d_out, offset_inn, offset_out, size} (touch.h:8-13).
+ * simplify() is applied inside, as build_touch does (src/engine/gpu/kernels.cc:150-152);
+ * more than four dimensions after simplify is an error. */
+int es_km_touch(es_km_t* km, const uint64_t* touchdims, int rank, char castable, int dtype,
+                void* stream, void* out, const void* inn);
+
+/* void constant_fill(fill_t::constant_t const&, cudaStream_t, void* out) const
+ *                                                               gpu_kernel_manager.h:321
+ * value_bits: the scalar's bytes, little-endian, in the low bytes of a uint64
+ * (scalar_t::data, scalarop.h:70-71); nelem = product of the fill's shape. */
+int es_km_fill_constant(es_km_t* km, int dtype, uint64_t value_bits, uint64_t nelem, void* stream,
+                        void* out);
+
+/* void lowerTri_fill(fill_t::lowertri_t const&, cudaStream_t, void* out) const
+ *                                                               gpu_kernel_manager.h:320
+ * out[i, j] = (i - start >= j) ? lower : upper with signed i - start (fill.h:14-24). */
+int es_km_fill_lowertri(es_km_t* km, int dtype, uint64_t lower_bits, uint64_t upper_bits,
+                        uint64_t nrow, uint64_t ncol, int64_t start, void* stream, void* out);
+
+/* Diagnostics without a device: generate (and, with compile != 0, runtime-compile for
+ * gfx950) the kernel source the scalarop code generator emits for an elementwise or
+ * elementwise-then-reduce einsummable.  No counterpart in the reference (its closest
+ * relative is scalarop_t::to_cppstr, src/einsummable/scalarop.cc:1495-1555). */
+int es_km_codegen_source(const uint64_t* join_shape, int join_rank, const int* inns_flat,
+                         const int* inns_offsets, int n_inns, int out_rank, const char* join_text,
+                         char castable, int compile, char* out, size_t cap);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

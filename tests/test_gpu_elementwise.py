@@ -1,0 +1,229 @@
+"""Parity of the generated elementwise / reduction kernels with the CPU oracle, through the
+C ABI.  The forms are the ones the LLaMA layer and the benchmark configurations use (the
+reference exercises the same forms in exps/gpuexec_kernelmanager.cc and
+exps/cpuexec_kernels.cc:88-318) plus ragged shapes that force the scalar paths."""
+import numpy as np
+import pytest
+
+import einsummable_amd as ea
+import oracle
+from helpers import (NP, assert_bits_equal, assert_close, normal, oracle_einsummable, rng,
+                     run_einsummable, uniform)
+
+pytestmark = pytest.mark.gpu
+
+E = ea.Einsummable
+
+RELU_MUL = "*[ite_>=[constant{f16|0},hole|f16@0,constant{f16|0},hole|f16@0],hole|f16@1]"
+EXP_SUB = "exp[+[hole|f16@0,*[constant{f16|-1},hole|f16@1]]]"
+SILU = "*[hole|f16@0,power{-1}[+[constant{f16|1},exp[*[constant{f16|-1},hole|f16@0]]]]]"
+
+
+def inputs_for(e, r, sd=1.0, positive=False):
+    _, dts = oracle.scalarop_info(e.join)
+    xs = []
+    for k, dt in enumerate(dts):
+        n = int(np.prod(e.inn_shape(k)))
+        x = normal(r, n, NP[dt], sd)
+        if positive:
+            x = np.abs(x) + np.asarray(0.5, dtype=x.dtype)
+        xs.append(x)
+    return xs
+
+
+def check(km, e, seed=0, positive=False, sd=1.0, exact=False, scale=None):
+    xs = inputs_for(e, rng(seed), sd, positive)
+    got = run_einsummable(km, e, xs)
+    od, _ = oracle.scalarop_info(e.join)
+    if exact:
+        want = oracle_einsummable(e, xs, oracle.EXACT)
+        assert_bits_equal(got, want, "%s %s" % (e.join_shape, e.join))
+    else:
+        want = oracle_einsummable(e, xs, oracle.WIDE)
+        assert_close(got, want, od, scale=scale, what="%s %s" % (e.join_shape, e.join))
+    return got
+
+
+UNARY = [
+    ("to_f32[hole|f16@0]", True),
+    ("to_f16[hole|f32@0]", True),
+    ("to_f64[hole|f32@0]", True),
+    ("to_f32[hole|f64@0]", True),
+    ("power{2}[hole|f32@0]", False),
+    ("power{-0.5}[hole|f32@0]", False),
+    ("power{-1}[hole|f32@0]", False),
+    ("power{0.5}[hole|f64@0]", False),
+    ("power{1.7}[hole|f32@0]", False),
+    ("exp[hole|f32@0]", False),
+    ("exp[hole|f64@0]", False),
+    ("log[hole|f32@0]", False),
+    ("+[*[constant{f32|0.000244141},hole|f32@0],constant{f32|1e-06}]", False),
+    ("*[constant{f16|0.0883789},hole|f16@0]", True),
+    (SILU, False),
+    ("ite_<[hole|f32@0,constant{f32|0},constant{f32|0},hole|f32@0]", True),
+    ("conj[hole|c64@0]", True),
+    ("real[hole|c64@0]", True),
+    ("imag[hole|c64@0]", True),
+]
+
+
+@pytest.mark.parametrize("join,exact", UNARY)
+@pytest.mark.parametrize("n", [1, 5, 1000, 4099, 65536])
+def test_unary(km, join, exact, n):
+    positive = "log" in join or "power{-0.5}" in join or "power{0.5}" in join or "power{1.7}" in join
+    check(km, E([n], [[0]], 1, join), seed=n, positive=positive, exact=exact)
+
+
+BINARY = [
+    ("+[hole|f16@0,hole|f16@1]", True),
+    ("*[hole|f16@0,hole|f16@1]", True),
+    ("+[hole|f32@0,hole|f32@1]", True),
+    ("*[hole|f64@0,hole|f64@1]", True),
+    ("*[hole|f32@0,power{-1}[hole|f32@1]]", False),
+    ("+[hole|f32@0,*[constant{f32|-1},hole|f32@1]]", True),
+    (RELU_MUL, True),
+    (EXP_SUB, False),
+    ("*[hole|c64@0,hole|c64@1]", False),
+    ("+[hole|c64@0,hole|c64@1]", True),
+    ("complex[hole|f32@0,hole|f32@1]", True),
+    ("ite_==[hole|f32@0,hole|f32@1,constant{f32|1},constant{f32|0}]", True),
+]
+
+
+@pytest.mark.parametrize("join,exact", BINARY)
+def test_binary_straight_and_broadcast(km, join, exact):
+    positive = "power{-1}" in join
+    for shape in ([37], [4096], [3, 5], [64, 96], [7, 1024]):
+        R = len(shape)
+        full = list(range(R))
+        check(km, E(shape, [full, full], R, join), seed=R, positive=positive, exact=exact)
+    # ab,a->ab and ab,b->ab and a,ab->ab
+    for a, b in ((5, 7), (64, 256), (33, 1000)):
+        check(km, E([a, b], [[0, 1], [0]], 2, join), seed=a, positive=positive, exact=exact)
+        check(km, E([a, b], [[0, 1], [1]], 2, join), seed=b, positive=positive, exact=exact)
+        check(km, E([a, b], [[0], [0, 1]], 2, join), seed=a + b, positive=positive, exact=exact)
+
+
+def test_softmax_elementwise_three_inputs(km):
+    # ab,a,a->ab : exp(x - m[a]) / s[a]
+    join = "*[exp[+[hole|f32@0,*[constant{f32|-1},hole|f32@1]]],power{-1}[hole|f32@2]]"
+    check(km, E([48, 512], [[0, 1], [0], [0]], 2, join), seed=3, positive=True)
+
+
+def test_rotary_complex_broadcast(km):
+    # abcd,bd->abcd complex multiply (src/engine/cpu/kernel_executor.cc:272-314)
+    check(km, E([2, 16, 4, 32], [[0, 1, 2, 3], [1, 3]], 4, "*[hole|c64@0,hole|c64@1]"), seed=11)
+
+
+def test_outer_product_and_pure_broadcast(km):
+    check(km, E([40, 72], [[0], [1]], 2, "*[hole|f32@0,hole|f32@1]"), seed=1, exact=True)
+    check(km, E([6, 40], [[1]], 2, "hole|f32@0"), seed=2, exact=True)   # b->ab
+    check(km, E([40, 6], [[0]], 2, "hole|f16@0"), seed=3, exact=True)   # a->ab
+
+
+@pytest.mark.parametrize("dt", ["f16", "f32", "f64"])
+def test_permute_inner_preserved(km, dt):
+    # abcd->acbd: the innermost mode stays innermost (a strided row copy)
+    check(km, E([4, 6, 5, 64], [[0, 2, 1, 3]], 4, "hole|%s@0" % dt), seed=4, exact=True)
+    check(km, E([3, 5, 4, 7], [[0, 2, 1, 3]], 4, "hole|%s@0" % dt), seed=5, exact=True)
+
+
+def test_transposed_input_elementwise(km):
+    # ba,ab->ab: the first input is read transposed
+    check(km, E([24, 40], [[1, 0], [0, 1]], 2, "+[hole|f32@0,hole|f32@1]"), seed=6, exact=True)
+
+
+def test_output_may_alias_input(km):
+    """Straight elementwise ops may be run in place (donation, memgraph.h:278-287)."""
+    import torch
+    from helpers import stream_handle, to_device, to_host
+
+    e = E([10000], [[0], [0]], 1, "+[hole|f16@0,hole|f16@1]")
+    km.build(e)
+    r = rng(8)
+    x, y = normal(r, 10000, np.float16), normal(r, 10000, np.float16)
+    dx, dy = to_device(x), to_device(y)
+    km(e, stream_handle(), dx.data_ptr(), [dx.data_ptr(), dy.data_ptr()])
+    torch.cuda.synchronize()
+    assert_bits_equal(to_host(dx, np.float16), (x + y).astype(np.float16), "in-place add")
+
+
+REDUCTIONS = ["+", "x", "v", "^"]
+
+
+@pytest.mark.parametrize("castable", REDUCTIONS)
+@pytest.mark.parametrize("dt", ["f16", "f32", "f64"])
+def test_row_reduction_ab_a(km, castable, dt):
+    for a, b in ((1, 1), (3, 5), (17, 64), (9, 1000), (130, 4096), (4, 20000)):
+        sd = 1.0
+        if castable == "x":
+            if b > 1000:
+                continue
+            sd = 0.05  # products stay in range
+        e = E([a, b], [[0, 1]], 1, "hole|%s@0" % dt, castable)
+        xs = inputs_for(e, rng(a * 7 + b), sd)
+        if castable == "x":
+            xs = [np.asarray(1.0, xs[0].dtype) + xs[0]]
+        got = run_einsummable(km, e, xs)
+        od, _ = oracle.scalarop_info(e.join)
+        if castable in ("v", "^"):
+            assert_bits_equal(got, oracle_einsummable(e, xs, oracle.EXACT), "min/max reduce")
+        else:
+            assert_close(got, oracle_einsummable(e, xs, oracle.WIDE), od, what="reduce %s" % castable)
+
+
+def test_fused_exp_sub_row_sum(km):
+    # ab,a->a : sum_b exp(x[a,b] - m[a])
+    for dt, shape in (("f16", (64, 2048)), ("f32", (33, 1000)), ("f32", (8, 8))):
+        join = "exp[+[hole|%s@0,*[constant{%s|-1},hole|%s@1]]]" % (dt, dt, dt)
+        check(km, E(list(shape), [[0, 1], [0]], 1, join, "+"), seed=9)
+
+
+def test_column_and_middle_reductions(km):
+    check(km, E([64, 40], [[1, 0]], 1, "hole|f32@0", "+"), seed=10)             # ba->a
+    check(km, E([6, 32, 20], [[0, 2, 1]], 2, "hole|f32@0", "+"), seed=11)       # acb->ab
+    check(km, E([6, 32, 20], [[0, 2, 1]], 2, "hole|f16@0", "^"), seed=12, exact=True)
+    check(km, E([5, 7, 3, 4], [[0, 2, 1, 3]], 2, "hole|f64@0", "+"), seed=13)   # two agg modes
+    check(km, E([5, 3, 4], [[0, 1, 2], [0, 1, 2]], 1, "*[hole|f32@0,hole|f32@1]", "+"), seed=14)
+
+
+def test_generic_contractions_through_codegen(km):
+    """Contractions in dtypes without a matrix-core kernel fall back to generated code."""
+    check(km, E([6, 5, 7], [[0, 2], [2, 1]], 2, "*[hole|c64@0,hole|c64@1]", "+"), seed=15)
+
+
+def test_merged_and_unmerged_descriptors_agree(km):
+    r = rng(16)
+    x = normal(r, 3 * 4 * 5 * 6, np.float32)
+    y = normal(r, 3 * 4, np.float32)
+    full = E([3, 4, 5, 6], [[0, 1, 2, 3], [0, 1]], 4, "*[hole|f32@0,hole|f32@1]")
+    merged = E([12, 30], [[0, 1], [0]], 2, "*[hole|f32@0,hole|f32@1]")
+    assert oracle.merge_adjacent_dims(full.join_shape, full.inns, 4) == ([12, 30], [[0, 1], [0]], 2)
+    a = run_einsummable(km, full, [x, y])
+    b = run_einsummable(km, merged, [x, y])
+    assert_bits_equal(a, b, "merge_adjacent_dims invariance")
+
+
+def test_error_contract(km):
+    import torch
+
+    e = E([123], [[0]], 1, "exp[hole|f32@0]")
+    d = torch.zeros(123, device="cuda")
+    with pytest.raises(ea.KmError) as ei:   # not built
+        km(e, 0, d.data_ptr(), [d.data_ptr()])
+    assert ei.value.code == -2
+    with pytest.raises(ea.KmError) as ei:
+        km.workspace_size(e)
+    assert ei.value.code == -2
+    assert km.build(e) == 0
+    assert km.workspace_size(e) == 0
+    with pytest.raises(ea.KmError) as ei:   # wrong number of inputs
+        km(e, 0, d.data_ptr(), [d.data_ptr(), d.data_ptr()])
+    assert ei.value.code == -4
+    with pytest.raises(ea.KmError) as ei:   # malformed join
+        km.build(E([4], [[0]], 1, "exp[hole|f32@0"))
+    assert ei.value.code == -1
+    with pytest.raises(ea.KmError):         # aggregation without castable
+        km.build(E([4, 4], [[0, 1]], 1, "hole|f32@0"))
+    # scalar variables must be substituted by the caller: unsupported, not an error
+    assert km.build(E([4], [[0]], 1, "*[variable{lr|f32},hole|f32@0]")) is None
