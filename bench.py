@@ -1,0 +1,310 @@
+#!/usr/bin/env python3
+"""Benchmark of the apply-node kernel path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c1|c3|c4|all]
+
+The headline workload is the fused elementwise + reduce configuration (f16, 8192 x 8192):
+one "step" runs its four apply nodes through the C-ABI kernel manager on buffers that are
+already resident in HBM:
+    (i)   ij,ij->ij   max(x,0) * y
+    (ii)  ij->i       row max of x
+    (iii) ij,i->ij    exp(x - rowmax)
+    (iv)  ij->i       row sum of (iii)
+`value` is algorithmic bytes per step / wall time per step (host launch cost included).
+`roofline` is the dominant kernel -- node (i) -- timed with events on the launch stream.
+`cpu_baseline` times the CPU oracle (a single-threaded C port of the reference semantics) on
+a bounded sample of the same workload.  Other workloads are reported under "others".
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E
+PEAK_TFLOPS = {"f16": 2500.0, "f32": 157.3, "f64": 78.6}
+
+RELU_MUL = "*[ite_>=[constant{f16|0},hole|f16@0,constant{f16|0},hole|f16@0],hole|f16@1]"
+EXP_SUB = "exp[+[hole|f16@0,*[constant{f16|-1},hole|f16@1]]]"
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="all", choices=["c2", "c1", "c3", "c4", "all"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    return ap.parse_args()
+
+
+class Timed:
+    """Average duration of one launch site, from events recorded on the launch stream."""
+
+    def __init__(self):
+        self.pairs = []
+
+    def record(self, fn):
+        import torch
+
+        a = torch.cuda.Event(enable_timing=True)
+        b = torch.cuda.Event(enable_timing=True)
+        a.record()
+        fn()
+        b.record()
+        self.pairs.append((a, b))
+
+    def mean_ms(self):
+        return sum(a.elapsed_time(b) for a, b in self.pairs) / max(len(self.pairs), 1)
+
+
+def c2_nodes(n):
+    import einsummable_amd as ea
+
+    E = ea.Einsummable
+    return [
+        ("relu_mul ij,ij->ij", E([n, n], [[0, 1], [0, 1]], 2, RELU_MUL), 3 * n * n * 2),
+        ("rowmax ij->i", E([n, n], [[0, 1]], 1, "hole|f16@0", "^"), n * n * 2 + n * 2),
+        ("exp_sub ij,i->ij", E([n, n], [[0, 1], [0]], 2, EXP_SUB), 2 * n * n * 2 + n * 2),
+        ("rowsum ij->i", E([n, n], [[0, 1]], 1, "hole|f16@0", "+"), n * n * 2 + n * 2),
+    ]
+
+
+def run_c2(km, steps, warmup):
+    import torch
+
+    n = 8192
+    g = torch.Generator(device="cuda").manual_seed(0)
+    x = torch.randn(n, n, device="cuda", dtype=torch.float16, generator=g)
+    y = torch.randn(n, n, device="cuda", dtype=torch.float16, generator=g)
+    z = torch.empty_like(x)
+    ex = torch.empty_like(x)
+    m = torch.empty(n, device="cuda", dtype=torch.float16)
+    s = torch.empty(n, device="cuda", dtype=torch.float16)
+    nodes = c2_nodes(n)
+    for _, e, _ in nodes:
+        assert km.build(e) == 0
+    stream = torch.cuda.current_stream().cuda_stream
+    calls = [
+        lambda: km(nodes[0][1], stream, z.data_ptr(), [x.data_ptr(), y.data_ptr()]),
+        lambda: km(nodes[1][1], stream, m.data_ptr(), [x.data_ptr()]),
+        lambda: km(nodes[2][1], stream, ex.data_ptr(), [x.data_ptr(), m.data_ptr()]),
+        lambda: km(nodes[3][1], stream, s.data_ptr(), [ex.data_ptr()]),
+    ]
+    timers = [Timed() for _ in calls]
+
+    for _ in range(warmup):
+        for c in calls:
+            c()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        for c, t in zip(calls, timers):
+            t.record(c)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+
+    total_bytes = sum(b for _, _, b in nodes)
+    per_node = []
+    for (name, e, nbytes), t in zip(nodes, timers):
+        ms = t.mean_ms()
+        per_node.append({"node": name, "kernel": km.describe(e), "bytes": nbytes,
+                         "ms": round(ms, 5), "GBps": round(nbytes / ms / 1e6, 1),
+                         "hbm_frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4)})
+    return {"wall_s": wall, "bytes_per_step": total_bytes, "per_node": per_node,
+            "tensors": (x, y, m)}
+
+
+def cpu_baseline_c2(rows=4096):
+    """The CPU oracle (kind "port": a single-threaded C restatement of the reference's scalar
+    interpreter semantics) on the first `rows` rows of the same four nodes."""
+    import numpy as np
+
+    import oracle
+
+    n = 8192
+    r = np.random.RandomState(0)
+    x = r.normal(0, 1, (rows, n)).astype(np.float16)
+    y = r.normal(0, 1, (rows, n)).astype(np.float16)
+    t0 = time.perf_counter()
+    oracle.einsummable([rows, n], [[0, 1], [0, 1]], 2, RELU_MUL, None, [x, y], oracle.EXACT)
+    m = oracle.einsummable([rows, n], [[0, 1]], 1, "hole|f16@0", "^", [x], oracle.EXACT)
+    ex = oracle.einsummable([rows, n], [[0, 1], [0]], 2, EXP_SUB, None, [x, m], oracle.EXACT)
+    oracle.einsummable([rows, n], [[0, 1]], 1, "hole|f16@0", "+", [ex], oracle.EXACT)
+    dt = time.perf_counter() - t0
+    nbytes = rows * n * 2 * (3 + 1 + 2 + 1) + 3 * rows * 2
+    return {"value": round(nbytes / dt / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": "first %d of 8192 rows of the four nodes, %.1f s" % (rows, dt)}
+
+
+def run_contraction(km, name, e, shapes, dtype, flops, steps, warmup):
+    import torch
+
+    tdt = {"f16": torch.float16, "f32": torch.float32, "f64": torch.float64}[dtype]
+    g = torch.Generator(device="cuda").manual_seed(1)
+    ins = [torch.randn(*s, device="cuda", dtype=tdt, generator=g) for s in shapes[:-1]]
+    out = torch.empty(*shapes[-1], device="cuda", dtype=tdt)
+    ws = km.build(e)
+    if ws is None:
+        return {"node": name, "error": "unsupported"}
+    wbuf = torch.empty(max(ws, 1), device="cuda", dtype=torch.uint8)
+    if not km.describe(e).startswith("contraction"):
+        # generated fallback kernel (no matrix-core path for this form): keep the run short
+        steps, warmup = min(steps, 2), 1
+    stream = torch.cuda.current_stream().cuda_stream
+    call = lambda: km(e, stream, out.data_ptr(), [t.data_ptr() for t in ins],
+                      (wbuf.data_ptr(), ws) if ws else None)
+    for _ in range(warmup):
+        call()
+    torch.cuda.synchronize()
+    t = Timed()
+    for _ in range(steps):
+        t.record(call)
+    torch.cuda.synchronize()
+    ms = t.mean_ms()
+    tf = flops / ms / 1e9
+    return {"node": name, "kernel": km.describe(e), "flop": flops, "ms": round(ms, 5),
+            "TFLOPs": round(tf, 2), "mfma_frac": round(tf / PEAK_TFLOPS[dtype], 4)}
+
+
+def run_c1(km, steps, warmup):
+    import einsummable_amd as ea
+
+    n = 2048
+    e = ea.Einsummable([n, n, n], [[0, 2], [2, 1]], 2, "*[hole|f32@0,hole|f32@1]", "+")
+    return run_contraction(km, "c1 ij,jk->ik f32 2048^3", e, [(n, n), (n, n), (n, n)], "f32",
+                           2 * n ** 3, steps, warmup)
+
+
+def run_c3(km, steps, warmup):
+    import numpy as np
+    import torch
+
+    import einsummable_amd as ea
+
+    out = []
+    # (a) abcd->acbd of a [32, 2048, 32, 128] f16 tensor
+    a, b, c, d = 32, 2048, 32, 128
+    e = ea.Einsummable([a, c, b, d], [[0, 2, 1, 3]], 4, "hole|f16@0")
+    x = torch.randn(a, b, c, d, device="cuda", dtype=torch.float16)
+    y = torch.empty(a, c, b, d, device="cuda", dtype=torch.float16)
+    assert km.build(e) == 0
+    stream = torch.cuda.current_stream().cuda_stream
+    call = lambda: km(e, stream, y.data_ptr(), [x.data_ptr()])
+    for _ in range(warmup):
+        call()
+    torch.cuda.synchronize()
+    t = Timed()
+    for _ in range(steps):
+        t.record(call)
+    torch.cuda.synchronize()
+    nbytes = 2 * x.numel() * 2
+    ms = t.mean_ms()
+    out.append({"node": "c3a permute abcd->acbd f16 32x2048x32x128", "kernel": km.describe(e),
+                "bytes": nbytes, "ms": round(ms, 5), "GBps": round(nbytes / ms / 1e6, 1),
+                "hbm_frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4)})
+    del x, y
+    # (b) 64 accumulate touches of 512x512 into random windows of a zeroed 4096x4096 matrix
+    n, blk, count = 4096, 512, 64
+    r = np.random.RandomState(0)
+    acc = torch.zeros(n, n, device="cuda", dtype=torch.float16)
+    blocks = [torch.randn(blk, blk, device="cuda", dtype=torch.float16) for _ in range(count)]
+    touches = []
+    for _ in range(count):
+        ro, co = int(r.randint(0, n - blk + 1)), int(r.randint(0, n - blk + 1))
+        touches.append(ea.Touch([(blk, n, 0, ro, blk), (blk, n, 0, co, blk)], "+", ea.F16))
+
+    def all_touches():
+        for tch, bl in zip(touches, blocks):
+            km.touch(tch, stream, acc.data_ptr(), bl.data_ptr())
+
+    for _ in range(warmup):
+        all_touches()
+    torch.cuda.synchronize()
+    t = Timed()
+    for _ in range(steps):
+        t.record(all_touches)
+    torch.cuda.synchronize()
+    nbytes = count * 3 * blk * blk * 2
+    ms = t.mean_ms()
+    out.append({"node": "c3b 64 touch(add) 512x512 into 4096x4096 f16", "bytes": nbytes,
+                "ms": round(ms, 5), "GBps": round(nbytes / ms / 1e6, 1),
+                "hbm_frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4)})
+    return out
+
+
+def run_c4(km, steps, warmup):
+    import einsummable_amd as ea
+
+    b, h, s, d = 4, 32, 2048, 128
+    flops = 2 * b * h * s * s * d
+    mul = "*[hole|f16@0,hole|f16@1]"
+    e1 = ea.Einsummable([b, h, s, s, d], [[0, 1, 2, 4], [0, 1, 3, 4]], 4, mul, "+")
+    e2 = ea.Einsummable([b, h, s, d, s], [[0, 1, 2, 4], [0, 1, 4, 3]], 4, mul, "+")
+    r1 = run_contraction(km, "c4 scores bhid,bhjd->bhij f16", e1,
+                         [(b, h, s, d), (b, h, s, d), (b, h, s, s)], "f16", flops, steps, warmup)
+    r2 = run_contraction(km, "c4 values bhij,bhjd->bhid f16", e2,
+                         [(b, h, s, s), (b, h, s, d), (b, h, s, d)], "f16", flops, steps, warmup)
+    return [r1, r2]
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures the apply-node kernels of ONE GPU; --gpus %d is not supported "
+              "(an apply node never spans devices)." % args.gpus, file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    import einsummable_amd as ea
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.init()
+    km = ea.KernelManager(0)
+
+    c2 = run_c2(km, args.steps, args.warmup)
+    ms_per_step = c2["wall_s"] / args.steps * 1e3
+    value = c2["bytes_per_step"] / (c2["wall_s"] / args.steps) / 1e9
+    dom = max(c2["per_node"], key=lambda p: p["bytes"])
+    roofline = {"bound": "hbm", "kernel": dom["node"] + " [" + dom["kernel"] + "]",
+                "achieved": dom["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                "frac": round(dom["GBps"] / HBM_PEAK_GBPS, 4), "traffic": None}
+    others = {"c2_nodes": c2["per_node"]}
+    del c2
+    torch.cuda.empty_cache()
+    if args.workload in ("c1", "all"):
+        others["c1"] = run_c1(km, args.steps, args.warmup)
+    if args.workload in ("c3", "all"):
+        others["c3"] = run_c3(km, args.steps, args.warmup)
+    if args.workload in ("c4", "all"):
+        others["c4"] = run_c4(km, max(args.steps // 5, 3), max(args.warmup // 5, 1))
+
+    line = {
+        "metric": "elementwise/reduce GB/s (apply-node kernel path; contraction TFLOP/s and "
+                  "touch/permute GB/s under 'others')",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": "C2 fused elementwise + reduce, f16 8192x8192: max(x,0)*y; "
+                               "row max; exp(x-rowmax); row sum"},
+        "roofline": roofline,
+        "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline_c2(),
+        "others": others,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -127,3 +127,22 @@ def assert_bits_equal(got, want, what=""):
             "%s: %d of %d elements differ bitwise; first at %d: got %r want %r"
             % (what, idx.size, got.size, idx[0], got.reshape(-1)[idx[0]], want.reshape(-1)[idx[0]])
         )
+
+
+def assert_values_equal(got, want, what=""):
+    """Exact equality of values: bitwise, except that +0 and -0 compare equal and any NaN
+    matches any NaN.  Used for computed results whose single rounding is fully determined
+    (the GPU compiler may fuse a multiply into an fma with a +0 addend, which only changes
+    the sign of a zero result)."""
+    got = np.ascontiguousarray(got)
+    want = np.ascontiguousarray(want)
+    assert got.dtype == want.dtype and got.shape == want.shape, (got.dtype, want.dtype)
+    g = got.view(np.float32) if got.dtype == np.complex64 else got
+    w = want.view(np.float32) if want.dtype == np.complex64 else want
+    same = (g == w) | (np.isnan(g) & np.isnan(w))
+    if not same.all():
+        idx = np.nonzero(~same)[0]
+        raise AssertionError(
+            "%s: %d of %d values differ; first at %d: got %r want %r"
+            % (what, idx.size, g.size, idx[0], g[idx[0]], w[idx[0]])
+        )
