@@ -393,7 +393,7 @@ cg_kernel_t gen_elementwise(einsummable_t const& e, int max_vec)
     }
     s << "    idx_t vid[U];\n    bool live[U];\n";
     s << "#pragma unroll\n    for (int u = 0; u != U; ++u) {\n";
-    s << "        vid[u] = ((idx_t)blockIdx.x * U + u) * 256 + threadIdx.x;\n";
+    s << "        vid[u] = (((idx_t)blockIdx.y * gridDim.x + blockIdx.x) * U + u) * 256 + threadIdx.x;\n";
     s << "        live[u] = vid[u] < n_vec;\n";
     s << "        if (live[u]) {\n";
     if (!all_straight) {
@@ -451,7 +451,7 @@ cg_kernel_t gen_elementwise(einsummable_t const& e, int max_vec)
       << ", V>*>(a.out + vid[u] * V) = res;\n";
     s << "        }\n    }\n";
     if (tail) {
-        s << "    if (blockIdx.x == 0 && threadIdx.x < " << tail << ") {\n";
+        s << "    if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x < " << tail << ") {\n";
         s << "        const idx_t i = n_vec * V + threadIdx.x;\n";
         s << "        a.out[i] = " << g.store_cast([&] {
             std::string call = "join_fn(";
@@ -527,7 +527,7 @@ cg_kernel_t gen_reduce_row(einsummable_t const& e, int max_vec)
     s << "    const idx_t n_out = " << g.P(p_nout) << ";\n";
     s << "    const idx_t nvec = " << g.P(p_nvec) << ";\n";
     s << "    const unsigned lane = threadIdx.x % TEAM;\n";
-    s << "    const idx_t row = (idx_t)blockIdx.x * (" << BLOCK << " / TEAM) + threadIdx.x / TEAM;\n";
+    s << "    const idx_t row = ((idx_t)blockIdx.y * gridDim.x + blockIdx.x) * (" << BLOCK << " / TEAM) + threadIdx.x / TEAM;\n";
     s << "    " << ACC << " acc = " << identity_of(cast, od) << ";\n";
     s << "    if (row < n_out) {\n";
     s << "        idx_t rem = row;\n";
@@ -681,7 +681,7 @@ cg_kernel_t gen_reduce_col(einsummable_t const& e, int max_vec)
     s << "__device__ __forceinline__ " << ACC << " comb(" << ACC << " x, " << ACC
       << " y) { return " << combine_expr(cast, od, "x", "y") << "; }\n";
     s << "extern \"C\" __global__ __launch_bounds__(256) void es_kernel(args_t a)\n{\n";
-    s << "    const idx_t vid = (idx_t)blockIdx.x * 256 + threadIdx.x;\n";
+    s << "    const idx_t vid = ((idx_t)blockIdx.y * gridDim.x + blockIdx.x) * 256 + threadIdx.x;\n";
     s << "    if (vid >= " << g.P(p_nvec) << ") return;\n";
     s << "    idx_t rem = vid;\n";
     s << "    const idx_t c = (rem % " << g.P(p_vpr) << ") * V;\n";
@@ -886,8 +886,13 @@ struct codegen_plan_t : plan_t {
         }
         void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, buf, HIP_LAUNCH_PARAM_BUFFER_SIZE, &n,
                           HIP_LAUNCH_PARAM_END};
-        hipError_t err = hipModuleLaunchKernel(v.fn, unsigned(v.k.grid), 1, 1, v.k.block, 1, 1, 0,
-                                               stream, nullptr, config);
+        // a grid dimension times the block size must stay below 2^32: fold large grids
+        // into two dimensions (the kernels linearise blockIdx.y * gridDim.x + blockIdx.x)
+        uint64_t const gx_max = 1ull << 22;
+        unsigned gx = unsigned(std::min<uint64_t>(v.k.grid, gx_max));
+        unsigned gy = unsigned((v.k.grid + gx - 1) / gx);
+        hipError_t err = hipModuleLaunchKernel(v.fn, gx, gy, 1, v.k.block, 1, 1, 0, stream,
+                                               nullptr, config);
         if (err != hipSuccess) {
             throw km_error(km_status::device,
                            std::string("hipModuleLaunchKernel: ") + hipGetErrorString(err));
@@ -935,7 +940,7 @@ std::shared_ptr<plan_t> plan_codegen(einsummable_t const& e, int)
     } catch (ir_error const&) {
         return nullptr;
     }
-    if (k.grid >= (1ull << 31)) return nullptr;
+    if (k.grid >= (1ull << 36)) return nullptr;
     if (8 * (1 + k.n_inns) + 8 * k.params.size() > 1000) return nullptr;
     auto p = std::make_shared<codegen_plan_t>(e);
     p->wide.k = std::move(k);

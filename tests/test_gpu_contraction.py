@@ -1,0 +1,129 @@
+"""Parity of the MFMA contraction path with the CPU oracle (computed in double, rounded once):
+every b/i/j/k mode arrangement the planner distinguishes, ragged sizes that exercise the tile
+edges, and the LLaMA layer's forms at reduced sizes.  fp32 within 1e-4, fp16 within 1e-2 of
+the higher-precision result; f64 to 1e-10."""
+import numpy as np
+import pytest
+
+import einsummable_amd as ea
+import oracle
+from helpers import NP, assert_close, normal, oracle_einsummable, rng, run_einsummable, uniform
+
+pytestmark = pytest.mark.gpu
+
+E = ea.Einsummable
+DT = {"f16": ea.F16, "f32": ea.F32, "f64": ea.F64}
+
+
+def contraction(spec, sizes, dt):
+    join = "*[hole|%s@0,hole|%s@1]" % (dt, dt)
+    return E.from_str(spec, sizes, join, "+")
+
+
+def check(km, spec, sizes, dt, seed=0, expect_mfma=True):
+    e = contraction(spec, sizes, dt)
+    r = rng(seed)
+    xs = [uniform(r, int(np.prod(e.inn_shape(k))), NP[DT[dt]]) for k in range(2)]
+    got = run_einsummable(km, e, xs)
+    if expect_mfma:
+        assert km.describe(e).startswith("contraction_mfma_" + dt), km.describe(e)
+    want = oracle_einsummable(e, xs, oracle.WIDE)
+    assert_close(got, want, DT[dt], what="%s %s %s [%s]" % (spec, sizes, dt, km.describe(e)))
+
+
+@pytest.mark.parametrize("dt", ["f16", "f32", "f64"])
+def test_reference_known_answer_shape(km, dt):
+    # tests/reference.h:4-49: 3x4 times 4x5 with iota(8) / iota(100)
+    e = contraction("ij,jk->ik", dict(i=3, j=4, k=5), dt)
+    lhs = np.arange(8, 20, dtype=NP[DT[dt]])
+    rhs = np.arange(100, 120, dtype=NP[DT[dt]])
+    got = run_einsummable(km, e, [lhs, rhs])
+    want = np.array([4110, 4148, 4186, 4224, 4262, 5830, 5884, 5938, 5992, 6046, 7550, 7620, 7690,
+                     7760, 7830], dtype=np.float64)
+    assert_close(got, want, DT[dt], what="known-answer matmul")
+
+
+MATMULS = ["ij,jk->ik", "ij,kj->ik", "ji,jk->ik", "ji,kj->ik",
+           "jk,ij->ik", "kj,ij->ik", "jk,ji->ik", "kj,ji->ik"]
+
+
+@pytest.mark.parametrize("dt", ["f16", "f32", "f64"])
+@pytest.mark.parametrize("spec", MATMULS)
+def test_all_matmul_spellings(km, spec, dt):
+    check(km, spec, dict(i=64, j=96, k=80), dt, seed=1)       # vector paths
+    check(km, spec, dict(i=37, j=51, k=29), dt, seed=2)       # ragged: elementwise paths
+
+
+@pytest.mark.parametrize("dt", ["f16", "f32"])
+def test_tile_edges_and_deep_k(km, dt):
+    check(km, "ij,kj->ik", dict(i=130, j=264, k=136), dt, seed=3)
+    check(km, "ij,kj->ik", dict(i=256, j=1024, k=128), dt, seed=4)
+    check(km, "ij,jk->ik", dict(i=200, j=72, k=392), dt, seed=5)
+    check(km, "ij,jk->ik", dict(i=1, j=512, k=8), dt, seed=6)
+    check(km, "ij,jk->ik", dict(i=8, j=8, k=1), dt, seed=7)
+
+
+BATCHED = [
+    ("bij,bjk->bik", dict(b=3, i=40, j=48, k=56)),
+    ("bij,jk->bik", dict(b=3, i=40, j=48, k=56)),        # b is an m mode here
+    ("ibj,bjk->bik", dict(b=3, i=40, j=48, k=56)),       # batch in the middle of lhs
+    ("bij,bjk->ikb", dict(b=4, i=24, j=16, k=40)),       # batch innermost in out
+    ("bij,bkj->bki", dict(b=2, i=40, j=32, k=24)),       # lhs owns the innermost out mode
+    ("abij,abkj->abik", dict(a=2, b=3, i=24, j=32, k=40)),
+    ("aibj,akbj->abik", dict(a=2, b=3, i=24, j=32, k=40)),
+]
+
+
+@pytest.mark.parametrize("dt", ["f16", "f32", "f64"])
+@pytest.mark.parametrize("spec,sizes", BATCHED)
+def test_batched_forms(km, spec, sizes, dt):
+    check(km, spec, sizes, dt, seed=8)
+
+
+@pytest.mark.parametrize("dt", ["f16", "f32"])
+def test_llama_attention_forms(km, dt):
+    # scores acbe,adbe->abcd ; P.V abce,aebd->abcd ; out-proj adbe,cde->abc and adbe,dec->abc
+    # (exps/gpuexec_kernelmanager.cc:993, 3120-3132; llama/modules.cc:315-352), reduced sizes
+    check(km, "acbe,adbe->abcd", dict(a=1, b=4, c=72, d=88, e=64), dt, seed=9)
+    check(km, "abce,aebd->abcd", dict(a=1, b=4, c=72, e=88, d=64), dt, seed=10)
+    check(km, "adbe,cde->abc", dict(a=1, d=4, b=72, e=64, c=96), dt, seed=11)
+    check(km, "adbe,dec->abc", dict(a=1, d=4, b=72, e=64, c=96), dt, seed=12)
+    check(km, "bhid,bhjd->bhij", dict(b=2, h=3, i=40, j=56, d=128), dt, seed=13)
+    check(km, "bhij,bhjd->bhid", dict(b=2, h=3, i=40, j=56, d=128), dt, seed=14)
+
+
+@pytest.mark.parametrize("dt", ["f16", "f32"])
+def test_multi_mode_groups(km, dt):
+    # two k modes whose order differs between the operands, two m modes, two n modes
+    check(km, "ipq,qpk->ik", dict(i=24, p=6, q=16, k=40), dt, seed=15)
+    check(km, "xiyj,jk->xyik", dict(x=3, y=5, i=8, j=32, k=24), dt, seed=16)
+    check(km, "ij,xjyk->iyxk", dict(x=3, y=5, i=8, j=32, k=24), dt, seed=17)
+
+
+def test_one_sided_aggregation_is_not_a_gemm(km):
+    # j is summed over lhs only, l over rhs only: handled by the generated reduce kernel
+    e = E.from_str("ij,kl->ik", dict(i=6, j=5, k=7, l=4), "*[hole|f32@0,hole|f32@1]", "+")
+    r = rng(18)
+    xs = [uniform(r, 30, np.float32), uniform(r, 28, np.float32)]
+    got = run_einsummable(km, e, xs)
+    assert not km.describe(e).startswith("contraction")
+    assert_close(got, oracle_einsummable(e, xs, oracle.WIDE), ea.F32, what="one-sided agg")
+
+
+def test_misaligned_operands_fall_back_to_elementwise_loads(km):
+    import torch
+    from helpers import stream_handle, to_host
+
+    e = contraction("ij,kj->ik", dict(i=64, j=64, k=64), "f16")
+    km.build(e)
+    r = rng(19)
+    a, b = uniform(r, 64 * 64, np.float16), uniform(r, 64 * 64, np.float16)
+    da = torch.zeros(64 * 64 + 8, dtype=torch.float16, device="cuda")
+    db = torch.zeros(64 * 64 + 8, dtype=torch.float16, device="cuda")
+    dc = torch.zeros(64 * 64 + 8, dtype=torch.float16, device="cuda")
+    da[1:1 + 4096] = torch.from_numpy(a).cuda()
+    db[3:3 + 4096] = torch.from_numpy(b).cuda()
+    km(e, stream_handle(), dc.data_ptr() + 2, [da.data_ptr() + 2, db.data_ptr() + 6])
+    torch.cuda.synchronize()
+    got = dc[1:1 + 4096].cpu().numpy()
+    assert_close(got, oracle_einsummable(e, [a, b], oracle.WIDE), ea.F16, what="misaligned")
