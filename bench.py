@@ -37,7 +37,8 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="all", choices=["c2", "c1", "c3", "c4", "all"])
+    ap.add_argument("--workload", default="all",
+                    choices=["c2", "c1", "c3", "c4", "llama", "all"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     return ap.parse_args()
 
@@ -254,6 +255,33 @@ def run_c4(km, steps, warmup):
     return [r1, r2]
 
 
+def run_llama_contractions(km, steps, warmup):
+    """The contraction nodes of one LLaMA-7B decoder layer (dim 4096, 32 heads of 128,
+    ffn 11008, batch 1, seq 2048), fp16 in / fp32 accumulate, in the merged forms the
+    layer's graph produces (llama/modules.cc:282-356, 410-431)."""
+    import einsummable_amd as ea
+
+    mul = "*[hole|f16@0,hole|f16@1]"
+    s, d, h, hd, f = 2048, 4096, 32, 128, 11008
+    E = ea.Einsummable.from_str
+    cases = [
+        ("qkv/o proj ij,kj->ik 2048x4096x4096", E("ij,kj->ik", dict(i=s, j=d, k=d), mul, "+"),
+         [(s, d), (d, d), (s, d)], 2 * s * d * d),
+        ("w1/w3 ij,kj->ik 2048x4096x11008", E("ij,kj->ik", dict(i=s, j=d, k=f), mul, "+"),
+         [(s, d), (f, d), (s, f)], 2 * s * d * f),
+        ("w2 ij,kj->ik 2048x11008x4096", E("ij,kj->ik", dict(i=s, j=f, k=d), mul, "+"),
+         [(s, f), (d, f), (s, d)], 2 * s * d * f),
+        ("scores acbe,adbe->abcd", E("acbe,adbe->abcd", dict(a=1, b=h, c=s, d=s, e=hd), mul, "+"),
+         [(1, s, h, hd), (1, s, h, hd), (1, h, s, s)], 2 * h * s * s * hd),
+        ("values abce,aebd->abcd", E("abce,aebd->abcd", dict(a=1, b=h, c=s, e=s, d=hd), mul, "+"),
+         [(1, h, s, s), (1, s, h, hd), (1, h, s, hd)], 2 * h * s * s * hd),
+        ("out proj adbe,cde->abc", E("adbe,cde->abc", dict(a=1, d=h, b=s, e=hd, c=d), mul, "+"),
+         [(1, h, s, hd), (d, h, hd), (1, s, d)], 2 * s * d * d),
+    ]
+    return [run_contraction(km, name, e, shapes, "f16", flops, steps, warmup)
+            for name, e, shapes, flops in cases]
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -284,6 +312,9 @@ def main():
         others["c3"] = run_c3(km, args.steps, args.warmup)
     if args.workload in ("c4", "all"):
         others["c4"] = run_c4(km, max(args.steps // 5, 3), max(args.warmup // 5, 1))
+    if args.workload in ("llama", "all"):
+        others["llama7b_contractions"] = run_llama_contractions(km, max(args.steps // 5, 3),
+                                                                max(args.warmup // 5, 1))
 
     line = {
         "metric": "elementwise/reduce GB/s (apply-node kernel path; contraction TFLOP/s and "

@@ -306,6 +306,32 @@ struct gen_t {
     }
 };
 
+// Entry point name that identifies the kernel in profiles: kind, einsummable string, output
+// dtype and a hash of the join text, e.g. es_ew__ab_a__ab__f16_1a2b3c4d.
+std::string entry_name(einsummable_t const& e, const char* kind)
+{
+    std::string s = std::string("es_") + kind + "__";
+    for (char c : e.str()) {
+        if (c == ',') {
+            s += '_';
+        } else if (c == '-') {
+            s += "__";
+        } else if (c != '>') {
+            s += c;
+        }
+    }
+    s += std::string("__") + dtype_name(e.out_dtype());
+    if (e.castable) {
+        static const char* names[] = {"add", "mul", "min", "max"};
+        s += std::string("_") + names[int(e.castable.value())];
+    }
+    uint32_t h = 2166136261u;
+    for (char c : e.join.str()) h = (h ^ uint8_t(c)) * 16777619u;
+    char buf[16];
+    std::snprintf(buf, sizeof(buf), "_%08x", h);
+    return s + buf;
+}
+
 bool fits32(einsummable_t const& e)
 {
     uint64_t const lim = (1ull << 32) - 1;
@@ -341,7 +367,7 @@ cg_kernel_t gen_elementwise(einsummable_t const& e, int max_vec)
     g.k.kind = cg_kind::elementwise;
     g.k.n_inns = L.NI;
     g.k.idx64 = !fits32(e);
-    g.k.entry = "es_kernel";
+    g.k.entry = entry_name(e, "ew");
 
     std::vector<access_t> acc(L.NI);
     bool all_straight = true;
@@ -381,7 +407,7 @@ cg_kernel_t gen_elementwise(einsummable_t const& e, int max_vec)
     g.args_struct();
     auto& s = g.src;
     s << "#define V " << V << "\n#define U " << U << "\n";
-    s << "extern \"C\" __global__ __launch_bounds__(256) void es_kernel(args_t a)\n{\n";
+    s << "extern \"C\" __global__ __launch_bounds__(256) void " << g.k.entry << "(args_t a)\n{\n";
     s << "    const idx_t n_vec = " << g.P(p_nvec) << ";\n";
     for (int k = 0; k != L.NI; ++k) {
         std::string T = storage_type(e.inn_dtype(k));
@@ -488,7 +514,7 @@ cg_kernel_t gen_reduce_row(einsummable_t const& e, int max_vec)
     g.k.kind = cg_kind::reduce_row;
     g.k.n_inns = L.NI;
     g.k.idx64 = !fits32(e);
-    g.k.entry = "es_kernel";
+    g.k.entry = entry_name(e, "redrow");
     castable_t const cast = e.castable.value();
     dtype_t const od = e.out_dtype();
 
@@ -523,7 +549,7 @@ cg_kernel_t gen_reduce_row(einsummable_t const& e, int max_vec)
     s << "#define V " << V << "\n#define U " << U << "\n#define TEAM " << TEAM << "\n";
     s << "__device__ __forceinline__ " << ACC << " comb(" << ACC << " x, " << ACC
       << " y) { return " << combine_expr(cast, od, "x", "y") << "; }\n";
-    s << "extern \"C\" __global__ __launch_bounds__(" << BLOCK << ") void es_kernel(args_t a)\n{\n";
+    s << "extern \"C\" __global__ __launch_bounds__(" << BLOCK << ") void " << g.k.entry << "(args_t a)\n{\n";
     s << "    const idx_t n_out = " << g.P(p_nout) << ";\n";
     s << "    const idx_t nvec = " << g.P(p_nvec) << ";\n";
     s << "    const unsigned lane = threadIdx.x % TEAM;\n";
@@ -645,7 +671,7 @@ cg_kernel_t gen_reduce_col(einsummable_t const& e, int max_vec)
     g.k.kind = cg_kind::reduce_col;
     g.k.n_inns = L.NI;
     g.k.idx64 = !fits32(e);
-    g.k.entry = "es_kernel";
+    g.k.entry = entry_name(e, "redcol");
     castable_t const cast = e.castable.value();
     dtype_t const od = e.out_dtype();
 
@@ -680,7 +706,7 @@ cg_kernel_t gen_reduce_col(einsummable_t const& e, int max_vec)
     s << "#define V " << V << "\n";
     s << "__device__ __forceinline__ " << ACC << " comb(" << ACC << " x, " << ACC
       << " y) { return " << combine_expr(cast, od, "x", "y") << "; }\n";
-    s << "extern \"C\" __global__ __launch_bounds__(256) void es_kernel(args_t a)\n{\n";
+    s << "extern \"C\" __global__ __launch_bounds__(256) void " << g.k.entry << "(args_t a)\n{\n";
     s << "    const idx_t vid = ((idx_t)blockIdx.y * gridDim.x + blockIdx.x) * 256 + threadIdx.x;\n";
     s << "    if (vid >= " << g.P(p_nvec) << ") return;\n";
     s << "    idx_t rem = vid;\n";

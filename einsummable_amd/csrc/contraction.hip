@@ -109,6 +109,7 @@ struct traits_t<_Float16> {
     {
         return (i / 4) * 8 + (lane / 32) * 4 + (i % 4);
     }
+    static constexpr bool QUAD = true;  // registers 4q..4q+3 hold four consecutive rows
 };
 
 template <>
@@ -133,6 +134,7 @@ struct traits_t<float> {
     {
         return (i / 4) * 8 + (lane / 32) * 4 + (i % 4);
     }
+    static constexpr bool QUAD = true;  // registers 4q..4q+3 hold four consecutive rows
 };
 
 template <>
@@ -153,7 +155,10 @@ struct traits_t<double> {
             acc = __builtin_amdgcn_mfma_f64_16x16x4f64(r[j], c[j], acc, 0, 0, 0);
         }
     }
-    __device__ static __forceinline__ int acc_row(int i, int lane) { return (lane / 16) * 4 + i; }
+    // v_mfma_f64_16x16x4_f64 interleaves rows across registers: register i of lane l holds
+    // row 4 * i + l / 16, so a lane's four values are four rows apart
+    __device__ static __forceinline__ int acc_row(int i, int lane) { return 4 * i + lane / 16; }
+    static constexpr bool QUAD = false;
 };
 
 constexpr int ROW_BYTES = 128;  // bytes of k per tile row per stage
@@ -423,8 +428,8 @@ __global__ __launch_bounds__(256) void gemm_kernel(gemm_args_t a)
             uint32_t nb = tn * BN + wn * WN + j * MI;
 #pragma unroll
             for (int e0 = 0; e0 < tr::NACC; e0 += 4) {
-                uint32_t n = nb + uint32_t(tr::acc_row(e0, lane));
-                if (a.c_mode == 0) {
+                if (tr::QUAD && a.c_mode == 0) {
+                    uint32_t n = nb + uint32_t(tr::acc_row(e0, lane));
                     if (n < a.N) {
                         int64_t no_b, no_c;
                         group_offsets(a.gn, n, no_b, no_c);
@@ -438,9 +443,10 @@ __global__ __launch_bounds__(256) void gemm_kernel(gemm_args_t a)
                 } else {
 #pragma unroll
                     for (int t = 0; t != 4; ++t) {
-                        if (n + t < a.N) {
+                        uint32_t n = nb + uint32_t(tr::acc_row(e0 + t, lane));
+                        if (n < a.N) {
                             int64_t no_b, no_c;
-                            group_offsets(a.gn, n + t, no_b, no_c);
+                            group_offsets(a.gn, n, no_b, no_c);
                             C[mo_c + no_c] = T(acc[i][j][e0 + t]);
                         }
                     }
