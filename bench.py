@@ -38,7 +38,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="all",
-                    choices=["c2", "c1", "c3", "c4", "llama", "all"])
+                    choices=["c2", "c1", "c3", "c4", "llama", "copy", "all"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     return ap.parse_args()
 
@@ -282,6 +282,33 @@ def run_llama_contractions(km, steps, warmup):
             for name, e, shapes, flops in cases]
 
 
+def run_copy(km, steps, warmup):
+    """A plain copy of known size (1-D touch without castable, 512 MiB in, 512 MiB out): the
+    yardstick the FETCH_SIZE / WRITE_SIZE counters are scaled by."""
+    import torch
+
+    import einsummable_amd as ea
+
+    n = 1 << 28
+    x = torch.randn(n, device="cuda", dtype=torch.float16)
+    y = torch.empty_like(x)
+    t = ea.Touch([(n, n, 0, 0, n)], None, ea.F16)
+    stream = torch.cuda.current_stream().cuda_stream
+    call = lambda: km.touch(t, stream, y.data_ptr(), x.data_ptr())
+    for _ in range(warmup):
+        call()
+    torch.cuda.synchronize()
+    tm = Timed()
+    for _ in range(steps):
+        tm.record(call)
+    torch.cuda.synchronize()
+    nbytes = 2 * n * 2
+    ms = tm.mean_ms()
+    return {"node": "copy 2^28 f16", "bytes": nbytes, "ms": round(ms, 5),
+            "GBps": round(nbytes / ms / 1e6, 1),
+            "hbm_frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -295,6 +322,10 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.init()
     km = ea.KernelManager(0)
+
+    if args.workload == "copy":
+        print(json.dumps(run_copy(km, args.steps, args.warmup)))
+        return
 
     c2 = run_c2(km, args.steps, args.warmup)
     ms_per_step = c2["wall_s"] / args.steps * 1e3

@@ -19,4 +19,6 @@ from .km import (  # noqa: F401
     codegen_source,
     lib_path,
     load_library,
+    merge_adjacent_dims,
+    scalarop_roundtrip,
 )

@@ -267,4 +267,50 @@ int es_km_codegen_source(const uint64_t* join_shape, int join_rank, const int* i
         return ES_KM_OK;
     });
 }
+
+int es_km_scalarop_roundtrip(const char* text, char* out, size_t cap, int* out_dtype,
+                             int* n_inputs)
+{
+    return guarded(nullptr, [&]() -> int {
+        if (!text) throw es::ir_error("null text");
+        es::scalarop_t op = es::scalarop_t::parse(text);
+        std::string    s = op.str();
+        if (out && cap) {
+            if (s.size() + 1 > cap) throw es::ir_error("roundtrip: buffer too small");
+            std::memcpy(out, s.c_str(), s.size() + 1);
+        }
+        if (out_dtype) *out_dtype = int(op.out_dtype());
+        if (n_inputs) *n_inputs = op.num_inputs();
+        return ES_KM_OK;
+    });
+}
+
+int es_km_merge_adjacent_dims(const uint64_t* join_shape, int join_rank, const int* inns_flat,
+                              const int* inns_offsets, int n_inns, int out_rank,
+                              const char* join_text, char castable, uint64_t* new_join_shape,
+                              int* new_inns_flat, int* new_inns_offsets, int* new_out_rank,
+                              char* str_out, size_t str_cap)
+{
+    return guarded(nullptr, [&]() -> int {
+        check_descriptor(join_shape, join_rank, inns_flat, inns_offsets, n_inns, out_rank,
+                         join_text);
+        es::einsummable_t e = make_einsummable(join_shape, join_rank, inns_flat, inns_offsets,
+                                               n_inns, out_rank, join_text, castable)
+                                  .merge_adjacent_dims();
+        int pos = 0;
+        for (size_t i = 0; i != e.join_shape.size(); ++i) new_join_shape[i] = e.join_shape[i];
+        for (size_t k = 0; k != e.inns.size(); ++k) {
+            new_inns_offsets[k] = pos;
+            for (int m : e.inns[k]) new_inns_flat[pos++] = m;
+        }
+        new_inns_offsets[e.inns.size()] = pos;
+        *new_out_rank = e.out_rank;
+        if (str_out && str_cap) {
+            std::string s = e.str();
+            std::strncpy(str_out, s.c_str(), str_cap - 1);
+            str_out[str_cap - 1] = 0;
+        }
+        return int(e.join_shape.size());
+    });
+}
 }

@@ -21,6 +21,8 @@ EXPORTS = [
     "es_km_fill_constant",
     "es_km_fill_lowertri",
     "es_km_codegen_source",
+    "es_km_scalarop_roundtrip",
+    "es_km_merge_adjacent_dims",
 ]
 
 
@@ -104,6 +106,11 @@ def load_library():
         ctypes.c_void_p,
     ]
     lib.es_km_codegen_source.argtypes = desc + [ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t]
+    lib.es_km_scalarop_roundtrip.argtypes = [ctypes.c_char_p, ctypes.c_void_p, ctypes.c_size_t,
+                                             ctypes.c_void_p, ctypes.c_void_p]
+    lib.es_km_merge_adjacent_dims.argtypes = desc + [ctypes.c_void_p, ctypes.c_void_p,
+                                                     ctypes.c_void_p, ctypes.c_void_p,
+                                                     ctypes.c_void_p, ctypes.c_size_t]
     _lib = lib
     return lib
 
@@ -192,6 +199,34 @@ def codegen_source(e, compile=False):
     if rc != OK:
         raise KmError(rc, lib.es_km_last_error(None).decode())
     return buf.value.decode()
+
+
+def scalarop_roundtrip(text):
+    """(printed text, out dtype, number of holes) from the library's own scalarop parser."""
+    lib = load_library()
+    buf = ctypes.create_string_buffer(8192)
+    od, n = ctypes.c_int(), ctypes.c_int()
+    rc = lib.es_km_scalarop_roundtrip(text.encode(), ctypes.cast(buf, ctypes.c_void_p), 8192,
+                                      ctypes.byref(od), ctypes.byref(n))
+    if rc != OK:
+        raise KmError(rc, lib.es_km_last_error(None).decode())
+    return buf.value.decode(), od.value, n.value
+
+
+def merge_adjacent_dims(e):
+    """(join_shape, inns, out_rank, str) of e.merge_adjacent_dims() from the library."""
+    lib = load_library()
+    n_modes = sum(len(i) for i in e.inns)
+    js = (ctypes.c_uint64 * len(e.join_shape))()
+    flat = (ctypes.c_int * max(n_modes, 1))()
+    offs = (ctypes.c_int * (len(e.inns) + 1))()
+    orank = ctypes.c_int()
+    buf = ctypes.create_string_buffer(256)
+    rc = lib.es_km_merge_adjacent_dims(*e._args, js, flat, offs, ctypes.byref(orank), buf, 256)
+    if rc < 0:
+        raise KmError(rc, lib.es_km_last_error(None).decode())
+    inns = [[flat[i] for i in range(offs[k], offs[k + 1])] for k in range(len(e.inns))]
+    return [int(js[i]) for i in range(rc)], inns, orank.value, buf.value.decode()
 
 
 class KernelManager:

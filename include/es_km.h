@@ -114,6 +114,21 @@ int es_km_codegen_source(const uint64_t* join_shape, int join_rank, const int* i
                          const int* inns_offsets, int n_inns, int out_rank, const char* join_text,
                          char castable, int compile, char* out, size_t cap);
 
+/* Host-logic diagnostics without a device (used by the CPU test-suite).
+ * es_km_scalarop_roundtrip: parse a scalarop text with the library's parser and print it
+ *   back (operator>> / operator<< of scalar_ns::node_t, scalarop.cc:2881-3060), reporting
+ *   the output dtype and the number of holes.
+ * es_km_merge_adjacent_dims: einsummable_t::merge_adjacent_dims (einsummable.cc:166-218)
+ *   followed by str() (einsummable.cc:483-501); returns the new join rank (>= 1) or a
+ *   negative error.  Output arrays must hold join_rank / the input's mode count entries. */
+int es_km_scalarop_roundtrip(const char* text, char* out, size_t cap, int* out_dtype,
+                             int* n_inputs);
+int es_km_merge_adjacent_dims(const uint64_t* join_shape, int join_rank, const int* inns_flat,
+                              const int* inns_offsets, int n_inns, int out_rank,
+                              const char* join_text, char castable, uint64_t* new_join_shape,
+                              int* new_inns_flat, int* new_inns_offsets, int* new_out_rank,
+                              char* str_out, size_t str_cap);
+
 #ifdef __cplusplus
 }
 #endif
