@@ -48,7 +48,7 @@ def build(verbose=False):
         for _, err in results:
             if err.strip():
                 print(err, file=sys.stderr)
-    cmd = ["hipcc", "-shared", "-fPIC", "-o", LIB] + objs + ["-lhiprtc"]
+    cmd = ["hipcc", "-shared", "-fPIC", "-Wl,-soname,libes_km.so", "-o", LIB] + objs + ["-lhiprtc"]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n" + r.stderr)

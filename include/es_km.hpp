@@ -1,0 +1,213 @@
+// es_km.hpp -- header-only C++ face of the C ABI in es_km.h with the member names, argument
+// meaning and error behaviour of the reference's kernel_manager_t
+// (src/engine/gpu/gpu_kernel_manager.h:274-321):
+//
+//   optional<workspace_info_t> build(einsummable_t const&)   nullopt when unsupported
+//   workspace_info_t workspace_size(einsummable_t const&)    throws if not built
+//   operator()(einsummable_t, stream, out, inns, workspace)  throws std::runtime_error on a
+//                                                            missing build, a wrong input
+//                                                            count or a short workspace
+//   operator()(touch_t, stream, out, inn)
+//   constant_fill / lowerTri_fill
+//
+// The descriptor structs carry the same fields as the reference's einsummable_t
+// (src/einsummable/einsummable.h:8-20), touch_t (touch.h:8-29) and fill_t (fill.h:11-30); the
+// join travels as the text `operator<<(ostream&, scalarop_t)` writes.  Inside the reference
+// tree the adapter is three lines per call: see INTEGRATION.md.
+#pragma once
+#include "es_km.h"
+
+#include <complex>
+#include <cstring>
+#include <optional>
+#include <stdexcept>
+#include <string>
+#include <tuple>
+#include <vector>
+
+namespace eskm
+{
+
+enum class dtype_t { f16 = ES_KM_F16, f32 = ES_KM_F32, f64 = ES_KM_F64, c64 = ES_KM_C64 };
+enum class castable_t { add, mul, min, max };
+
+inline char castable_char(std::optional<castable_t> const& c)
+{
+    if (!c) return 0;
+    switch (c.value()) {
+        case castable_t::add:
+            return '+';
+        case castable_t::mul:
+            return 'x';
+        case castable_t::min:
+            return 'v';
+        case castable_t::max:
+            return '^';
+    }
+    return 0;
+}
+
+// scalar_t (src/einsummable/scalarop.h:24-75): a dtype and eight raw bytes
+struct scalar_t {
+    dtype_t dtype = dtype_t::f32;
+    uint8_t data[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+
+    scalar_t() = default;
+    explicit scalar_t(float v) : dtype(dtype_t::f32) { std::memcpy(data, &v, 4); }
+    explicit scalar_t(double v) : dtype(dtype_t::f64) { std::memcpy(data, &v, 8); }
+    explicit scalar_t(std::complex<float> v) : dtype(dtype_t::c64) { std::memcpy(data, &v, 8); }
+    static scalar_t from_f16_bits(uint16_t bits)
+    {
+        scalar_t s;
+        s.dtype = dtype_t::f16;
+        std::memcpy(s.data, &bits, 2);
+        return s;
+    }
+    uint64_t bits() const
+    {
+        uint64_t b;
+        std::memcpy(&b, data, 8);
+        return b;
+    }
+};
+
+struct einsummable_t {
+    std::vector<uint64_t>         join_shape;
+    std::vector<std::vector<int>> inns;
+    int                           out_rank;
+    std::string                   join;  // scalarop text
+    std::optional<castable_t>     castable;
+
+    // from_matmul (src/einsummable/einsummable.cc:307-323): ij,jk->ik
+    static einsummable_t from_matmul(uint64_t di, uint64_t dj, uint64_t dk, dtype_t d)
+    {
+        static const char* names[] = {"f16", "f32", "f64", "c64"};
+        std::string        n = names[int(d)];
+        return einsummable_t{{di, dk, dj},
+                             {{0, 2}, {2, 1}},
+                             2,
+                             "*[hole|" + n + "@0,hole|" + n + "@1]",
+                             castable_t::add};
+    }
+};
+
+struct touchdim_t {
+    uint64_t d_inn, d_out, offset_inn, offset_out, size;
+};
+
+struct touch_t {
+    std::vector<touchdim_t>   selection;
+    std::optional<castable_t> castable;
+    dtype_t                   dtype;
+};
+
+struct fill_t {
+    struct constant_t {
+        scalar_t              value;
+        std::vector<uint64_t> shape;
+    };
+    struct lowertri_t {
+        scalar_t lower, upper;
+        uint64_t nrow, ncol;
+        int64_t  start;
+    };
+};
+
+struct workspace_info_t {
+    workspace_info_t() {}
+    workspace_info_t(uint64_t sz) : workspace_size(sz) {}
+    std::optional<uint64_t> workspace_size;
+    uint64_t const&         value() const { return workspace_size.value(); }
+    bool                    known() const { return bool(workspace_size); }
+};
+
+class kernel_manager_t
+{
+public:
+    explicit kernel_manager_t(int device = 0) : h_(es_km_create(device))
+    {
+        if (!h_) throw std::runtime_error(std::string("kernel_manager_t: ") + es_km_last_error(nullptr));
+    }
+    ~kernel_manager_t() { es_km_destroy(h_); }
+    kernel_manager_t(kernel_manager_t const&) = delete;
+    kernel_manager_t& operator=(kernel_manager_t const&) = delete;
+
+    std::optional<workspace_info_t> build(einsummable_t const& e)
+    {
+        flat_t   f(e);
+        uint64_t ws = 0;
+        int rc = es_km_build(h_, e.join_shape.data(), int(e.join_shape.size()), f.flat.data(),
+                             f.offs.data(), int(e.inns.size()), e.out_rank, e.join.c_str(),
+                             castable_char(e.castable), &ws);
+        if (rc == ES_KM_UNSUPPORTED) return std::nullopt;
+        check(rc);
+        return workspace_info_t(ws);
+    }
+
+    workspace_info_t workspace_size(einsummable_t const& e) const
+    {
+        flat_t   f(e);
+        uint64_t ws = 0;
+        check(es_km_workspace_size(h_, e.join_shape.data(), int(e.join_shape.size()),
+                                   f.flat.data(), f.offs.data(), int(e.inns.size()), e.out_rank,
+                                   e.join.c_str(), castable_char(e.castable), &ws));
+        return workspace_info_t(ws);
+    }
+
+    void operator()(touch_t const& touch, void* stream, void* out, void const* inn) const
+    {
+        static_assert(sizeof(touchdim_t) == 5 * sizeof(uint64_t), "touchdim_t must be packed");
+        check(es_km_touch(h_, reinterpret_cast<uint64_t const*>(touch.selection.data()),
+                          int(touch.selection.size()), castable_char(touch.castable),
+                          int(touch.dtype), stream, out, inn));
+    }
+
+    void operator()(einsummable_t const& e, void* stream, void* out,
+                    std::vector<void const*>                    inns,
+                    std::optional<std::tuple<void*, uint64_t>> workspace = std::nullopt) const
+    {
+        flat_t f(e);
+        check(es_km_execute(h_, e.join_shape.data(), int(e.join_shape.size()), f.flat.data(),
+                            f.offs.data(), int(e.inns.size()), e.out_rank, e.join.c_str(),
+                            castable_char(e.castable), stream, out, inns.data(), int(inns.size()),
+                            workspace ? std::get<0>(workspace.value()) : nullptr,
+                            workspace ? std::get<1>(workspace.value()) : 0));
+    }
+
+    void lowerTri_fill(fill_t::lowertri_t const& l, void* stream, void* out) const
+    {
+        check(es_km_fill_lowertri(h_, int(l.lower.dtype), l.lower.bits(), l.upper.bits(), l.nrow,
+                                  l.ncol, l.start, stream, out));
+    }
+
+    void constant_fill(fill_t::constant_t const& c, void* stream, void* out) const
+    {
+        uint64_t n = 1;
+        for (uint64_t d : c.shape) n *= d;
+        check(es_km_fill_constant(h_, int(c.value.dtype), c.value.bits(), n, stream, out));
+    }
+
+private:
+    struct flat_t {
+        std::vector<int> flat, offs;
+        explicit flat_t(einsummable_t const& e)
+        {
+            offs.push_back(0);
+            for (auto const& inn : e.inns) {
+                flat.insert(flat.end(), inn.begin(), inn.end());
+                offs.push_back(int(flat.size()));
+            }
+        }
+    };
+
+    void check(int rc) const
+    {
+        if (rc != ES_KM_OK) {
+            throw std::runtime_error(std::string("kernel_manager_t: ") + es_km_last_error(h_));
+        }
+    }
+
+    es_km_t* h_;
+};
+
+}  // namespace eskm

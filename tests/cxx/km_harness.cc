@@ -1,0 +1,194 @@
+// C++ harness over es_km.hpp in the style of the reference's kernel-manager experiments
+// (exps/gpuexec_kernelmanager.cc:18-160, exps/cpuexec_kernels.cc:9-86): build an einsummable,
+// fill inputs from a seeded std::mt19937 the way dbuffer_t::random does
+// (src/einsummable/dbuffer.cc:198-229), run it through kernel_manager_t on device buffers,
+// and compare with the CPU oracle.  Exits non-zero on the first mismatch.
+#include "es_km.hpp"
+#include "es_oracle.h"
+
+#include <hip/hip_runtime_api.h>
+
+#include <cmath>
+#include <cstdio>
+#include <random>
+
+using namespace eskm;
+
+#define HIP_OK(x)                                                                      \
+    do {                                                                               \
+        hipError_t e_ = (x);                                                           \
+        if (e_ != hipSuccess) {                                                        \
+            std::printf("FAIL hip: %s at %s:%d\n", hipGetErrorString(e_), __FILE__, __LINE__); \
+            std::exit(2);                                                              \
+        }                                                                              \
+    } while (0)
+
+struct device_buffer_t {
+    void*  ptr = nullptr;
+    size_t bytes;
+    explicit device_buffer_t(size_t n) : bytes(n) { HIP_OK(hipMalloc(&ptr, n ? n : 1)); }
+    ~device_buffer_t() { (void)hipFree(ptr); }
+    void upload(void const* src) { HIP_OK(hipMemcpy(ptr, src, bytes, hipMemcpyHostToDevice)); }
+    void download(void* dst) { HIP_OK(hipMemcpy(dst, ptr, bytes, hipMemcpyDeviceToHost)); }
+};
+
+static std::vector<float> random_f32(std::mt19937& gen, size_t n, float lo, float hi)
+{
+    std::uniform_real_distribution<float> dist(lo, hi);
+    std::vector<float>                    v(n);
+    for (auto& x : v) x = dist(gen);
+    return v;
+}
+
+static std::vector<uint16_t> random_f16(std::mt19937& gen, size_t n, float lo, float hi)
+{
+    std::uniform_real_distribution<float> dist(lo, hi);
+    std::vector<uint16_t>                 v(n);
+    for (auto& x : v) x = es_oracle_f32_to_f16(dist(gen));
+    return v;
+}
+
+static void expect(bool ok, const char* what)
+{
+    if (!ok) {
+        std::printf("FAIL %s\n", what);
+        std::exit(1);
+    }
+    std::printf("ok   %s\n", what);
+}
+
+static std::vector<int> flatten(einsummable_t const& e, std::vector<int>& offs)
+{
+    std::vector<int> flat;
+    offs.assign(1, 0);
+    for (auto const& inn : e.inns) {
+        flat.insert(flat.end(), inn.begin(), inn.end());
+        offs.push_back(int(flat.size()));
+    }
+    return flat;
+}
+
+static void oracle_run(einsummable_t const& e, void* out, std::vector<void const*> inns)
+{
+    std::vector<int> offs;
+    std::vector<int> flat = flatten(e, offs);
+    int rc = es_oracle_einsummable(e.join_shape.data(), int(e.join_shape.size()), flat.data(),
+                                   offs.data(), int(e.inns.size()), e.out_rank, e.join.c_str(),
+                                   castable_char(e.castable), ES_O_WIDE, out, inns.data());
+    if (rc) {
+        std::printf("FAIL oracle: %s\n", es_oracle_last_error());
+        std::exit(1);
+    }
+}
+
+int main()
+{
+    HIP_OK(hipSetDevice(0));
+    hipStream_t stream;
+    HIP_OK(hipStreamCreate(&stream));
+    std::mt19937     gen(0);
+    kernel_manager_t km(0);
+
+    {  // test_mm: f32 matmul through from_matmul (exps/cpuexec_kernels.cc:9-33)
+        uint64_t      ni = 200, nj = 136, nk = 72;
+        einsummable_t e = einsummable_t::from_matmul(ni, nj, nk, dtype_t::f32);
+        auto          lhs = random_f32(gen, ni * nj, -1, 1), rhs = random_f32(gen, nj * nk, -1, 1);
+        std::vector<float> ref(ni * nk), got(ni * nk);
+        oracle_run(e, ref.data(), {lhs.data(), rhs.data()});
+        auto ws = km.build(e);
+        expect(ws.has_value() && km.workspace_size(e).value() == ws.value().value(), "build matmul");
+        device_buffer_t dl(lhs.size() * 4), dr(rhs.size() * 4), dout(got.size() * 4),
+            dws(ws.value().value());
+        dl.upload(lhs.data());
+        dr.upload(rhs.data());
+        km(e, stream, dout.ptr, {dl.ptr, dr.ptr}, std::make_tuple(dws.ptr, ws.value().value()));
+        HIP_OK(hipStreamSynchronize(stream));
+        dout.download(got.data());
+        double worst = 0;
+        for (size_t i = 0; i != got.size(); ++i) worst = std::max(worst, std::fabs(double(got[i]) - ref[i]));
+        expect(worst <= 1e-4 * 8.0, "matmul f32 200x136x72 within 1e-4 of its magnitude");
+    }
+
+    {  // silu on f16 (exps/gpuexec_kernelmanager.cc, llama/modules.cc:416)
+        uint64_t      n = 10000;
+        einsummable_t e{{n}, {{0}}, 1,
+                        "*[hole|f16@0,power{-1}[+[constant{f16|1},exp[*[constant{f16|-1},hole|f16@0]]]]]",
+                        std::nullopt};
+        auto          x = random_f16(gen, n, -4, 4);
+        std::vector<uint16_t> ref(n), got(n);
+        oracle_run(e, ref.data(), {x.data()});
+        expect(km.build(e).has_value(), "build silu");
+        device_buffer_t dx(n * 2), dout(n * 2);
+        dx.upload(x.data());
+        km(e, stream, dout.ptr, {dx.ptr});
+        HIP_OK(hipStreamSynchronize(stream));
+        dout.download(got.data());
+        double worst = 0;
+        for (size_t i = 0; i != n; ++i) {
+            double a = es_oracle_f16_to_f32(got[i]), b = es_oracle_f16_to_f32(ref[i]);
+            worst = std::max(worst, std::fabs(a - b) / std::max(std::fabs(b), 1.0));
+        }
+        expect(worst <= 1e-2, "silu f16 within 1e-2");
+    }
+
+    {  // touch with castable add: exact (exps/cpuexec_touch.cc:85-114)
+        touch_t t{{{16, 64, 0, 8, 16}, {16, 64, 0, 24, 16}}, castable_t::add, dtype_t::f32};
+        auto    inn = random_f32(gen, 256, -1, 1), out = random_f32(gen, 4096, -1, 1);
+        std::vector<float> ref = out, got(4096);
+        es_oracle_touch(reinterpret_cast<uint64_t const*>(t.selection.data()), 2, '+', ES_O_F32,
+                        ref.data(), inn.data());
+        device_buffer_t di(256 * 4), dout(4096 * 4);
+        di.upload(inn.data());
+        dout.upload(out.data());
+        km(t, stream, dout.ptr, di.ptr);
+        HIP_OK(hipStreamSynchronize(stream));
+        dout.download(got.data());
+        expect(std::memcmp(got.data(), ref.data(), 4096 * 4) == 0, "touch add bit exact");
+    }
+
+    {  // fills
+        fill_t::lowertri_t l{scalar_t(0.0f), scalar_t(-INFINITY), 40, 56, 3};
+        std::vector<float> ref(40 * 56), got(40 * 56);
+        es_oracle_fill_lowertri(ES_O_F32, l.lower.bits(), l.upper.bits(), 40, 56, 3, ref.data());
+        device_buffer_t d(ref.size() * 4);
+        km.lowerTri_fill(l, stream, d.ptr);
+        HIP_OK(hipStreamSynchronize(stream));
+        d.download(got.data());
+        expect(std::memcmp(got.data(), ref.data(), ref.size() * 4) == 0, "lowerTri_fill bit exact");
+        fill_t::constant_t c{scalar_t(2.5), {7, 11}};
+        std::vector<double> gc(77);
+        device_buffer_t     dc(77 * 8);
+        km.constant_fill(c, stream, dc.ptr);
+        HIP_OK(hipStreamSynchronize(stream));
+        dc.download(gc.data());
+        bool all = true;
+        for (double v : gc) all = all && v == 2.5;
+        expect(all, "constant_fill");
+    }
+
+    {  // error behaviour (gpu_kernel_manager.cc:957, 1103-1107, 1260)
+        einsummable_t unbuilt{{33}, {{0}}, 1, "exp[hole|f32@0]", std::nullopt};
+        device_buffer_t d(33 * 4);
+        bool threw = false;
+        try {
+            km(unbuilt, stream, d.ptr, {d.ptr});
+        } catch (std::runtime_error const&) {
+            threw = true;
+        }
+        expect(threw, "executing an un-built einsummable throws");
+        einsummable_t with_var{{33}, {{0}}, 1, "*[variable{lr|f32},hole|f32@0]", std::nullopt};
+        expect(!km.build(with_var).has_value(), "unsupported einsummable builds to nullopt");
+        km.build(unbuilt);
+        threw = false;
+        try {
+            km(unbuilt, stream, d.ptr, {d.ptr, d.ptr});
+        } catch (std::runtime_error const&) {
+            threw = true;
+        }
+        expect(threw, "wrong input count throws");
+    }
+
+    HIP_OK(hipStreamDestroy(stream));
+    std::printf("PASS\n");
+    return 0;
+}
