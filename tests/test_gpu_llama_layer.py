@@ -1,0 +1,142 @@
+"""The LLaMA decoder layer as a list of apply / touch / fill nodes, run end to end on the new
+kernels.  At a reduced size the same node list is replayed through the CPU oracle (each node
+computed in higher precision and rounded to its dtype, like the kernels do); at the full
+LLaMA-7B size the result is checked against a plain fp32 torch restatement of the layer and
+against properties the mathematics fixes (softmax rows sum to one, causal mask)."""
+import math
+
+import numpy as np
+import pytest
+
+import einsummable_amd as ea
+import oracle
+from einsummable_amd.llama_layer import DeviceRunner, LayerGraph, freqs_cis_table
+from helpers import NP, assert_close, normal, rng
+
+pytestmark = pytest.mark.gpu
+
+
+def make_inputs(g, seed):
+    r = rng(seed)
+    vals = {}
+    for name, (dt, shape) in g.inputs.items():
+        n = int(np.prod(shape))
+        if name == "x":
+            vals[name] = normal(r, n, np.float16, 1.0)
+        elif name == "full_freqs_cis":
+            vals[name] = freqs_cis_table(shape[0], shape[1]).reshape(-1).view(np.complex64)
+        elif name.endswith("norm.weight"):
+            vals[name] = (1.0 + normal(r, n, np.float32, 0.02)).astype(np.float16)
+        else:
+            vals[name] = normal(r, n, np.float16, 0.02)
+    return vals
+
+
+def oracle_run(g, vals):
+    """Replay the node list on the CPU oracle over byte buffers."""
+    mem = {k: np.zeros(nb, np.uint8) for k, nb in g.buffers.items()}
+    for k, v in vals.items():
+        mem[k][:] = np.ascontiguousarray(v).view(np.uint8).reshape(-1)
+    for n in g.nodes:
+        if n["kind"] == "einsummable":
+            e = n["e"]
+            od, dts = oracle.scalarop_info(e.join)
+            ins = [mem[b].view(NP[dt]) for b, dt in zip(n["inns"], dts)]
+            out = oracle.einsummable(e.join_shape, e.inns, e.out_rank, e.join, e.castable, ins,
+                                     oracle.WIDE)
+            mem[n["out"]][:] = out.view(np.uint8)
+        elif n["kind"] == "touch":
+            t = n["t"]
+            out = mem[n["out"]].view(NP[t.dtype])
+            oracle.touch(t.selection, t.castable, out, mem[n["inn"]].view(NP[t.dtype]))
+        else:
+            m = oracle.fill_lowertri(NP[n["dtype"]], n["lower"], n["upper"], n["nrow"], n["ncol"],
+                                     n["start"])
+            mem[n["out"]][:] = m.view(np.uint8).reshape(-1)
+    return mem
+
+
+def test_reduced_layer_matches_oracle_node_by_node_chain(km):
+    import torch
+
+    g = LayerGraph(dim=256, n_heads=4, ffn=688, seq=128)
+    vals = make_inputs(g, 0)
+    run = DeviceRunner(km, g)
+    for k, v in vals.items():
+        run.set_input(k, v)
+    run.run()
+    torch.cuda.synchronize()
+    want = oracle_run(g, vals)
+    # data movement and the mask are exact
+    assert np.array_equal(run.get("mask", np.uint8), want["mask"])
+    assert np.array_equal(run.get("freqs_cis", np.uint8), want["freqs_cis"])
+    # intermediate and final tensors within the fp16 / fp32 contract
+    for name, dt in [("an.weight", ea.F16), ("rq.to_f16", ea.F16), ("scores.f", ea.F16),
+                     ("sm.div", ea.F32), ("values.f", ea.F16), ("residual1", ea.F16),
+                     ("gate", ea.F16), ("residual2", ea.F16)]:
+        got = run.get(name, NP[dt])
+        ref = want[name].view(NP[dt])
+        if name == "scores.f":
+            pass
+        assert_close(got, ref, dt, what="layer tensor " + name)
+    # softmax rows sum to one
+    p = run.get("sm.div", np.float32).reshape(-1, g.seq).astype(np.float64)
+    np.testing.assert_allclose(p.sum(axis=1), 1.0, rtol=1e-5)
+
+
+def torch_layer_fp32(g, vals):
+    import torch
+
+    s, d, h, hd = g.seq, g.dim, g.n_heads, g.hd
+    T = lambda name, shape: torch.from_numpy(vals[name].astype(np.float32)).cuda().reshape(shape)
+    x = T("x", (s, d))
+
+    def rms(v, w):
+        return (v * torch.rsqrt((v * v).mean(-1, keepdim=True) + g.eps)) * w
+
+    def rot(v):
+        fc = torch.from_numpy(freqs_cis_table(2 * s, hd // 2)[:s]).cuda()
+        fc = torch.view_as_complex(fc.contiguous())
+        vc = torch.view_as_complex(v.reshape(s, h, hd // 2, 2).contiguous())
+        return torch.view_as_real(vc * fc[:, None, :]).reshape(s, h, hd)
+
+    xa = rms(x, T("attention_norm.weight", (d,)))
+    q = rot(xa @ T("wq", (d, d)).T).transpose(0, 1)
+    k = rot(xa @ T("wk", (d, d)).T).transpose(0, 1)
+    v = (xa @ T("wv", (d, d)).T).reshape(s, h, hd).transpose(0, 1)
+    sc = q @ k.transpose(1, 2)      # no 1/sqrt(hd): the reference drops it
+    sc = sc + torch.triu(torch.full((s, s), -math.inf, device="cuda"), diagonal=1)
+    p = torch.softmax(sc, dim=-1)
+    at = (p @ v)                    # [h, s, hd]
+    wo = T("wo", (d, h, hd))
+    ao = torch.einsum("dbe,cde->bc", at, wo)
+    h1 = x + ao
+    xf = rms(h1, T("ffn_norm.weight", (d,)))
+    a1 = xf @ T("w1", (g.ffn, d)).T
+    a3 = xf @ T("w3", (g.ffn, d)).T
+    y = (torch.nn.functional.silu(a1) * a3) @ T("w2", (d, g.ffn)).T
+    return (h1 + y).cpu().numpy().reshape(-1)
+
+
+def test_full_llama7b_layer_end_to_end(km):
+    import torch
+
+    torch.backends.cuda.matmul.allow_tf32 = False
+    g = LayerGraph()     # dim 4096, 32 heads of 128, ffn 11008, seq 2048
+    assert abs(g.contraction_flops() / 1e12 - 0.898) < 0.01
+    vals = make_inputs(g, 1)
+    run = DeviceRunner(km, g)
+    for k, v in vals.items():
+        run.set_input(k, v)
+    run.run()
+    torch.cuda.synchronize()
+    got = run.get("residual2", np.float16)
+    assert np.isfinite(got.astype(np.float32)).all()
+    p = run.get("sm.div", np.float32).reshape(-1, g.seq)
+    rows = p[:: 997].astype(np.float64)
+    np.testing.assert_allclose(rows.sum(axis=1), 1.0, rtol=1e-5)
+    pm = p.reshape(g.n_heads, g.seq, g.seq)[3]
+    assert np.all(np.triu(pm, 1) == 0.0)            # causal: nothing above the diagonal
+    want = torch_layer_fp32(g, vals)
+    # every tensor between nodes is rounded to fp16 here and kept in fp32 there
+    assert_close(got, want, ea.F16, what="LLaMA-7B layer vs fp32 restatement")
