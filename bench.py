@@ -28,6 +28,11 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E
 PEAK_TFLOPS = {"f16": 2500.0, "f32": 157.3, "f64": 78.6}
 
+# HBM bytes per launch of the dominant kernel (C2 node (i)) from two rocprofv3 --pmc runs:
+# FETCH_SIZE 131087.2 KiB x 1.9994 + WRITE_SIZE 131072.0 KiB x 1.0000, the factors being what
+# the same counters read for a 512 MiB copy of known size.
+DOMINANT_KERNEL_TRAFFIC_BYTES = 402609175
+
 RELU_MUL = "*[ite_>=[constant{f16|0},hole|f16@0,constant{f16|0},hole|f16@0],hole|f16@1]"
 EXP_SUB = "exp[+[hole|f16@0,*[constant{f16|-1},hole|f16@1]]]"
 
@@ -38,7 +43,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="all",
-                    choices=["c2", "c1", "c3", "c4", "llama", "copy", "all"])
+                    choices=["c2", "c1", "c3", "c4", "c5", "llama", "copy", "all"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     return ap.parse_args()
 
@@ -282,6 +287,50 @@ def run_llama_contractions(km, steps, warmup):
             for name, e, shapes, flops in cases]
 
 
+def run_c5(km, steps, warmup):
+    """One LLaMA-7B decoder layer (dim 4096, 32 heads of 128, SwiGLU 11008, RMSNorm, rotary,
+    batch 1, seq 2048, fp16, weights N(0, 0.02)) as its list of apply / touch / fill nodes,
+    every node on the kernel manager, in order on one stream."""
+    import numpy as np
+    import torch
+
+    from einsummable_amd.llama_layer import DeviceRunner, LayerGraph, freqs_cis_table
+
+    g = LayerGraph()
+    run = DeviceRunner(km, g)
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    for name, (dt, shape) in g.inputs.items():
+        n = int(np.prod(shape))
+        if name == "full_freqs_cis":
+            run.set_input(name, freqs_cis_table(shape[0], shape[1]))
+            continue
+        sd = 1.0 if name == "x" else 0.02
+        t = torch.randn(n, device="cuda", dtype=torch.float32, generator=gen) * sd
+        if name.endswith("norm.weight"):
+            t = t + 1.0
+        run.mem[name].copy_(t.half().view(torch.uint8))
+    for _ in range(warmup):
+        run.run()
+    torch.cuda.synchronize()
+    timers = [Timed() for _ in g.nodes]
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        run.run(timers=timers)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) / steps * 1e3
+    rows = []
+    for n, t in zip(g.nodes, timers):
+        rows.append((n["label"], n["kind"], t.mean_ms(), n.get("flops", 0)))
+    gemm_ms = sum(ms for _, _, ms, fl in rows if fl)
+    top = sorted(rows, key=lambda r: -r[2])[:12]
+    return {"node": "c5 LLaMA-7B decoder layer, b=1 s=2048 f16", "layer_ms": round(wall_ms, 4),
+            "nodes": len(rows), "sum_node_ms": round(sum(r[2] for r in rows), 4),
+            "contraction_ms": round(gemm_ms, 4),
+            "contraction_TFLOPs": round(g.contraction_flops() / gemm_ms / 1e9, 1),
+            "other_ms": round(sum(r[2] for r in rows) - gemm_ms, 4),
+            "top_nodes": [{"label": l, "ms": round(ms, 4)} for l, _, ms, _ in top]}
+
+
 def run_copy(km, steps, warmup):
     """A plain copy of known size (1-D touch without castable, 512 MiB in, 512 MiB out): the
     yardstick the FETCH_SIZE / WRITE_SIZE counters are scaled by."""
@@ -333,7 +382,8 @@ def main():
     dom = max(c2["per_node"], key=lambda p: p["bytes"])
     roofline = {"bound": "hbm", "kernel": dom["node"] + " [" + dom["kernel"] + "]",
                 "achieved": dom["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                "frac": round(dom["GBps"] / HBM_PEAK_GBPS, 4), "traffic": None}
+                "frac": round(dom["GBps"] / HBM_PEAK_GBPS, 4),
+                "traffic": DOMINANT_KERNEL_TRAFFIC_BYTES}
     others = {"c2_nodes": c2["per_node"]}
     del c2
     torch.cuda.empty_cache()
@@ -343,6 +393,10 @@ def main():
         others["c3"] = run_c3(km, args.steps, args.warmup)
     if args.workload in ("c4", "all"):
         others["c4"] = run_c4(km, max(args.steps // 5, 3), max(args.warmup // 5, 1))
+    if args.workload in ("c5", "all"):
+        torch.cuda.empty_cache()
+        others["c5"] = run_c5(km, max(args.steps // 5, 3), max(args.warmup // 5, 1))
+        torch.cuda.empty_cache()
     if args.workload in ("llama", "all"):
         others["llama7b_contractions"] = run_llama_contractions(km, max(args.steps // 5, 3),
                                                                 max(args.warmup // 5, 1))

@@ -88,7 +88,8 @@ class LayerGraph:
         s = self.seq
         e = Einsummable.from_str("ij,kj->ik", dict(i=s, j=n_in, k=n_out),
                                  "*[hole|f16@0,hole|f16@1]", "+")
-        y = self.es(label, e, self.buf(label, F16, s * n_out), [x, w], flops=2 * s * n_in * n_out)
+        y = self.es(label, e, self.buf(label + ".mm", F16, s * n_out), [x, w],
+                    flops=2 * s * n_in * n_out)
         return self.formation(label, y, F16, s * n_out)
 
     def rotary(self, p, x, freqs):
@@ -159,7 +160,7 @@ class LayerGraph:
                      flops=2 * h * s * s * hd)
         at = self.formation("values", at, F16, s * d)
         e_o = Einsummable.from_str("adbe,cde->abc", dict(a=1, d=h, b=s, e=hd, c=d), mul, "+")
-        ao = self.es("wo", e_o, self.buf("wo", F16, s * d), [at, wo], flops=2 * s * d * d)
+        ao = self.es("wo", e_o, self.buf("wo.mm", F16, s * d), [at, wo], flops=2 * s * d * d)
         ao = self.formation("wo", ao, F16, s * d)
         add = "+[hole|f16@0,hole|f16@1]"
         h1 = self.es("residual1", Einsummable([s * d], [[0], [0]], 1, add),
