@@ -23,6 +23,9 @@ SOURCES = [
     "touch.hip",
     "transpose.hip",
     "contraction.hip",
+    "gemm_f16.hip",
+    "gemm_f32.hip",
+    "gemm_f64.hip",
 ]
 
 COMMON = ["-std=c++17", "-O3", "-fPIC", "-Wall", "-Wno-unused-function"]

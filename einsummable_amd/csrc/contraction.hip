@@ -20,11 +20,14 @@
 // four consecutive n of one m: the epilogue stores them with one 8 / 16-byte write.
 // fp16 inputs accumulate in fp32 (v_mfma_f32_32x32x16_f16), fp32 uses v_mfma_f32_32x32x2_f32,
 // f64 uses v_mfma_f64_16x16x4_f64.
+#include "gemm_kernel.h"
 #include "kernel_manager.h"
 
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <cstdio>
+#include <cstdlib>
 #include <cstring>
 
 namespace es
@@ -32,429 +35,7 @@ namespace es
 namespace
 {
 
-constexpr int MAXG = 4;  // modes per group
-
-// One group of modes, innermost first.  Unused slots have size 1 and stride 0.
-struct group_t {
-    uint32_t n;
-    uint32_t size[MAXG];
-    int64_t  sx[MAXG];  // stride in the first tensor that holds the group
-    int64_t  sy[MAXG];  // stride in the second tensor that holds the group
-    int64_t  sz[MAXG];  // batch only: stride in C
-};
-
-struct gemm_args_t {
-    const void* A;
-    const void* B;
-    void*       C;
-    uint32_t    M, N, K, batch;
-    uint32_t    tiles_m, tiles_n;
-    group_t     gm;  // sx: A, sy: C
-    group_t     gn;  // sx: B, sy: C
-    group_t     gk;  // sx: A, sy: B
-    group_t     gb;  // sx: A, sy: B, sz: C
-    int         a_mode, b_mode;  // 0: 16-byte vectors along k, 1: along m / n, 2: elementwise
-    int         c_mode;          // 0: four consecutive n per store, 2: elementwise
-};
-
-__device__ __forceinline__ void group_offsets(group_t const& g, uint32_t i, int64_t& ox,
-                                              int64_t& oy)
-{
-    if (g.n == 1) {
-        ox = int64_t(i) * g.sx[0];
-        oy = int64_t(i) * g.sy[0];
-        return;
-    }
-    ox = 0;
-    oy = 0;
-#pragma unroll
-    for (int d = 0; d != MAXG; ++d) {
-        uint32_t q = i / g.size[d];
-        uint32_t r = i - q * g.size[d];
-        ox += int64_t(r) * g.sx[d];
-        oy += int64_t(r) * g.sy[d];
-        i = q;
-    }
-}
-
-typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
-typedef float    float16_t __attribute__((ext_vector_type(16)));
-typedef float    float4_t __attribute__((ext_vector_type(4)));
-typedef double   double4_t __attribute__((ext_vector_type(4)));
-
-struct alignas(16) chunk_t {
-    uint32_t w[4];
-};
-
-template <typename T>
-struct traits_t;
-
-template <>
-struct traits_t<_Float16> {
-    static constexpr int MI = 32;    // rows/cols of one MFMA tile
-    static constexpr int VL = 8;     // elements in a 16-byte chunk
-    static constexpr int KG = 2;     // lane groups along k (64 / MI)
-    static constexpr int NACC = 16;  // accumulator elements per lane per tile
-    using acc_elem = float;
-    using acc_t = float16_t;
-    __device__ static __forceinline__ void mma(acc_t& acc, chunk_t const& row, chunk_t const& col)
-    {
-        half8_t r, c;
-        __builtin_memcpy(&r, &row, 16);
-        __builtin_memcpy(&c, &col, 16);
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(r, c, acc, 0, 0, 0);
-    }
-    // n of accumulator element i in lane l
-    __device__ static __forceinline__ int acc_row(int i, int lane)
-    {
-        return (i / 4) * 8 + (lane / 32) * 4 + (i % 4);
-    }
-    static constexpr bool QUAD = true;  // registers 4q..4q+3 hold four consecutive rows
-};
-
-template <>
-struct traits_t<float> {
-    static constexpr int MI = 32;
-    static constexpr int VL = 4;
-    static constexpr int KG = 2;
-    static constexpr int NACC = 16;
-    using acc_elem = float;
-    using acc_t = float16_t;
-    __device__ static __forceinline__ void mma(acc_t& acc, chunk_t const& row, chunk_t const& col)
-    {
-        float r[4], c[4];
-        __builtin_memcpy(r, &row, 16);
-        __builtin_memcpy(c, &col, 16);
-#pragma unroll
-        for (int j = 0; j != 4; ++j) {
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(r[j], c[j], acc, 0, 0, 0);
-        }
-    }
-    __device__ static __forceinline__ int acc_row(int i, int lane)
-    {
-        return (i / 4) * 8 + (lane / 32) * 4 + (i % 4);
-    }
-    static constexpr bool QUAD = true;  // registers 4q..4q+3 hold four consecutive rows
-};
-
-template <>
-struct traits_t<double> {
-    static constexpr int MI = 16;
-    static constexpr int VL = 2;
-    static constexpr int KG = 4;
-    static constexpr int NACC = 4;
-    using acc_elem = double;
-    using acc_t = double4_t;
-    __device__ static __forceinline__ void mma(acc_t& acc, chunk_t const& row, chunk_t const& col)
-    {
-        double r[2], c[2];
-        __builtin_memcpy(r, &row, 16);
-        __builtin_memcpy(c, &col, 16);
-#pragma unroll
-        for (int j = 0; j != 2; ++j) {
-            acc = __builtin_amdgcn_mfma_f64_16x16x4f64(r[j], c[j], acc, 0, 0, 0);
-        }
-    }
-    // v_mfma_f64_16x16x4_f64 interleaves rows across registers: register i of lane l holds
-    // row 4 * i + l / 16, so a lane's four values are four rows apart
-    __device__ static __forceinline__ int acc_row(int i, int lane) { return 4 * i + lane / 16; }
-    static constexpr bool QUAD = false;
-};
-
-constexpr int ROW_BYTES = 128;  // bytes of k per tile row per stage
-constexpr int ROW_PITCH = 144;  // padded LDS row
-constexpr int CHUNKS_PER_ROW = ROW_BYTES / 16;
-
-// Loads one BR x (128 byte) operand slice into registers (NV chunks per thread).
-//   mode 0: the slice is [row][k] in memory with k contiguous
-//   mode 1: the slice is [k][row] in memory with row contiguous
-//   mode 2: arbitrary strides, element by element
-// `row_off[v]` / `row_ok[v]` describe the thread's rows (mode 0, 2) or its row-vector (mode 1).
-template <typename T, int BR, int NV>
-struct operand_loader_t {
-    using tr = traits_t<T>;
-    static constexpr int VL = tr::VL;
-    static constexpr int BK = ROW_BYTES / int(sizeof(T));
-
-    T const*       base;        // tensor + batch offset
-    group_t const* grow;        // m or n group
-    group_t const* gk;
-    bool           use_sy_k;    // k strides: sx for A, sy for B
-    int            mode;
-    uint32_t       R, K;        // extents
-    uint32_t       row0;        // first row of the tile
-    // mode 0 / 2: per-chunk row offsets
-    int64_t        row_off[NV];
-    bool           row_ok[NV];
-
-    __device__ __forceinline__ int64_t k_off(uint32_t k) const
-    {
-        int64_t a, b;
-        group_offsets(*gk, k, a, b);
-        return use_sy_k ? b : a;
-    }
-
-    __device__ __forceinline__ int64_t r_off(uint32_t r) const
-    {
-        int64_t a, b;
-        group_offsets(*grow, r, a, b);
-        return a;
-    }
-
-    __device__ void init(int tid)
-    {
-        if (mode == 1) {
-            // chunk v: k-row kk = v / (BR / VL), row vector rv = v % (BR / VL)
-#pragma unroll
-            for (int i = 0; i != NV; ++i) {
-                int      v = tid + 256 * i;
-                uint32_t r = row0 + uint32_t(v % (BR / VL)) * VL;
-                row_ok[i] = r < R;
-                row_off[i] = row_ok[i] ? r_off(r) : 0;
-            }
-        } else {
-#pragma unroll
-            for (int i = 0; i != NV; ++i) {
-                int      v = tid + 256 * i;
-                uint32_t r = row0 + uint32_t(v / CHUNKS_PER_ROW);
-                row_ok[i] = r < R;
-                row_off[i] = row_ok[i] ? r_off(r) : 0;
-            }
-        }
-    }
-
-    __device__ __forceinline__ void load(int tid, uint32_t k0, chunk_t (&regs)[NV]) const
-    {
-        if (mode == 0) {
-            uint32_t k = k0 + uint32_t(tid % CHUNKS_PER_ROW) * VL;
-            bool     kok = k < K;
-            int64_t  ko = kok ? k_off(k) : 0;
-#pragma unroll
-            for (int i = 0; i != NV; ++i) {
-                chunk_t c = {{0, 0, 0, 0}};
-                if (kok && row_ok[i]) {
-                    c = *reinterpret_cast<chunk_t const*>(base + row_off[i] + ko);
-                }
-                regs[i] = c;
-            }
-        } else if (mode == 1) {
-#pragma unroll
-            for (int i = 0; i != NV; ++i) {
-                int      v = tid + 256 * i;
-                uint32_t k = k0 + uint32_t(v / (BR / VL));
-                chunk_t  c = {{0, 0, 0, 0}};
-                if (k < K && row_ok[i]) {
-                    c = *reinterpret_cast<chunk_t const*>(base + row_off[i] + k_off(k));
-                }
-                regs[i] = c;
-            }
-        } else {
-            uint32_t kb = k0 + uint32_t(tid % CHUNKS_PER_ROW) * VL;
-#pragma unroll
-            for (int i = 0; i != NV; ++i) {
-                T e[VL];
-#pragma unroll
-                for (int j = 0; j != VL; ++j) {
-                    uint32_t k = kb + uint32_t(j);
-                    e[j] = (k < K && row_ok[i]) ? base[row_off[i] + k_off(k)] : T(0);
-                }
-                __builtin_memcpy(&regs[i], e, 16);
-            }
-        }
-    }
-
-    // registers -> LDS slice laid out [row][k] with ROW_PITCH bytes per row
-    __device__ __forceinline__ void store(int tid, char* lds, chunk_t const (&regs)[NV]) const
-    {
-        if (mode == 1) {
-#pragma unroll
-            for (int i = 0; i != NV; ++i) {
-                int v = tid + 256 * i;
-                int kk = v / (BR / VL);
-                int r = (v % (BR / VL)) * VL;
-                T   e[VL];
-                __builtin_memcpy(e, &regs[i], 16);
-#pragma unroll
-                for (int j = 0; j != VL; ++j) {
-                    *reinterpret_cast<T*>(lds + (r + j) * ROW_PITCH + kk * int(sizeof(T))) = e[j];
-                }
-            }
-        } else {
-#pragma unroll
-            for (int i = 0; i != NV; ++i) {
-                int v = tid + 256 * i;
-                int r = v / CHUNKS_PER_ROW;
-                int c = v % CHUNKS_PER_ROW;
-                *reinterpret_cast<chunk_t*>(lds + r * ROW_PITCH + c * 16) = regs[i];
-            }
-        }
-    }
-};
-
-template <typename T, int BM, int BN>
-__global__ __launch_bounds__(256) void gemm_kernel(gemm_args_t a)
-{
-    using tr = traits_t<T>;
-    constexpr int MI = tr::MI;
-    constexpr int VL = tr::VL;
-    constexpr int BK = ROW_BYTES / int(sizeof(T));
-    constexpr int WM = BM / 2, WN = BN / 2;  // wave tile
-    constexpr int TM = WM / MI, TN = WN / MI;
-    constexpr int NVA = BM * CHUNKS_PER_ROW / 256;
-    constexpr int NVB = BN * CHUNKS_PER_ROW / 256;
-    constexpr int STEPS = BK / (tr::KG * VL);
-
-    extern __shared__ __attribute__((aligned(16))) char lds[];
-    constexpr int A_BYTES = BM * ROW_PITCH;
-    constexpr int STAGE = (BM + BN) * ROW_PITCH;
-
-    int const tid = threadIdx.x;
-    int const lane = tid & 63;
-    int const wave = tid >> 6;
-    int const wm = wave >> 1, wn = wave & 1;
-
-    // tile coordinates; consecutive blocks walk down m first so that they share the B panel
-    uint32_t const tile = blockIdx.x;
-    uint32_t const tm = tile % a.tiles_m;
-    uint32_t const tn = tile / a.tiles_m;
-    uint32_t const bz = blockIdx.y;
-
-    int64_t boa, bob, boc;
-    {
-        int64_t x, y;
-        group_offsets(a.gb, bz, x, y);
-        boa = x;
-        bob = y;
-        // C strides of the batch group
-        boc = 0;
-        uint32_t i = bz;
-#pragma unroll
-        for (int d = 0; d != MAXG; ++d) {
-            uint32_t q = i / a.gb.size[d];
-            boc += int64_t(i - q * a.gb.size[d]) * a.gb.sz[d];
-            i = q;
-        }
-    }
-
-    operand_loader_t<T, BM, NVA> la;
-    la.base = static_cast<T const*>(a.A) + boa;
-    la.grow = &a.gm;
-    la.gk = &a.gk;
-    la.use_sy_k = false;
-    la.mode = a.a_mode;
-    la.R = a.M;
-    la.K = a.K;
-    la.row0 = tm * BM;
-    la.init(tid);
-
-    operand_loader_t<T, BN, NVB> lb;
-    lb.base = static_cast<T const*>(a.B) + bob;
-    lb.grow = &a.gn;
-    lb.gk = &a.gk;
-    lb.use_sy_k = true;
-    lb.mode = a.b_mode;
-    lb.R = a.N;
-    lb.K = a.K;
-    lb.row0 = tn * BN;
-    lb.init(tid);
-
-    typename tr::acc_t acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i != TM; ++i) {
-#pragma unroll
-        for (int j = 0; j != TN; ++j) {
-#pragma unroll
-            for (int e = 0; e != tr::NACC; ++e) acc[i][j][e] = 0;
-        }
-    }
-
-    chunk_t ra[NVA], rb[NVB];
-    uint32_t const nk = (a.K + BK - 1) / BK;
-
-    la.load(tid, 0, ra);
-    lb.load(tid, 0, rb);
-    la.store(tid, lds, ra);
-    lb.store(tid, lds + A_BYTES, rb);
-    __syncthreads();
-
-    // fragment addresses of this lane inside a stage
-    int const frow = lane % MI;
-    int const fk = (lane / MI) * 16;
-
-    for (uint32_t kt = 0; kt != nk; ++kt) {
-        char const* cur = lds + (kt & 1) * STAGE;
-        char*       nxt = lds + ((kt + 1) & 1) * STAGE;
-        bool const  more = kt + 1 != nk;
-        if (more) {
-            la.load(tid, (kt + 1) * BK, ra);
-            lb.load(tid, (kt + 1) * BK, rb);
-        }
-#pragma unroll
-        for (int s = 0; s != STEPS; ++s) {
-            chunk_t fa[TM], fb[TN];
-#pragma unroll
-            for (int i = 0; i != TM; ++i) {
-                fa[i] = *reinterpret_cast<chunk_t const*>(
-                    cur + (wm * WM + i * MI + frow) * ROW_PITCH + s * tr::KG * 16 + fk);
-            }
-#pragma unroll
-            for (int j = 0; j != TN; ++j) {
-                fb[j] = *reinterpret_cast<chunk_t const*>(
-                    cur + A_BYTES + (wn * WN + j * MI + frow) * ROW_PITCH + s * tr::KG * 16 + fk);
-            }
-#pragma unroll
-            for (int i = 0; i != TM; ++i) {
-#pragma unroll
-                for (int j = 0; j != TN; ++j) tr::mma(acc[i][j], fb[j], fa[i]);
-            }
-        }
-        if (more) {
-            la.store(tid, nxt, ra);
-            lb.store(tid, nxt + A_BYTES, rb);
-        }
-        __syncthreads();
-    }
-
-    // epilogue: lane holds, per tile, NACC values: n = acc_row(e, lane), m = lane % MI
-    T* const C = static_cast<T*>(a.C) + boc;
-#pragma unroll
-    for (int i = 0; i != TM; ++i) {
-        uint32_t m = tm * BM + wm * WM + i * MI + lane % MI;
-        if (m >= a.M) continue;
-        int64_t mo_a, mo_c;
-        group_offsets(a.gm, m, mo_a, mo_c);
-#pragma unroll
-        for (int j = 0; j != TN; ++j) {
-            uint32_t nb = tn * BN + wn * WN + j * MI;
-#pragma unroll
-            for (int e0 = 0; e0 < tr::NACC; e0 += 4) {
-                if (tr::QUAD && a.c_mode == 0) {
-                    uint32_t n = nb + uint32_t(tr::acc_row(e0, lane));
-                    if (n < a.N) {
-                        int64_t no_b, no_c;
-                        group_offsets(a.gn, n, no_b, no_c);
-                        struct alignas(4 * sizeof(T)) quad_t {
-                            T v[4];
-                        } q;
-#pragma unroll
-                        for (int t = 0; t != 4; ++t) q.v[t] = T(acc[i][j][e0 + t]);
-                        *reinterpret_cast<quad_t*>(C + mo_c + no_c) = q;
-                    }
-                } else {
-#pragma unroll
-                    for (int t = 0; t != 4; ++t) {
-                        uint32_t n = nb + uint32_t(tr::acc_row(e0 + t, lane));
-                        if (n < a.N) {
-                            int64_t no_b, no_c;
-                            group_offsets(a.gn, n, no_b, no_c);
-                            C[mo_c + no_c] = T(acc[i][j][e0 + t]);
-                        }
-                    }
-                }
-            }
-        }
-    }
-}
+using namespace gemm;
 
 // ----------------------------------------------------------------------------- planner
 
@@ -480,6 +61,33 @@ void fill_group(group_t& g, std::vector<mode_info_t> const& ms,
     }
 }
 
+// Macro tile for a problem.  128x128 tiles keep two workgroups per compute unit, which hide
+// each other's slice boundaries; 256x256 tiles halve the LDS and L2 traffic per flop but run
+// one wave per SIMD, so they only pay when there are several full rounds of them over the
+// 256 compute units (measured crossover on MI355X: ~3 rounds).
+// ES_KM_GEMM_TILE=128x128|256x256 overrides the choice (tuning aid).
+void choose_tile(dtype_t dt, uint64_t M, uint64_t N, uint64_t K, uint64_t batch, int& bm, int& bn)
+{
+    bm = 128;
+    bn = 128;
+    if (dt == dtype_t::f64) return;
+    if (const char* env = std::getenv("ES_KM_GEMM_TILE")) {
+        int x = 0, y = 0;
+        if (std::sscanf(env, "%dx%d", &x, &y) == 2 && x == y && (x == 128 || x == 256)) {
+            bm = x;
+            bn = y;
+            return;
+        }
+    }
+    // short reductions are bound by the output write, narrow outputs waste a wide tile
+    if (K < 1024 || M < 512 || N < 512) return;
+    uint64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256) * batch;
+    if (big_tiles >= 768) {
+        bm = 256;
+        bn = 256;
+    }
+}
+
 // Adjacent modes of a group that are also adjacent (same order, dense) in every tensor that
 // holds them were already fused by merge_adjacent_dims; what is left is genuinely strided.
 struct contraction_plan_t : plan_t {
@@ -499,39 +107,25 @@ struct contraction_plan_t : plan_t {
         if (mis(a.A) && a.a_mode != 2) a.a_mode = 2;
         if (mis(a.B) && a.b_mode != 2) a.b_mode = 2;
         if (mis(a.C) && a.c_mode != 2) a.c_mode = 2;
-        dim3   grid(a.tiles_m * a.tiles_n, a.batch, 1);
-        size_t lds = size_t(2) * size_t(bm + bn) * ROW_PITCH;
-        // more than 64 KiB of dynamic LDS has to be requested once per kernel
-        static bool const raised = [lds] {
-            int n = int(lds);
-            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<_Float16, 128, 128>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, n);
-            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<float, 128, 128>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, n);
-            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<double, 128, 128>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, n);
-            return true;
-        }();
-        (void)raised;
-        switch (dtype) {
-            case dtype_t::f16:
-                hipLaunchKernelGGL((gemm_kernel<_Float16, 128, 128>), grid, dim3(256), lds, stream,
-                                   a);
-                break;
-            case dtype_t::f32:
-                hipLaunchKernelGGL((gemm_kernel<float, 128, 128>), grid, dim3(256), lds, stream, a);
-                break;
-            case dtype_t::f64:
-                hipLaunchKernelGGL((gemm_kernel<double, 128, 128>), grid, dim3(256), lds, stream,
-                                   a);
-                break;
-            default:
-                break;
-        }
+        launch(a, stream);
         hipError_t err = hipGetLastError();
         if (err != hipSuccess) {
             throw km_error(km_status::device,
                            std::string("contraction launch: ") + hipGetErrorString(err));
+        }
+    }
+
+    void launch(gemm_args_t const& a, hipStream_t stream) const
+    {
+        switch (dtype) {
+            case dtype_t::f16:
+                return launch_gemm_f16(bm, bn, a, stream);
+            case dtype_t::f32:
+                return launch_gemm_f32(bm, bn, a, stream);
+            case dtype_t::f64:
+                return launch_gemm_f64(bm, bn, a, stream);
+            default:
+                return;
         }
     }
 };
@@ -629,9 +223,6 @@ std::shared_ptr<plan_t> plan_contraction(einsummable_t const& e, int)
     a.N = uint32_t(N);
     a.K = uint32_t(K);
     a.batch = uint32_t(Bt);
-    a.tiles_m = uint32_t((M + p->bm - 1) / p->bm);
-    a.tiles_n = uint32_t((N + p->bn - 1) / p->bn);
-    if (uint64_t(a.tiles_m) * a.tiles_n >= lim) return nullptr;
 
     int const VL = 16 / int(dtype_size(dt));
     auto vec_ok = [&](std::vector<mode_info_t> const& g, int64_t mode_info_t::*s, int q) {
@@ -641,9 +232,16 @@ std::shared_ptr<plan_t> plan_contraction(einsummable_t const& e, int)
     a.b_mode = vec_ok(js, sB, VL) ? 0 : (vec_ok(gn, sB, VL) ? 1 : 2);
     a.c_mode = vec_ok(gn, sC, 4) ? 0 : 2;
 
+    // large tiles exist for the vector load paths (A along k; B along k or n)
+    if (a.a_mode == 0 && a.b_mode != 2) choose_tile(dt, M, N, K, Bt, p->bm, p->bn);
+    a.tiles_m = uint32_t((M + p->bm - 1) / p->bm);
+    a.tiles_n = uint32_t((N + p->bn - 1) / p->bn);
+    if (uint64_t(a.tiles_m) * a.tiles_n >= lim) return nullptr;
+
     p->workspace_bytes = 0;
     static const char* mode_name[] = {"k", "mn", "elem"};
-    p->description = std::string("contraction_mfma_") + dtype_name(dt) + " tile=128x128 A=" +
+    p->description = std::string("contraction_mfma_") + dtype_name(dt) + " tile=" +
+                     std::to_string(p->bm) + "x" + std::to_string(p->bn) + " A=" +
                      mode_name[a.a_mode] + " B=" + mode_name[a.b_mode] + " C=" +
                      (a.c_mode == 0 ? "vec" : "elem") + (swapped ? " swapped" : "") +
                      " M=" + std::to_string(M) + " N=" + std::to_string(N) + " K=" +
