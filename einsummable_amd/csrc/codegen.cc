@@ -8,6 +8,7 @@
 #include <algorithm>
 #include <cmath>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <sstream>
@@ -102,7 +103,9 @@ struct emitter_t {
                 if (n.dtype == dtype_t::c64) return define(n.dtype, "c_mul(" + c[0] + ", " + c[1] + ")");
                 return define(n.dtype, c[0] + " * " + c[1]);
             case op_kind::exp:
-                return define(n.dtype, std::string(dbl ? "exp(" : "expf(") + c[0] + ")");
+                // f16 / f32: v_exp_f32 on x * log2(e); relative error ~ (2 + |x|) * 2^-24, well
+                // inside the 1e-4 contract on the whole finite range of expf
+                return define(n.dtype, std::string(dbl ? "exp(" : "__expf(") + c[0] + ")");
             case op_kind::log:
                 return define(n.dtype, std::string(dbl ? "log(" : "logf(") + c[0] + ")");
             case op_kind::power: {
@@ -161,6 +164,35 @@ __device__ __forceinline__ c64 c_mul(c64 a, c64 b)
 }
 template <typename T, int N>
 struct __attribute__((aligned(sizeof(T) * N))) vec_t { T v[N]; };
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+struct u32x8 { u32x4 lo, hi; };
+// vector load / store; NT != 0 marks the access non-temporal (streamed once, no reuse)
+template <int NT, typename VT>
+__device__ __forceinline__ VT ldv(const VT* p)
+{
+    if constexpr (NT && sizeof(VT) == 16) {
+        return __builtin_bit_cast(VT, __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p)));
+    } else if constexpr (NT && sizeof(VT) == 32) {
+        const u32x4* q = reinterpret_cast<const u32x4*>(p);
+        return __builtin_bit_cast(VT, u32x8{__builtin_nontemporal_load(q),
+                                            __builtin_nontemporal_load(q + 1)});
+    } else {
+        return *p;
+    }
+}
+template <int NT, typename VT>
+__device__ __forceinline__ void stv(VT* p, VT v)
+{
+    if constexpr (NT && sizeof(VT) == 16) {
+        __builtin_nontemporal_store(__builtin_bit_cast(u32x4, v), reinterpret_cast<u32x4*>(p));
+    } else if constexpr (NT && sizeof(VT) == 32) {
+        u32x8 w = __builtin_bit_cast(u32x8, v);
+        __builtin_nontemporal_store(w.lo, reinterpret_cast<u32x4*>(p));
+        __builtin_nontemporal_store(w.hi, reinterpret_cast<u32x4*>(p) + 1);
+    } else {
+        *p = v;
+    }
+}
 __device__ __forceinline__ float  cvt_in(f16 v) { return (float)v; }
 __device__ __forceinline__ float  cvt_in(float v) { return v; }
 __device__ __forceinline__ double cvt_in(double v) { return v; }
@@ -251,10 +283,14 @@ std::string combine_expr(castable_t c, dtype_t d, std::string const& a, std::str
             return a + " + " + v;
         case castable_t::mul:
             return a + " * " + v;
+        // one v_min / v_max instead of compare + select; identical to make_min / make_max
+        // (scalarop.cc:2267-2280) for every pair of non-NaN values up to the sign of a zero
         case castable_t::min:
-            return "(" + a + " < " + v + ") ? " + a + " : " + v;
+            return std::string(is_double(d) ? "__builtin_fmin(" : "__builtin_fminf(") + a + ", " +
+                   v + ")";
         case castable_t::max:
-            return "(" + a + " > " + v + ") ? " + a + " : " + v;
+            return std::string(is_double(d) ? "__builtin_fmax(" : "__builtin_fmaxf(") + a + ", " +
+                   v + ")";
     }
     return a;
 }
@@ -332,6 +368,16 @@ std::string entry_name(einsummable_t const& e, const char* kind)
     return s + buf;
 }
 
+// Tuning aids: ES_KM_EW_UNROLL (vectors per thread of the elementwise kernels) and
+// ES_KM_RED_UNROLL / ES_KM_RED_TEAM (row reductions) override the generators' defaults.
+int env_int(const char* name, int fallback)
+{
+    const char* v = std::getenv(name);
+    if (!v || !*v) return fallback;
+    int x = std::atoi(v);
+    return x > 0 ? x : fallback;
+}
+
 bool fits32(einsummable_t const& e)
 {
     uint64_t const lim = (1ull << 32) - 1;
@@ -387,8 +433,15 @@ cg_kernel_t gen_elementwise(einsummable_t const& e, int max_vec)
     } else {
         V = pow2_divisor(inner, vcap);
     }
-    int const U = (L.NI <= 2) ? 4 : 2;
-    uint64_t const n_vec = all_straight ? n_out / uint64_t(V) : n_out / uint64_t(V);
+    int const U = env_int("ES_KM_EW_UNROLL", 1);
+    // Outputs far larger than the last-level cache are written non-temporally: they would
+    // only evict inputs that later nodes still read (measured on 8192^2 f16: +20% on the
+    // producing kernel).  ES_KM_EW_NT: 1 loads and stores, 2 loads only, 3 stores only, 4 none.
+    uint64_t const out_bytes = n_out * dtype_size(e.out_dtype());
+    int const nt_mode = env_int("ES_KM_EW_NT", out_bytes >= (64ull << 20) ? 3 : 4);
+    int const NT_LD = (nt_mode == 1 || nt_mode == 2) ? 1 : 0;
+    int const NT_ST = (nt_mode == 1 || nt_mode == 3) ? 1 : 0;
+    uint64_t const n_vec = n_out / uint64_t(V);
     g.k.vec = V;
 
     int p_nvec = g.param(n_vec);
@@ -435,8 +488,8 @@ cg_kernel_t gen_elementwise(einsummable_t const& e, int max_vec)
     for (int k = 0; k != L.NI; ++k) {
         std::string T = storage_type(e.inn_dtype(k));
         if (acc[k] == access_t::straight) {
-            s << "            r" << k << "[u] = *reinterpret_cast<const vec_t<" << T
-              << ", V>*>(a.in" << k << " + vid[u] * V);\n";
+            s << "            r" << k << "[u] = ldv<" << NT_LD << ">(reinterpret_cast<const vec_t<" << T
+              << ", V>*>(a.in" << k << " + vid[u] * V));\n";
             continue;
         }
         std::string off = "0";
@@ -444,8 +497,8 @@ cg_kernel_t gen_elementwise(einsummable_t const& e, int max_vec)
             if (p_str[k][m] >= 0) off += " + d" + std::to_string(m) + " * " + g.P(p_str[k][m]);
         }
         if (acc[k] == access_t::vec) {
-            s << "            r" << k << "[u] = *reinterpret_cast<const vec_t<" << T
-              << ", V>*>(a.in" << k << " + (" << off << " + c));\n";
+            s << "            r" << k << "[u] = ldv<" << NT_LD << ">(reinterpret_cast<const vec_t<" << T
+              << ", V>*>(a.in" << k << " + (" << off << " + c)));\n";
         } else if (acc[k] == access_t::bcast) {
             s << "            s" << k << "[u] = a.in" << k << "[" << off << "];\n";
         } else {
@@ -473,8 +526,8 @@ cg_kernel_t gen_elementwise(einsummable_t const& e, int max_vec)
         return call + ")";
     }()) << ";\n";
     s << "            }\n";
-    s << "            *reinterpret_cast<vec_t<" << storage_type(e.out_dtype())
-      << ", V>*>(a.out + vid[u] * V) = res;\n";
+    s << "            stv<" << NT_ST << ">(reinterpret_cast<vec_t<" << storage_type(e.out_dtype())
+      << ", V>*>(a.out + vid[u] * V), res);\n";
     s << "        }\n    }\n";
     if (tail) {
         s << "    if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x < " << tail << ") {\n";
@@ -526,9 +579,10 @@ cg_kernel_t gen_reduce_row(einsummable_t const& e, int max_vec)
     int const vcap = std::min(max_vec, 16 / min_elem_size(e));
     int const V = pow2_divisor(L.shape[R - 1], vcap);
     uint64_t const nvecA = nA / uint64_t(V);
-    int const TEAM = (nvecA >= 512) ? 256 : 64;
+    int const TEAM = env_int("ES_KM_RED_TEAM", (nvecA >= 512) ? 256 : 64) == 256 ? 256 : 64;
     int const BLOCK = 256;
-    int const U = (nvecA >= uint64_t(TEAM) * 4) ? 4 : ((nvecA >= uint64_t(TEAM) * 2) ? 2 : 1);
+    int const U = env_int("ES_KM_RED_UNROLL",
+                          (nvecA >= uint64_t(TEAM) * 4) ? 4 : ((nvecA >= uint64_t(TEAM) * 2) ? 2 : 1));
     g.k.vec = V;
 
     int p_nout = g.param(n_out);
@@ -554,7 +608,17 @@ cg_kernel_t gen_reduce_row(einsummable_t const& e, int max_vec)
     s << "    const idx_t nvec = " << g.P(p_nvec) << ";\n";
     s << "    const unsigned lane = threadIdx.x % TEAM;\n";
     s << "    const idx_t row = ((idx_t)blockIdx.y * gridDim.x + blockIdx.x) * (" << BLOCK << " / TEAM) + threadIdx.x / TEAM;\n";
+    // min / max of f16 values is exact in f16: keep V packed half accumulators per lane
+    // (v_pk_max_f16 / v_pk_min_f16, no conversions) and widen once after the loop
+    bool const half_minmax = od == dtype_t::f16 && L.NI == 1 && e.join.is_identity() &&
+                             acc[0] == access_t::vec &&
+                             (cast == castable_t::min || cast == castable_t::max);
     s << "    " << ACC << " acc = " << identity_of(cast, od) << ";\n";
+    if (half_minmax) {
+        s << "    vec_t<f16, V> accv;\n#pragma unroll\n    for (int j = 0; j != V; ++j) accv.v[j] = "
+             "(f16)("
+          << identity_of(cast, od) << ");\n";
+    }
     s << "    if (row < n_out) {\n";
     s << "        idx_t rem = row;\n";
     for (int m = O - 1; m >= 1; --m) {
@@ -621,19 +685,27 @@ cg_kernel_t gen_reduce_row(einsummable_t const& e, int max_vec)
     s << "#pragma unroll\n            for (int u = 0; u != U; ++u) {\n";
     s << "                if (v0 + (idx_t)u * TEAM < nvec) {\n";
     s << "#pragma unroll\n                    for (int j = 0; j != V; ++j) {\n";
-    s << "                        acc = comb(acc, join_fn(";
-    for (int k = 0; k != L.NI; ++k) {
-        s << (k ? ", " : "");
-        if (row_const[k]) {
-            s << "c" << k;
-        } else if (acc[k] == access_t::bcast) {
-            s << "cvt_in(s" << k << "[u])";
-        } else {
-            s << "cvt_in(r" << k << "[u].v[j])";
+    if (half_minmax) {
+        s << "                        accv.v[j] = "
+          << (cast == castable_t::max ? "__builtin_fmaxf16" : "__builtin_fminf16")
+          << "(accv.v[j], r0[u].v[j]);\n                    }\n                }\n            }\n";
+        s << "        }\n    }\n";
+        s << "#pragma unroll\n    for (int j = 0; j != V; ++j) acc = comb(acc, (float)accv.v[j]);\n";
+    } else {
+        s << "                        acc = comb(acc, join_fn(";
+        for (int k = 0; k != L.NI; ++k) {
+            s << (k ? ", " : "");
+            if (row_const[k]) {
+                s << "c" << k;
+            } else if (acc[k] == access_t::bcast) {
+                s << "cvt_in(s" << k << "[u])";
+            } else {
+                s << "cvt_in(r" << k << "[u].v[j])";
+            }
         }
+        s << "));\n                    }\n                }\n            }\n";
+        s << "        }\n    }\n";
     }
-    s << "));\n                    }\n                }\n            }\n";
-    s << "        }\n    }\n";
     s << "#pragma unroll\n    for (int m = 32; m >= 1; m >>= 1) acc = comb(acc, lane_xor(acc, m));\n";
     if (TEAM == 256) {
         s << "    __shared__ " << ACC << " part[4];\n";
