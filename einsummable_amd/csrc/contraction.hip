@@ -107,6 +107,8 @@ struct contraction_plan_t : plan_t {
         if (mis(a.A) && a.a_mode != 2) a.a_mode = 2;
         if (mis(a.B) && a.b_mode != 2) a.b_mode = 2;
         if (mis(a.C) && a.c_mode != 2) a.c_mode = 2;
+        // the wide epilogue lives in the tuned kernel (A along k, B along k or n)
+        if (a.c_mode == 3 && !(a.a_mode == 0 && a.b_mode != 2)) a.c_mode = 0;
         launch(a, stream);
         hipError_t err = hipGetLastError();
         if (err != hipSuccess) {
@@ -230,7 +232,7 @@ std::shared_ptr<plan_t> plan_contraction(einsummable_t const& e, int)
     };
     a.a_mode = vec_ok(js, sA, VL) ? 0 : (vec_ok(gm, sA, VL) ? 1 : 2);
     a.b_mode = vec_ok(js, sB, VL) ? 0 : (vec_ok(gn, sB, VL) ? 1 : 2);
-    a.c_mode = vec_ok(gn, sC, 4) ? 0 : 2;
+    a.c_mode = vec_ok(gn, sC, VL) ? 3 : (vec_ok(gn, sC, 4) ? 0 : 2);
 
     // large tiles exist for the vector load paths (A along k; B along k or n)
     if (a.a_mode == 0 && a.b_mode != 2) choose_tile(dt, M, N, K, Bt, p->bm, p->bn);
@@ -243,7 +245,8 @@ std::shared_ptr<plan_t> plan_contraction(einsummable_t const& e, int)
     p->description = std::string("contraction_mfma_") + dtype_name(dt) + " tile=" +
                      std::to_string(p->bm) + "x" + std::to_string(p->bn) + " A=" +
                      mode_name[a.a_mode] + " B=" + mode_name[a.b_mode] + " C=" +
-                     (a.c_mode == 0 ? "vec" : "elem") + (swapped ? " swapped" : "") +
+                     (a.c_mode == 3 ? "wide" : (a.c_mode == 0 ? "vec" : "elem")) +
+                     (swapped ? " swapped" : "") +
                      " M=" + std::to_string(M) + " N=" + std::to_string(N) + " K=" +
                      std::to_string(K) + " batch=" + std::to_string(Bt);
     return p;

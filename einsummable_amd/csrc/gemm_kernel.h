@@ -34,7 +34,8 @@ struct gemm_args_t {
     group_t     gk;  // sx: A, sy: B
     group_t     gb;  // sx: A, sy: B, sz: C
     int         a_mode, b_mode;  // 0: 16-byte vectors along k, 1: along m / n, 2: elementwise
-    int         c_mode;          // 0: four consecutive n per store, 2: elementwise
+    int         c_mode;          // 0: four consecutive n per store, 2: elementwise,
+                                 // 3: 16-byte row segments through LDS (tuned kernel)
 };
 
 __device__ __forceinline__ void group_offsets(group_t const& g, uint32_t i, int64_t& ox,
@@ -430,7 +431,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(gemm_args_t a)
             uint32_t nb = tn * BN + wn * WN + j * MI;
 #pragma unroll
             for (int e0 = 0; e0 < tr::NACC; e0 += 4) {
-                if (tr::QUAD && a.c_mode == 0) {
+                if (tr::QUAD && a.c_mode != 2) {
                     uint32_t n = nb + uint32_t(tr::acc_row(e0, lane));
                     if (n < a.N) {
                         int64_t no_b, no_c;
@@ -484,6 +485,9 @@ __global__ __launch_bounds__(256) void gemm_fast_kernel(gemm_args_t a)
     constexpr int STEPS = BK / (tr::KG * VL);
     constexpr int A_BYTES = BM * ROW_PITCH;
     constexpr int STAGE = (BM + BN) * ROW_PITCH;
+    // B kept as [k][n] (BMODE 1): BK rows of BN elements, padded by 16 bytes
+    constexpr int PITCH_KN = BN * int(sizeof(T)) + 16;
+    static_assert(BK * PITCH_KN <= BN * ROW_PITCH, "the [k][n] layout fits the B region");
 
     extern __shared__ __attribute__((aligned(16))) char lds[];
 
@@ -596,16 +600,12 @@ __global__ __launch_bounds__(256) void gemm_fast_kernel(gemm_args_t a)
                                         (tid % CHUNKS_PER_ROW) * 16) =
                 ok ? regs[q] : chunk_t{0, 0, 0, 0};
         } else {
+            // B arrives as rows of consecutive n: kept that way in LDS ([k][n], PITCH_KN bytes
+            // per k row); the fragment reads do the transposition
             int  kk = tid / (BN / VL) + q * (256 / (BN / VL));
-            int  r = (tid % (BN / VL)) * VL;
             bool ok = k0 + uint32_t(kk) < a.K;
-            typename elems_of<T>::type e = __builtin_bit_cast(
-                typename elems_of<T>::type, ok ? regs[q] : chunk_t{0, 0, 0, 0});
-#pragma unroll
-            for (int j = 0; j != VL; ++j) {
-                *reinterpret_cast<T*>(stage + A_BYTES + (r + j) * ROW_PITCH + kk * int(sizeof(T))) =
-                    e[j];
-            }
+            *reinterpret_cast<chunk_t*>(stage + A_BYTES + kk * PITCH_KN + (tid % (BN / VL)) * 16) =
+                ok ? regs[q] : chunk_t{0, 0, 0, 0};
         }
     };
 
@@ -631,9 +631,37 @@ __global__ __launch_bounds__(256) void gemm_fast_kernel(gemm_args_t a)
         if (q < TM) {
             fa[q] = *reinterpret_cast<chunk_t const*>(cur + fa_base + q * MI * ROW_PITCH +
                                                       s * tr::KG * 16);
-        } else {
+        } else if constexpr (BMODE == 0) {
             fb[q - TM] = *reinterpret_cast<chunk_t const*>(cur + fb_base + (q - TM) * MI * ROW_PITCH +
                                                            s * tr::KG * 16);
+        } else if constexpr (sizeof(T) == 2) {
+            // ds_read_b64_tr_b16: within 16 lanes, lane i supplies the address of 4
+            // consecutive n of k-row i / 4 (column group i % 4) and receives, for its own n,
+            // the 4 consecutive k: two reads give the 8 k of the MFMA operand.
+            typedef short tr_t __attribute__((ext_vector_type(4)));
+            int const i16 = lane & 15, blk = lane >> 4;
+            int const n0 = wn * WN + (q - TM) * MI + (blk & 1) * 16 + 4 * (i16 & 3);
+            int const k0 = s * tr::KG * VL + (blk >> 1) * VL + (i16 >> 2);
+            char const* p = cur + A_BYTES + k0 * PITCH_KN + n0 * 2;
+            tr_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (__attribute__((address_space(3))) tr_t*)(p));
+            tr_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (__attribute__((address_space(3))) tr_t*)(p + 4 * PITCH_KN));
+            typedef short tr8_t __attribute__((ext_vector_type(8)));
+            tr8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            fb[q - TM] = __builtin_bit_cast(chunk_t, both);
+        } else {
+            // 4-byte elements: the operand is one element per lane per instruction, so the
+            // [k][n] rows are read directly, lanes along n
+            int const n0 = wn * WN + (q - TM) * MI + lane % MI;
+            int const k0 = s * tr::KG * VL + (lane / MI) * VL;
+            char const* p = cur + A_BYTES + k0 * PITCH_KN + n0 * int(sizeof(T));
+            chunk_t v;
+#pragma unroll
+            for (int t = 0; t != VL; ++t) {
+                v[t] = *reinterpret_cast<uint32_t const*>(p + t * PITCH_KN);
+            }
+            fb[q - TM] = v;
         }
     };
     constexpr int PAIRS = TM * TN;          // matrix-instruction groups per k-step
@@ -713,6 +741,52 @@ __global__ __launch_bounds__(256) void gemm_fast_kernel(gemm_args_t a)
     slice(nk - 1, std::false_type{});
 
     T* const C = static_cast<T*>(a.C) + boc;
+    if (a.c_mode == 3) {
+        // Wide epilogue: each wave turns MI rows of its tile through a private LDS strip so
+        // that the global stores are 16 bytes per lane and whole row segments per wavefront
+        // (the accumulator layout alone gives 8-byte stores scattered over 32 rows).
+        constexpr int STRIP_PITCH = WN * int(sizeof(T)) + 16;
+        constexpr int CPR = WN * int(sizeof(T)) / 16;  // 16-byte chunks per strip row
+        __syncthreads();                                // every wave is done with the stages
+        char* const strip = lds + wave * (MI * STRIP_PITCH);
+        typedef T quad_t __attribute__((ext_vector_type(4)));
+#pragma unroll
+        for (int i = 0; i != TM; ++i) {
+#pragma unroll
+            for (int j = 0; j != TN; ++j) {
+#pragma unroll
+                for (int e0 = 0; e0 < tr::NACC; e0 += 4) {
+                    quad_t q;
+#pragma unroll
+                    for (int t = 0; t != 4; ++t) q[t] = T(acc[i][j][e0 + t]);
+                    int n = j * MI + tr::acc_row(e0, lane);
+                    *reinterpret_cast<quad_t*>(strip + (lane % MI) * STRIP_PITCH +
+                                               n * int(sizeof(T))) = q;
+                }
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+            for (int c = 0; c != MI * CPR / 64; ++c) {
+                int      idx = c * 64 + lane;
+                int      r = idx / CPR, ch = idx % CPR;
+                uint32_t m = tm * BM + wm * WM + i * MI + uint32_t(r);
+                uint32_t n = tn * BN + wn * WN + uint32_t(ch) * VL;
+                chunk_t  v = *reinterpret_cast<chunk_t const*>(strip + r * STRIP_PITCH + ch * 16);
+                if (m < a.M && n < a.N) {
+                    int64_t mo_a, mo_c, no_b, no_c;
+                    group_offsets(a.gm, m, mo_a, mo_c);
+                    group_offsets(a.gn, n, no_b, no_c);
+                    *reinterpret_cast<chunk_t*>(C + mo_c + no_c) = v;
+                }
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i != TM; ++i) {
         uint32_t m = tm * BM + wm * WM + i * MI + lane % MI;
@@ -724,7 +798,7 @@ __global__ __launch_bounds__(256) void gemm_fast_kernel(gemm_args_t a)
             uint32_t nb = tn * BN + wn * WN + j * MI;
 #pragma unroll
             for (int e0 = 0; e0 < tr::NACC; e0 += 4) {
-                if (a.c_mode == 0) {
+                if (a.c_mode != 2) {
                     uint32_t n = nb + uint32_t(tr::acc_row(e0, lane));
                     if (n < a.N) {
                         int64_t no_b, no_c;
