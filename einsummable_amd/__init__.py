@@ -16,6 +16,7 @@ from .km import (  # noqa: F401
     KernelManager,
     KmError,
     Touch,
+    TouchBatch,
     codegen_source,
     lib_path,
     load_library,

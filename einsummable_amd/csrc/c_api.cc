@@ -313,4 +313,33 @@ int es_km_merge_adjacent_dims(const uint64_t* join_shape, int join_rank, const i
         return int(e.join_shape.size());
     });
 }
+
+int es_km_touch_batch(es_km_t* h, int n_touches, const uint64_t* touchdims, const int* ranks,
+                      const char* castables, int dtype, void* stream, void* out,
+                      const void* const* inns)
+{
+    return guarded(h, [&]() -> int {
+        if (!h) throw es::ir_error("null handle");
+        if (n_touches < 0 || (n_touches > 0 && (!touchdims || !ranks || !castables || !inns))) {
+            throw es::ir_error("touch_batch: bad arguments");
+        }
+        if (dtype < 0 || dtype > 3) throw es::ir_error("touch_batch: bad dtype");
+        if (!out) throw es::ir_error("touch_batch: null buffer");
+        std::vector<es::touch_t> ts;
+        ts.resize(size_t(n_touches));
+        std::vector<void const*> ptrs(inns, inns + n_touches);
+        const uint64_t*          d = touchdims;
+        for (int i = 0; i != n_touches; ++i) {
+            if (ranks[i] < 1 || ranks[i] > 64) throw es::ir_error("touch_batch: bad rank");
+            ts[i].dtype = es::dtype_t(dtype);
+            ts[i].castable = es::castable_from_char(castables[i]);
+            for (int k = 0; k != ranks[i]; ++k, d += 5) {
+                ts[i].selection.push_back(es::touchdim_t{d[0], d[1], d[2], d[3], d[4]});
+            }
+            if (!ptrs[i]) throw es::ir_error("touch_batch: null input");
+        }
+        h->km->touch_batch(ts, static_cast<hipStream_t>(stream), out, ptrs);
+        return ES_KM_OK;
+    });
+}
 }

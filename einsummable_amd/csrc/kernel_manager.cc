@@ -4,6 +4,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
+
 namespace es
 {
 
@@ -173,6 +175,148 @@ void kernel_manager_t::operator()(touch_t const& touch_, hipStream_t stream, voi
     if (t.castable) op = 1 + int(t.castable.value());
     launch_touch(a, esz, int(t.dtype), op, stream, out, inn);
     hip_check(hipGetLastError(), "touch launch");
+}
+
+void kernel_manager_t::touch_batch(std::vector<touch_t> const& touches_, hipStream_t stream,
+                                   void* out, std::vector<void const*> const& inns) const
+{
+    if (touches_.empty()) return;
+    if (touches_.size() != inns.size()) {
+        throw km_error(km_status::inputs, "touch_batch: one input per touch expected");
+    }
+    size_t const n = touches_.size();
+    size_t const rank0 = touches_[0].selection.size();
+    dtype_t const dt = touches_[0].dtype;
+    for (auto const& t : touches_) {
+        t.validate();
+        if (t.dtype != dt || t.selection.size() != rank0) {
+            throw km_error(km_status::invalid, "touch_batch: touches differ in dtype or rank");
+        }
+        for (size_t d = 0; d != rank0; ++d) {
+            if (t.selection[d].d_out != touches_[0].selection[d].d_out) {
+                throw km_error(km_status::invalid,
+                               "touch_batch: touches address differently shaped outputs");
+            }
+        }
+    }
+    // joint simplify: a dimension is folded into its predecessor only when every touch copies
+    // it in full (touch.cc:3-28 applied to the whole group)
+    std::vector<touch_t> ts(n);
+    for (size_t i = 0; i != n; ++i) {
+        ts[i].castable = touches_[i].castable;
+        ts[i].dtype = dt;
+    }
+    for (size_t d = 0; d != rank0; ++d) {
+        bool whole = d > 0;
+        for (auto const& t : touches_) {
+            touchdim_t const& x = t.selection[d];
+            whole = whole && x.d_inn == x.d_out && x.offset_inn == 0 && x.offset_out == 0 &&
+                    x.d_inn == x.size;
+        }
+        for (size_t i = 0; i != n; ++i) {
+            touchdim_t const& x = touches_[i].selection[d];
+            if (whole) {
+                touchdim_t& b = ts[i].selection.back();
+                b.d_inn *= x.d_inn;
+                b.d_out *= x.d_inn;
+                b.offset_inn *= x.d_inn;
+                b.offset_out *= x.d_inn;
+                b.size *= x.d_inn;
+            } else {
+                ts[i].selection.push_back(x);
+            }
+        }
+    }
+    int const r = int(ts[0].selection.size());
+    if (r > 4) throw km_error(km_status::invalid, "touch_batch: more than four dimensions");
+    int const esz = int(dtype_size(dt));
+    int const vmax = 16 / esz;
+
+    // the output is walked in 16-byte vectors whenever its rows allow it; the windows
+    // themselves only need to be vector aligned for the inputs to be read as vectors too
+    bool out_wide = reinterpret_cast<uintptr_t>(out) % 16 == 0;
+    bool aligned = true;
+    for (size_t i = 0; i != n; ++i) {
+        touchdim_t const& last = ts[i].selection[r - 1];
+        out_wide = out_wide && last.d_out % vmax == 0;
+        aligned = aligned && last.size % vmax == 0 && last.offset_inn % vmax == 0 &&
+                  last.offset_out % vmax == 0 && reinterpret_cast<uintptr_t>(inns[i]) % 16 == 0;
+        if (r > 1) aligned = aligned && last.d_inn % vmax == 0;
+        for (auto const& d : ts[i].selection) {
+            if (d.d_out >= (1ull << 32)) {
+                throw km_error(km_status::invalid, "touch_batch: extent beyond 2^32");
+            }
+        }
+    }
+    bool const wide = out_wide;
+    uint64_t out_str[4];
+    {
+        uint64_t s = 1;
+        for (int d = r - 1; d >= 0; --d) {
+            out_str[d] = s;
+            s *= ts[0].selection[d].d_out;
+        }
+    }
+    for (size_t first = 0; first < n; first += TOUCH_BATCH_MAX) {
+        size_t const  cnt = std::min<size_t>(TOUCH_BATCH_MAX, n - first);
+        touch_batch_t b;
+        b.n = int(cnt);
+        b.vec = wide ? vmax : 1;
+        b.aligned = (wide && aligned) ? 1 : 0;
+        b.any_castable = 0;
+        uint64_t lo[4] = {0, 0, 0, 0}, hi[4] = {1, 1, 1, 1};
+        for (int s = 0; s != 4; ++s) {
+            int d = r - 4 + s;
+            if (d < 0) continue;
+            lo[s] = ~0ull;
+            hi[s] = 0;
+        }
+        for (size_t i = 0; i != cnt; ++i) {
+            touch_t const& t = ts[first + i];
+            touch_item_t&  it = b.items[i];
+            it.inn = inns[first + i];
+            it.op = t.castable ? 1 + int(t.castable.value()) : 0;
+            it.pad_ = 0;
+            if (it.op) b.any_castable = 1;
+            it.base_inn = 0;
+            uint64_t si = 1;
+            uint64_t str_i[4] = {0, 0, 0, 0};
+            for (int d = r - 1; d >= 0; --d) {
+                str_i[d] = si;
+                it.base_inn += t.selection[d].offset_inn * si;
+                si *= t.selection[d].d_inn;
+            }
+            for (int s = 0; s != 4; ++s) {
+                int d = r - 4 + s;  // dimension feeding slot s
+                if (d >= 0) {
+                    it.lo[s] = uint32_t(t.selection[d].offset_out);
+                    it.size[s] = uint32_t(t.selection[d].size);
+                    if (s < 3) it.str_inn[s] = str_i[d];
+                    lo[s] = std::min<uint64_t>(lo[s], t.selection[d].offset_out);
+                    hi[s] = std::max<uint64_t>(hi[s], t.selection[d].offset_out + t.selection[d].size);
+                } else {
+                    it.lo[s] = 0;
+                    it.size[s] = 1;
+                    if (s < 3) it.str_inn[s] = 0;
+                }
+            }
+        }
+        lo[3] = lo[3] / uint64_t(b.vec) * uint64_t(b.vec);
+        hi[3] = (hi[3] + uint64_t(b.vec) - 1) / uint64_t(b.vec) * uint64_t(b.vec);
+        b.n_vec = 1;
+        for (int s = 0; s != 4; ++s) {
+            b.box_lo[s] = uint32_t(lo[s]);
+            b.box_size[s] = uint32_t(hi[s] - lo[s]);
+            b.n_vec *= (s == 3) ? (hi[s] - lo[s]) / uint64_t(b.vec) : (hi[s] - lo[s]);
+            int d = r - 4 + s;
+            if (s < 3) b.out_str[s] = d >= 0 ? out_str[d] : 0;
+        }
+        if (b.n_vec >= (1ull << 40)) {
+            throw km_error(km_status::invalid, "touch_batch: bounding box too large");
+        }
+        launch_touch_batch(b, esz, int(dt), stream, out);
+        hip_check(hipGetLastError(), "touch_batch launch");
+    }
 }
 
 void kernel_manager_t::constant_fill(dtype_t dtype, uint64_t value_bits, uint64_t nelem,

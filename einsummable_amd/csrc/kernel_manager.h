@@ -58,6 +58,11 @@ public:
 
     void operator()(touch_t const& touch, hipStream_t stream, void* out, void const* inn) const;
 
+    // All touches write the same output tensor; the result equals applying them one after
+    // the other in list order, in one launch per 32 touches.
+    void touch_batch(std::vector<touch_t> const& touches, hipStream_t stream, void* out,
+                     std::vector<void const*> const& inns) const;
+
     void constant_fill(dtype_t dtype, uint64_t value_bits, uint64_t nelem, hipStream_t stream,
                        void* out) const;
     void lowerTri_fill(dtype_t dtype, uint64_t lower_bits, uint64_t upper_bits, uint64_t nrow,

@@ -25,6 +25,36 @@ struct touch_launch_t {
 void launch_touch(touch_launch_t const& a, int elem_size, int dtype_code, int op,
                   hipStream_t stream, void* out, void const* inn);
 
+// A group of touches into one output tensor, applied in list order by a single launch: every
+// thread owns one output vector and folds the touches that cover it, so overlapping windows
+// see exactly the sequential result.  All items are normalised to four dimensions.
+struct touch_item_t {
+    void const* inn;
+    uint64_t    base_inn;    // element offset of the window's origin in the input
+    uint64_t    str_inn[3];  // element strides of the three outer dimensions of the input
+    uint32_t    lo[4];       // window origin in the output
+    uint32_t    size[4];     // window extents
+    int         op;          // 0 copy, 1 add, 2 mul, 3 min, 4 max
+    int         pad_;
+};
+
+constexpr int TOUCH_BATCH_MAX = 32;  // items per launch (kernel-argument budget)
+
+struct touch_batch_t {
+    int          n;
+    int          vec;           // elements per output vector
+    int          any_castable;  // some item reads the old output value
+    int          aligned;       // every window is vector aligned in both tensors
+    uint32_t     box_lo[4];     // bounding box of the windows
+    uint32_t     box_size[4];   // inner extent in elements
+    uint64_t     out_str[3];    // element strides of the output's outer dimensions
+    uint64_t     n_vec;
+    touch_item_t items[TOUCH_BATCH_MAX];
+};
+
+void launch_touch_batch(touch_batch_t const& b, int elem_size, int dtype_code, hipStream_t stream,
+                        void* out);
+
 void launch_fill_constant(int elem_size, uint64_t bits, uint64_t nelem, hipStream_t stream,
                           void* out);
 

@@ -176,6 +176,133 @@ void launch_touch_op(touch_launch_t const& a, int op, hipStream_t stream, void* 
     }
 }
 
+// ---- batched touches
+
+// V: elements per output vector.  ALIGNED: every window starts and ends on a vector boundary
+// in both tensors, so inputs are read as vectors too; otherwise a window may cut through an
+// output vector and its input is read element by element under a per-element mask.
+template <typename T, int V, bool ALIGNED>
+__global__ __launch_bounds__(256) void touch_batch_kernel(touch_batch_t b, T* __restrict__ out)
+{
+    using vt = vec_t<T, V>;
+    uint64_t idx = uint64_t(blockIdx.x) * 256 + threadIdx.x;
+    if (idx >= b.n_vec) return;
+    // position inside the bounding box, then absolute output coordinates
+    uint32_t vpr = b.box_size[3] / V;
+    uint32_t c[4];
+    {
+        uint64_t r = idx;
+        c[3] = b.box_lo[3] + uint32_t(r % vpr) * V;
+        r /= vpr;
+        c[2] = b.box_lo[2] + uint32_t(r % b.box_size[2]);
+        r /= b.box_size[2];
+        c[1] = b.box_lo[1] + uint32_t(r % b.box_size[1]);
+        c[0] = b.box_lo[0] + uint32_t(r / b.box_size[1]);
+    }
+    uint64_t const oo = c[0] * b.out_str[0] + c[1] * b.out_str[1] + c[2] * b.out_str[2] + c[3];
+    // Workgroup-level culling on values that are uniform over the workgroup (scalar unit):
+    // when its 256 vectors lie in one row, an item whose window misses that row or that
+    // column range is skipped without any per-lane work.
+    uint64_t const first = uint64_t(blockIdx.x) * 256;
+    uint64_t const last = (first + 255 < b.n_vec ? first + 255 : b.n_vec - 1);
+    bool const     one_row = first / vpr == last / vpr;
+    uint32_t       u[3] = {0, 0, 0};
+    uint32_t       col_lo = 0, col_hi = 0;
+    if (one_row) {
+        uint64_t r = first;
+        col_lo = b.box_lo[3] + uint32_t(r % vpr) * V;
+        col_hi = b.box_lo[3] + uint32_t(last % vpr) * V + V;
+        r /= vpr;
+        u[2] = b.box_lo[2] + uint32_t(r % b.box_size[2]);
+        r /= b.box_size[2];
+        u[1] = b.box_lo[1] + uint32_t(r % b.box_size[1]);
+        u[0] = b.box_lo[0] + uint32_t(r / b.box_size[1]);
+    }
+    vt   val;
+    bool have = false;
+    // fully unrolled so that every item is read from the kernel arguments at a fixed offset
+    // (scalar loads); a dynamic index would make each thread copy the argument block to scratch
+#pragma unroll
+    for (int t = 0; t != TOUCH_BATCH_MAX; ++t) {
+        if (t >= b.n) break;
+        touch_item_t const& it = b.items[t];
+        if (one_row && !(u[0] - it.lo[0] < it.size[0] && u[1] - it.lo[1] < it.size[1] &&
+                         u[2] - it.lo[2] < it.size[2] && col_lo < it.lo[3] + it.size[3] &&
+                         col_hi > it.lo[3])) {
+            continue;
+        }
+        uint32_t d0 = c[0] - it.lo[0], d1 = c[1] - it.lo[1], d2 = c[2] - it.lo[2];
+        // columns [c3, c3 + V) against the window [lo3, lo3 + size3)
+        bool cols = c[3] < it.lo[3] + it.size[3] && c[3] + V > it.lo[3];
+        if (d0 < it.size[0] && d1 < it.size[1] && d2 < it.size[2] && cols) {
+            uint64_t const row = it.base_inn + d0 * it.str_inn[0] + d1 * it.str_inn[1] +
+                                 d2 * it.str_inn[2];
+            T const* const src = static_cast<T const*>(it.inn) + row;
+            vt   x;
+            bool in[V];
+            bool full = true;
+            if constexpr (ALIGNED) {
+                x = *reinterpret_cast<vt const*>(src + (c[3] - it.lo[3]));
+#pragma unroll
+                for (int j = 0; j != V; ++j) in[j] = true;
+            } else {
+#pragma unroll
+                for (int j = 0; j != V; ++j) {
+                    uint32_t d3 = c[3] + uint32_t(j) - it.lo[3];
+                    in[j] = d3 < it.size[3];
+                    full = full && in[j];
+                    if (in[j]) x.v[j] = src[d3];
+                }
+            }
+            if (!have && (it.op != OP_COPY || !full)) val = *reinterpret_cast<vt const*>(out + oo);
+#pragma unroll
+            for (int j = 0; j != V; ++j) {
+                if (!in[j]) continue;
+                switch (it.op) {
+                    case OP_COPY:
+                        val.v[j] = x.v[j];
+                        break;
+                    case OP_ADD:
+                        val.v[j] = apply<OP_ADD, T>(val.v[j], x.v[j]);
+                        break;
+                    case OP_MUL:
+                        val.v[j] = apply<OP_MUL, T>(val.v[j], x.v[j]);
+                        break;
+                    case OP_MIN:
+                        if constexpr (!(sizeof(T) == 8 && alignof(T) == 4)) {
+                            val.v[j] = apply<OP_MIN, T>(val.v[j], x.v[j]);
+                        }
+                        break;
+                    default:
+                        if constexpr (!(sizeof(T) == 8 && alignof(T) == 4)) {
+                            val.v[j] = apply<OP_MAX, T>(val.v[j], x.v[j]);
+                        }
+                        break;
+                }
+            }
+            have = true;
+        }
+    }
+    if (have) *reinterpret_cast<vt*>(out + oo) = val;
+}
+
+template <typename T>
+void launch_touch_batch_t(touch_batch_t const& b, hipStream_t stream, void* out)
+{
+    constexpr int VMAX = 16 / sizeof(T);
+    unsigned      blocks = unsigned((b.n_vec + 255) / 256);
+    if (b.vec == VMAX && b.aligned) {
+        hipLaunchKernelGGL((touch_batch_kernel<T, VMAX, true>), dim3(blocks), dim3(256), 0, stream,
+                           b, static_cast<T*>(out));
+    } else if (b.vec == VMAX) {
+        hipLaunchKernelGGL((touch_batch_kernel<T, VMAX, false>), dim3(blocks), dim3(256), 0,
+                           stream, b, static_cast<T*>(out));
+    } else {
+        hipLaunchKernelGGL((touch_batch_kernel<T, 1, true>), dim3(blocks), dim3(256), 0, stream, b,
+                           static_cast<T*>(out));
+    }
+}
+
 // ---- fills
 
 template <int V>
@@ -265,6 +392,32 @@ void launch_touch(touch_launch_t const& a, int elem_size, int dtype_code, int op
         default:
             if (op == OP_ADD) return launch_touch_t<c64_t, OP_ADD>(a, stream, out, inn);
             return launch_touch_t<c64_t, OP_MUL>(a, stream, out, inn);
+    }
+}
+
+void launch_touch_batch(touch_batch_t const& b, int elem_size, int dtype_code, hipStream_t stream,
+                        void* out)
+{
+    if (b.n == 0 || b.n_vec == 0) return;
+    if (!b.any_castable) {
+        switch (elem_size) {
+            case 2:
+                return launch_touch_batch_t<uint16_t>(b, stream, out);
+            case 4:
+                return launch_touch_batch_t<uint32_t>(b, stream, out);
+            default:
+                return launch_touch_batch_t<uint64_t>(b, stream, out);
+        }
+    }
+    switch (dtype_code) {
+        case 0:
+            return launch_touch_batch_t<_Float16>(b, stream, out);
+        case 1:
+            return launch_touch_batch_t<float>(b, stream, out);
+        case 2:
+            return launch_touch_batch_t<double>(b, stream, out);
+        default:
+            return launch_touch_batch_t<c64_t>(b, stream, out);
     }
 }
 

@@ -1,5 +1,184 @@
+// N-D permute whose innermost mode changes (a true transposition), through LDS tiles.
+//
+// A permutation einsummable (one input, identity join, no aggregation, no broadcast;
+// einsummable_t::is_permutation, src/einsummable/einsummable.cc:740-743) that keeps its
+// innermost mode is a strided row copy and is handled by the generated elementwise kernel.
+// When the innermost mode of the input is not the innermost mode of the output, a direct
+// copy is uncoalesced on one side.  Here a 64 x 64 tile over (input-inner mode, output-inner
+// mode) goes through LDS: rows are read along the input's contiguous mode and written along
+// the output's contiguous mode, so both sides move whole 128..512-byte row segments.  All
+// other modes form the batch.  Pure data movement: results are bit-identical to the CPU's
+// permute_t (src/base/permute_.h) and to the interpreter.
 #include "kernel_manager.h"
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+
 namespace es
 {
-std::shared_ptr<plan_t> plan_transpose(einsummable_t const&, int) { return nullptr; }
+namespace
+{
+
+constexpr int TT = 64;      // tile edge
+constexpr int MAXB = 6;     // batch modes
+
+struct transpose_args_t {
+    void const* in;
+    void*       out;
+    uint32_t    n_i, n_o;           // extents of the input-inner and output-inner modes
+    int64_t     so_i;               // output stride of the input-inner mode
+    int64_t     si_o;               // input stride of the output-inner mode
+    uint32_t    tiles_i, tiles_o;
+    uint64_t    n_blocks;
+    uint32_t    nb;                 // number of batch modes
+    uint32_t    bsize[MAXB];        // innermost batch mode first
+    int64_t     bsi[MAXB], bso[MAXB];
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_kernel(transpose_args_t a)
+{
+    // pitch chosen odd in 4-byte words so that the column reads spread over all banks
+    constexpr int PITCH = sizeof(T) == 2 ? TT + 2 : TT + 1;
+    __shared__ T tile[TT][PITCH];
+
+    uint32_t const lane = threadIdx.x & 63;
+    uint32_t const wave = threadIdx.x >> 6;
+    uint64_t const linear = uint64_t(blockIdx.y) * gridDim.x + blockIdx.x;
+    if (linear >= a.n_blocks) return;  // uniform over the workgroup
+    uint32_t t = uint32_t(linear);
+    uint32_t const ti = t % a.tiles_i;
+    t /= a.tiles_i;
+    uint32_t const to = t % a.tiles_o;
+    uint32_t bidx = t / a.tiles_o;
+
+    int64_t off_i = 0, off_o = 0;
+#pragma unroll
+    for (int d = 0; d != MAXB; ++d) {
+        if (d < int(a.nb)) {
+            uint32_t q = bidx / a.bsize[d];
+            uint32_t r = bidx - q * a.bsize[d];
+            off_i += int64_t(r) * a.bsi[d];
+            off_o += int64_t(r) * a.bso[d];
+            bidx = q;
+        }
+    }
+    T const* const in = static_cast<T const*>(a.in) + off_i;
+    T* const       out = static_cast<T*>(a.out) + off_o;
+    uint32_t const i0 = ti * TT, o0 = to * TT;
+
+    // rows of the tile along the input's contiguous mode
+#pragma unroll
+    for (int rr = 0; rr != TT / 4; ++rr) {
+        uint32_t o = o0 + wave * (TT / 4) + rr;
+        uint32_t i = i0 + lane;
+        if (o < a.n_o && i < a.n_i) tile[wave * (TT / 4) + rr][lane] = in[int64_t(o) * a.si_o + i];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int rr = 0; rr != TT / 4; ++rr) {
+        uint32_t i = i0 + wave * (TT / 4) + rr;
+        uint32_t o = o0 + lane;
+        if (i < a.n_i && o < a.n_o) out[int64_t(i) * a.so_i + o] = tile[lane][wave * (TT / 4) + rr];
+    }
+}
+
+struct transpose_plan_t : plan_t {
+    transpose_args_t args;
+    int              elem_size;
+    uint64_t         blocks;
+
+    void run(hipStream_t stream, void* out, void const* const* inns, void*, uint64_t) const override
+    {
+        transpose_args_t a = args;
+        a.in = inns[0];
+        a.out = out;
+        a.n_blocks = blocks;
+        // a grid dimension times the block size must stay below 2^32
+        unsigned gx = unsigned(std::min<uint64_t>(blocks, 1ull << 22));
+        unsigned gy = unsigned((blocks + gx - 1) / gx);
+        dim3     grid(gx, gy), block(256);
+        switch (elem_size) {
+            case 2:
+                hipLaunchKernelGGL((transpose_kernel<uint16_t>), grid, block, 0, stream, a);
+                break;
+            case 4:
+                hipLaunchKernelGGL((transpose_kernel<uint32_t>), grid, block, 0, stream, a);
+                break;
+            default:
+                hipLaunchKernelGGL((transpose_kernel<uint64_t>), grid, block, 0, stream, a);
+                break;
+        }
+        hipError_t err = hipGetLastError();
+        if (err != hipSuccess) {
+            throw km_error(km_status::device,
+                           std::string("transpose launch: ") + hipGetErrorString(err));
+        }
+    }
+};
+
+}  // namespace
+
+std::shared_ptr<plan_t> plan_transpose(einsummable_t const& e, int)
+{
+    if (!e.is_permutation()) return nullptr;
+    int const R = e.out_rank;
+    if (R < 2) return nullptr;
+    std::vector<int> const& inn = e.inns[0];
+    int const mode_i = inn.back();  // contiguous in the input
+    int const mode_o = R - 1;       // contiguous in the output
+    if (mode_i == mode_o) return nullptr;  // inner mode preserved: a row copy, not a transpose
+    if (R - 2 > MAXB) return nullptr;
+
+    auto in_stride = [&](int m) {
+        int64_t s = 1;
+        for (int k = int(inn.size()) - 1; k >= 0; --k) {
+            if (inn[k] == m) return s;
+            s *= int64_t(e.join_shape[inn[k]]);
+        }
+        return int64_t(0);
+    };
+    auto out_stride = [&](int m) {
+        int64_t s = 1;
+        for (int k = R - 1; k > m; --k) s *= int64_t(e.join_shape[k]);
+        return s;
+    };
+    if (e.out_nelem() >= (1ull << 40)) return nullptr;
+    for (uint64_t d : e.join_shape) {
+        if (d >= (1ull << 31)) return nullptr;
+    }
+
+    auto p = std::make_shared<transpose_plan_t>();
+    transpose_args_t& a = p->args;
+    a.in = nullptr;
+    a.out = nullptr;
+    a.n_i = uint32_t(e.join_shape[mode_i]);
+    a.n_o = uint32_t(e.join_shape[mode_o]);
+    a.so_i = out_stride(mode_i);
+    a.si_o = in_stride(mode_o);
+    a.tiles_i = (a.n_i + TT - 1) / TT;
+    a.tiles_o = (a.n_o + TT - 1) / TT;
+    a.nb = 0;
+    uint64_t batch = 1;
+    for (int d = 0; d != MAXB; ++d) {
+        a.bsize[d] = 1;
+        a.bsi[d] = a.bso[d] = 0;
+    }
+    for (int m = R - 1; m >= 0; --m) {
+        if (m == mode_i || m == mode_o) continue;
+        a.bsize[a.nb] = uint32_t(e.join_shape[m]);
+        a.bsi[a.nb] = in_stride(m);
+        a.bso[a.nb] = out_stride(m);
+        batch *= e.join_shape[m];
+        ++a.nb;
+    }
+    p->blocks = uint64_t(a.tiles_i) * a.tiles_o * batch;
+    if (p->blocks >= (1ull << 31) || batch >= (1ull << 31)) return nullptr;
+    p->elem_size = int(dtype_size(e.out_dtype()));
+    p->workspace_bytes = 0;
+    p->description = "transpose_lds tile=64x64 batch=" + std::to_string(batch);
+    return p;
+}
+
 }  // namespace es

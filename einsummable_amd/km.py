@@ -18,6 +18,7 @@ EXPORTS = [
     "es_km_execute",
     "es_km_describe",
     "es_km_touch",
+    "es_km_touch_batch",
     "es_km_fill_constant",
     "es_km_fill_lowertri",
     "es_km_codegen_source",
@@ -81,6 +82,17 @@ def load_library():
         ctypes.c_void_p,
         ctypes.c_int,
         ctypes.c_char,
+        ctypes.c_int,
+        ctypes.c_void_p,
+        ctypes.c_void_p,
+        ctypes.c_void_p,
+    ]
+    lib.es_km_touch_batch.argtypes = [
+        ctypes.c_void_p,
+        ctypes.c_int,
+        ctypes.c_void_p,
+        ctypes.c_void_p,
+        ctypes.c_char_p,
         ctypes.c_int,
         ctypes.c_void_p,
         ctypes.c_void_p,
@@ -191,6 +203,18 @@ class Touch:
         self._dims = (ctypes.c_uint64 * len(flat))(*flat)
 
 
+class TouchBatch:
+    """Flattened descriptors of a list of Touch objects (built once, reused per call)."""
+
+    def __init__(self, touches):
+        flat = [v for t in touches for d in t.selection for v in d]
+        self.n = len(touches)
+        self.dtype = touches[0].dtype if touches else F32
+        self.dims = (ctypes.c_uint64 * max(len(flat), 1))(*flat)
+        self.ranks = (ctypes.c_int * max(self.n, 1))(*[len(t.selection) for t in touches])
+        self.castables = b"".join(_castable_char(t.castable) for t in touches) + b"\0"
+
+
 def codegen_source(e, compile=False):
     lib = load_library()
     buf = ctypes.create_string_buffer(1 << 16)
@@ -289,6 +313,16 @@ class KernelManager:
         rc = self._lib.es_km_touch(self._h, ctypes.cast(t._dims, ctypes.c_void_p),
                                    len(t.selection), _castable_char(t.castable), t.dtype, stream,
                                    out, inn)
+        if rc != OK:
+            self._fail(rc)
+
+    def touch_batch(self, touches, stream, out, inns):
+        """Apply `touches` (all into `out`) in list order with one launch per 32 touches."""
+        batch = TouchBatch(touches) if not isinstance(touches, TouchBatch) else touches
+        ptrs = (ctypes.c_void_p * max(len(inns), 1))(*inns)
+        rc = self._lib.es_km_touch_batch(self._h, batch.n, ctypes.cast(batch.dims, ctypes.c_void_p),
+                                         ctypes.cast(batch.ranks, ctypes.c_void_p),
+                                         batch.castables, batch.dtype, stream, out, ptrs)
         if rc != OK:
             self._fail(rc)
 

@@ -93,6 +93,19 @@ int es_km_describe(es_km_t* km, const uint64_t* join_shape, int join_rank, const
 int es_km_touch(es_km_t* km, const uint64_t* touchdims, int rank, char castable, int dtype,
                 void* stream, void* out, const void* inn);
 
+/* A group of touches into ONE output tensor in one call (one launch per 32 touches): the
+ * result is bit-identical to calling es_km_touch on each, in list order, including where
+ * windows overlap.  touchdims holds the selections back to back (ranks[i] x 5 values each),
+ * castables[i] is '+','x','v','^' or 0, inns[i] the input of touch i.  All touches share the
+ * dtype, the rank and the output extents.  No counterpart in the reference, whose engine
+ * issues the touches of a group one by one (src/engine/gpu/exec_graph.cc:354-404); offered
+ * because a partialize unit's inputs all hit the same output region
+ * (src/einsummable/taskgraph.cc:3224-3266) and each launch otherwise costs more than the
+ * copy it performs. */
+int es_km_touch_batch(es_km_t* km, int n_touches, const uint64_t* touchdims, const int* ranks,
+                      const char* castables, int dtype, void* stream, void* out,
+                      const void* const* inns);
+
 /* void constant_fill(fill_t::constant_t const&, cudaStream_t, void* out) const
  *                                                               gpu_kernel_manager.h:321
  * value_bits: the scalar's bytes, little-endian, in the low bytes of a uint64

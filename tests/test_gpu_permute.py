@@ -1,0 +1,56 @@
+"""N-D permutes through the C ABI, bit-exact against numpy's transpose and the oracle
+(procedure of exps/cpuexec_permute.cc:33-77: every permutation of a 10x11x12x130 iota tensor
+compared exactly with the interpreter)."""
+import itertools
+
+import numpy as np
+import pytest
+
+import einsummable_amd as ea
+import oracle
+from helpers import NP, assert_bits_equal, normal, rng, run_einsummable
+
+pytestmark = pytest.mark.gpu
+
+
+def permute_einsummable(in_shape, perm, dt):
+    """out mode z is input mode perm[z] (numpy.transpose convention)."""
+    out_shape = [in_shape[p] for p in perm]
+    inn = [perm.index(i) for i in range(len(in_shape))]
+    return ea.Einsummable(out_shape, [inn], len(in_shape), "hole|%s@0" % dt)
+
+
+@pytest.mark.parametrize("perm", list(itertools.permutations(range(4))))
+def test_all_permutations_of_a_4d_iota_tensor(km, perm):
+    shape = (10, 11, 12, 130)
+    t = np.arange(int(np.prod(shape)), dtype=np.float32).reshape(shape)
+    e = permute_einsummable(shape, perm, "f32")
+    got = run_einsummable(km, e, [t])
+    want = np.ascontiguousarray(np.transpose(t, perm)).reshape(-1)
+    assert_bits_equal(got, want, "permute %s [%s]" % (perm, km.describe(e)))
+
+
+@pytest.mark.parametrize("dt,npdt", [("f16", np.float16), ("f64", np.float64), ("c64", np.complex64)])
+def test_transposes_of_other_widths_and_ragged_tiles(km, dt, npdt):
+    r = rng(50)
+    for shape, perm in [((70, 33), (1, 0)), ((64, 64), (1, 0)), ((1, 200), (1, 0)),
+                        ((5, 65, 67), (2, 1, 0)), ((3, 4, 129, 2), (3, 0, 2, 1)),
+                        ((257, 3, 66), (2, 0, 1))]:
+        x = normal(r, int(np.prod(shape)), npdt).reshape(shape)
+        e = permute_einsummable(shape, perm, dt)
+        got = run_einsummable(km, e, [x])
+        want = np.ascontiguousarray(np.transpose(x, perm)).reshape(-1)
+        assert_bits_equal(got, want, "permute %s %s" % (shape, perm))
+        od, _ = oracle.scalarop_info(e.join)
+        ref = oracle.einsummable(e.join_shape, e.inns, e.out_rank, e.join, None, [x])
+        assert_bits_equal(ref, want, "oracle permute")
+
+
+def test_kernel_choice(km):
+    # innermost mode preserved: generated row copy; innermost mode changed: LDS transpose
+    e1 = permute_einsummable((8, 16, 4, 64), (0, 2, 1, 3), "f16")
+    e2 = permute_einsummable((8, 16, 4, 64), (0, 3, 2, 1), "f16")
+    km.build(e1)
+    km.build(e2)
+    assert km.describe(e1).startswith("elementwise")
+    assert km.describe(e2).startswith("transpose_lds")

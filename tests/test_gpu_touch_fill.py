@@ -119,3 +119,66 @@ def test_lowertri_fill(km, dt):
         # closed form (src/einsummable/fill.h:17-19)
         i, j = np.indices((nrow, ncol))
         assert np.array_equal(np.isinf(want), ~(i - start >= j))
+
+
+def _apply_sequentially(touches, blocks, out0):
+    ref = out0.copy()
+    for t, blk in zip(touches, blocks):
+        oracle.touch(t.selection, t.castable, ref, blk)
+    return ref
+
+
+@pytest.mark.parametrize("dt", [ea.F16, ea.F32, ea.C64])
+def test_touch_batch_equals_sequential_touches(km, dt):
+    """One call for a whole group of touches into the same output: bit-identical to applying
+    them one by one in list order, also where windows overlap and castables are mixed."""
+    r = rng(40 + dt)
+    for rank, aligned in ((1, True), (2, True), (2, False), (3, False), (4, True)):
+        d_out = [int(r.randint(6, 14)) for _ in range(rank)]
+        if aligned:
+            d_out[-1] = 8 * int(r.randint(4, 9))
+        touches, blocks = [], []
+        for _ in range(int(r.randint(1, 70))):
+            dims = []
+            for i, do in enumerate(d_out):
+                q = 8 if (aligned and i == rank - 1) else 1
+                size = q * int(r.randint(1, do // q + 1))
+                off_o = q * int(r.randint(0, (do - size) // q + 1))
+                off_i = q * int(r.randint(0, 3))
+                dims.append((size + off_i + q * int(r.randint(0, 2)), do, off_i, off_o, size))
+            castable = [None, "+", "x", "v", "^"][int(r.randint(0, 5 if dt != ea.C64 else 3))]
+            touches.append(ea.Touch(dims, castable, dt))
+            blocks.append(normal(r, int(np.prod([d[0] for d in dims])), NP[dt], 0.5))
+        out0 = normal(r, int(np.prod(d_out)), NP[dt], 0.5)
+        want = _apply_sequentially(touches, blocks, out0)
+        d_out_t = to_device(out0)
+        d_blocks = [to_device(b) for b in blocks]
+        km.touch_batch(touches, stream_handle(), d_out_t.data_ptr(), [b.data_ptr() for b in d_blocks])
+        assert_bits_equal(to_host(d_out_t, NP[dt]), want, "touch batch rank %d" % rank)
+
+
+def test_touch_batch_memory_movement_configuration(km):
+    """The 64 accumulate touches of 512x512 blocks into a zeroed 4096x4096 f16 matrix as one
+    batch, against the sequential oracle."""
+    r = rng(41)
+    n, b, count = 4096, 512, 64
+    touches, blocks = [], []
+    for _ in range(count):
+        ro, co = int(r.randint(0, n - b + 1)), int(r.randint(0, n - b + 1))
+        touches.append(ea.Touch([(b, n, 0, ro, b), (b, n, 0, co, b)], "+", ea.F16))
+        blocks.append(normal(r, b * b, np.float16))
+    want = _apply_sequentially(touches, blocks, np.zeros(n * n, np.float16))
+    d_out = empty_device(n * n, np.float16, 0.0)
+    d_blocks = [to_device(x) for x in blocks]
+    km.touch_batch(touches, stream_handle(), d_out.data_ptr(), [x.data_ptr() for x in d_blocks])
+    assert_bits_equal(to_host(d_out, np.float16), want, "64 accumulate touches, batched")
+
+
+def test_touch_batch_errors(km):
+    d = to_device(np.zeros(64, np.float32))
+    a = ea.Touch([(4, 8, 0, 0, 4)], None, ea.F32)
+    b = ea.Touch([(4, 16, 0, 0, 4)], None, ea.F32)     # another output extent
+    with pytest.raises(ea.KmError) as ei:
+        km.touch_batch([a, b], 0, d.data_ptr(), [d.data_ptr(), d.data_ptr()])
+    assert ei.value.code == -1
+    km.touch_batch([], 0, d.data_ptr(), [])
