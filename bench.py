@@ -43,7 +43,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="all",
-                    choices=["c2", "c1", "c3", "c4", "c5", "llama", "copy", "all"])
+                    choices=["c2", "c1", "c3", "c4", "c5", "llama", "copy", "mfma_peak", "all"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     return ap.parse_args()
 
@@ -216,6 +216,27 @@ def run_c3(km, steps, warmup):
                 "bytes": nbytes, "ms": round(ms, 5), "GBps": round(nbytes / ms / 1e6, 1),
                 "hbm_frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4)})
     del x, y
+    # (a') a permute that changes the innermost mode (not part of the configuration; shows the
+    # LDS-tiled transpose): ba->ab of an 8192 x 8192 f16 matrix
+    n2 = 8192
+    e = ea.Einsummable([n2, n2], [[1, 0]], 2, "hole|f16@0")
+    x = torch.randn(n2, n2, device="cuda", dtype=torch.float16)
+    y = torch.empty_like(x)
+    assert km.build(e) == 0
+    call = lambda: km(e, stream, y.data_ptr(), [x.data_ptr()])
+    for _ in range(warmup):
+        call()
+    torch.cuda.synchronize()
+    t = Timed()
+    for _ in range(steps):
+        t.record(call)
+    torch.cuda.synchronize()
+    nbytes = 2 * x.numel() * 2
+    ms = t.mean_ms()
+    out.append({"node": "transpose ba->ab f16 8192x8192", "kernel": km.describe(e),
+                "bytes": nbytes, "ms": round(ms, 5), "GBps": round(nbytes / ms / 1e6, 1),
+                "hbm_frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4)})
+    del x, y
     # (b) 64 accumulate touches of 512x512 into random windows of a zeroed 4096x4096 matrix
     n, blk, count = 4096, 512, 64
     r = np.random.RandomState(0)
@@ -347,6 +368,26 @@ def run_c5(km, steps, warmup):
             "top_nodes": [{"label": l, "ms": round(ms, 4)} for l, _, ms, _ in top]}
 
 
+def run_mfma_peak(km):
+    """fp16 matrix-core throughput with operands in registers (no memory traffic at all): the
+    ceiling a GEMM can approach on this device, for zero and for random operand bits."""
+    import torch
+
+    out = {}
+    stream = torch.cuda.current_stream().cuda_stream
+    blocks = 1024
+    scratch = torch.empty(blocks * 256, device="cuda", dtype=torch.float32)
+    for label, ops in (("zeros", torch.zeros(4096, device="cuda", dtype=torch.float16)),
+                       ("random", torch.rand(4096, device="cuda", dtype=torch.float16) - 0.5)):
+        best = 0.0
+        for _ in range(3):
+            best = max(best, km.probe_mfma_f16(ops.data_ptr(), scratch.data_ptr(), blocks, 20000,
+                                               stream))
+        out[label + "_TFLOPs"] = round(best, 1)
+    out["published_peak_TFLOPs"] = PEAK_TFLOPS["f16"]
+    return out
+
+
 def run_copy(km, steps, warmup):
     """A plain copy of known size (1-D touch without castable, 512 MiB in, 512 MiB out): the
     yardstick the FETCH_SIZE / WRITE_SIZE counters are scaled by."""
@@ -388,6 +429,9 @@ def main():
     torch.cuda.init()
     km = ea.KernelManager(0)
 
+    if args.workload == "mfma_peak":
+        print(json.dumps(run_mfma_peak(km)))
+        return
     if args.workload == "copy":
         print(json.dumps(run_copy(km, args.steps, args.warmup)))
         return
@@ -413,6 +457,8 @@ def main():
         torch.cuda.empty_cache()
         others["c5"] = run_c5(km, max(args.steps // 5, 3), max(args.warmup // 5, 1))
         torch.cuda.empty_cache()
+    if args.workload == "all":
+        others["mfma_f16_register_ceiling"] = run_mfma_peak(km)
     if args.workload in ("llama", "all"):
         others["llama7b_contractions"] = run_llama_contractions(km, max(args.steps // 5, 3),
                                                                 max(args.warmup // 5, 1))

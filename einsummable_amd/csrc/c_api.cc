@@ -4,6 +4,7 @@
 #include "../../include/es_km.h"
 
 #include "codegen.h"
+#include "gemm_kernel.h"
 #include "kernel_manager.h"
 
 #include <cstring>
@@ -341,5 +342,13 @@ int es_km_touch_batch(es_km_t* h, int n_touches, const uint64_t* touchdims, cons
         h->km->touch_batch(ts, static_cast<hipStream_t>(stream), out, ptrs);
         return ES_KM_OK;
     });
+}
+
+double es_km_probe_mfma_f16(es_km_t* h, const void* operands, void* scratch, int blocks, int iters,
+                            void* stream)
+{
+    if (!h || !operands || !scratch || blocks < 1 || iters < 1) return -1.0;
+    return es::gemm::probe_mfma_f16(operands, scratch, blocks, iters,
+                                    static_cast<hipStream_t>(stream));
 }
 }

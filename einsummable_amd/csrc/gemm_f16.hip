@@ -16,5 +16,56 @@ void launch_gemm_f16(int bm, int bn, gemm_args_t const& a, hipStream_t stream)
     if (!done) launch_gemm_kernel<T, 128, 128, -1, -1>(a, stream);
 }
 
+// Measurement aid: matrix-core throughput with register-resident operands, i.e. the ceiling
+// any fp16 GEMM on this device can approach.  With operands of random bits the cores draw more
+// power than with zeros and the clock drops, so both are reported.
+__global__ __launch_bounds__(256) void mfma_probe_kernel(chunk_t const* in, float* out, int iters)
+{
+    half8_t   x = __builtin_bit_cast(half8_t, in[threadIdx.x]);
+    half8_t   y = __builtin_bit_cast(half8_t, in[threadIdx.x + 256]);
+    float16_t acc[8];
+#pragma unroll
+    for (int i = 0; i != 8; ++i) {
+#pragma unroll
+        for (int e = 0; e != 16; ++e) acc[i][e] = 0;
+    }
+    for (int it = 0; it != iters; ++it) {
+#pragma unroll
+        for (int i = 0; i != 8; ++i) {
+            acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(x, y, acc[i], 0, 0, 0);
+        }
+    }
+    float s = 0;
+#pragma unroll
+    for (int i = 0; i != 8; ++i) {
+#pragma unroll
+        for (int e = 0; e != 16; ++e) s += acc[i][e];
+    }
+    out[blockIdx.x * 256 + threadIdx.x] = s;
+}
+
+// Returns TFLOP/s, or a negative value on a device error.  `operands`: 512 x 16 bytes on the
+// device; `scratch`: blocks x 256 floats.
+double probe_mfma_f16(void const* operands, void* scratch, int blocks, int iters,
+                      hipStream_t stream)
+{
+    hipEvent_t e0, e1;
+    if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) return -1.0;
+    hipLaunchKernelGGL(mfma_probe_kernel, dim3(blocks), dim3(256), 0, stream,
+                       static_cast<chunk_t const*>(operands), static_cast<float*>(scratch), 64);
+    hipEventRecord(e0, stream);
+    hipLaunchKernelGGL(mfma_probe_kernel, dim3(blocks), dim3(256), 0, stream,
+                       static_cast<chunk_t const*>(operands), static_cast<float*>(scratch), iters);
+    hipEventRecord(e1, stream);
+    float ms = 0;
+    bool  ok = hipEventSynchronize(e1) == hipSuccess &&
+              hipEventElapsedTime(&ms, e0, e1) == hipSuccess && ms > 0;
+    hipEventDestroy(e0);
+    hipEventDestroy(e1);
+    if (!ok) return -1.0;
+    double flop = double(blocks) * 4.0 * double(iters) * 8.0 * 32768.0;
+    return flop / (double(ms) * 1e-3) / 1e12;
+}
+
 }  // namespace gemm
 }  // namespace es

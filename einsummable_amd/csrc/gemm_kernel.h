@@ -830,6 +830,8 @@ __global__ __launch_bounds__(256) void gemm_fast_kernel(gemm_args_t a)
 void launch_gemm_f16(int bm, int bn, gemm_args_t const& a, hipStream_t stream);
 void launch_gemm_f32(int bm, int bn, gemm_args_t const& a, hipStream_t stream);
 void launch_gemm_f64(int bm, int bn, gemm_args_t const& a, hipStream_t stream);
+double probe_mfma_f16(void const* operands, void* scratch, int blocks, int iters,
+                      hipStream_t stream);
 // whether launch_gemm_* has a specialised kernel for this tile
 bool gemm_has_tile(int elem_size, int bm, int bn);
 

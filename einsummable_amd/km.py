@@ -24,6 +24,7 @@ EXPORTS = [
     "es_km_codegen_source",
     "es_km_scalarop_roundtrip",
     "es_km_merge_adjacent_dims",
+    "es_km_probe_mfma_f16",
 ]
 
 
@@ -117,6 +118,9 @@ def load_library():
         ctypes.c_void_p,
         ctypes.c_void_p,
     ]
+    lib.es_km_probe_mfma_f16.restype = ctypes.c_double
+    lib.es_km_probe_mfma_f16.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                         ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
     lib.es_km_codegen_source.argtypes = desc + [ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t]
     lib.es_km_scalarop_roundtrip.argtypes = [ctypes.c_char_p, ctypes.c_void_p, ctypes.c_size_t,
                                              ctypes.c_void_p, ctypes.c_void_p]
@@ -325,6 +329,9 @@ class KernelManager:
                                          batch.castables, batch.dtype, stream, out, ptrs)
         if rc != OK:
             self._fail(rc)
+
+    def probe_mfma_f16(self, operands, scratch, blocks, iters, stream):
+        return self._lib.es_km_probe_mfma_f16(self._h, operands, scratch, blocks, iters, stream)
 
     def constant_fill(self, dtype, value_bits, nelem, stream, out):
         rc = self._lib.es_km_fill_constant(self._h, dtype, value_bits, nelem, stream, out)

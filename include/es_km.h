@@ -142,6 +142,14 @@ int es_km_merge_adjacent_dims(const uint64_t* join_shape, int join_rank, const i
                               int* new_inns_flat, int* new_inns_offsets, int* new_out_rank,
                               char* str_out, size_t str_cap);
 
+/* Measurement aid (no counterpart in the reference): fp16 matrix-core throughput in TFLOP/s
+ * with register-resident operands -- `blocks` workgroups of 4 wavefronts each issue
+ * 8 * iters v_mfma_f32_32x32x16_f16.  operands: 8 KiB on the device (their bit patterns set
+ * the power draw, hence the clock); scratch: blocks * 1 KiB on the device.  Synchronises the
+ * stream.  Negative on error. */
+double es_km_probe_mfma_f16(es_km_t* km, const void* operands, void* scratch, int blocks, int iters,
+                            void* stream);
+
 #ifdef __cplusplus
 }
 #endif
