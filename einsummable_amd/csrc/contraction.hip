@@ -20,6 +20,7 @@
 // four consecutive n of one m: the epilogue stores them with one 8 / 16-byte write.
 // fp16 inputs accumulate in fp32 (v_mfma_f32_32x32x16_f16), fp32 uses v_mfma_f32_32x32x2_f32,
 // f64 uses v_mfma_f64_16x16x4_f64.
+#include "gemm_dma_kernel.h"
 #include "gemm_kernel.h"
 #include "kernel_manager.h"
 
@@ -61,30 +62,56 @@ void fill_group(group_t& g, std::vector<mode_info_t> const& ms,
     }
 }
 
-// Macro tile for a problem.  128x128 tiles keep two workgroups per compute unit, which hide
-// each other's slice boundaries; 256x256 tiles halve the LDS and L2 traffic per flop but run
-// one wave per SIMD, so they only pay when there are several full rounds of them over the
-// 256 compute units (measured crossover on MI355X: ~3 rounds).
-// ES_KM_GEMM_TILE=128x128|256x256 overrides the choice (tuning aid).
-void choose_tile(dtype_t dt, uint64_t M, uint64_t N, uint64_t K, uint64_t batch, int& bm, int& bn)
+// Macro tile for a problem.  Larger tiles cost less LDS and L1 traffic per flop, which is what
+// limits the kernels (measured full-chip rates on MI355X, fp16: 256x256 ~1.2 PFLOP/s,
+// 128x256 ~0.98, 128x128 ~0.8), but there are fewer of them to spread over the 256 compute
+// units.  The estimate below is rounds of resident workgroups times the time of one tile.
+// ES_KM_GEMM_TILE=128x128|128x256|256x128|256x256 overrides the choice (tuning aid).
+struct tile_option_t {
+    int    bm, bn;
+    int    per_cu;  // workgroups resident on one compute unit
+    double eff;     // relative rate of one compute unit running this tile
+};
+
+void choose_tile(dtype_t dt, uint64_t M, uint64_t N, uint64_t K, uint64_t batch, bool dma_ok,
+                 int& bm, int& bn)
 {
     bm = 128;
     bn = 128;
     if (dt == dtype_t::f64) return;
     if (const char* env = std::getenv("ES_KM_GEMM_TILE")) {
         int x = 0, y = 0;
-        if (std::sscanf(env, "%dx%d", &x, &y) == 2 && x == y && (x == 128 || x == 256)) {
-            bm = x;
-            bn = y;
+        if (std::sscanf(env, "%dx%d", &x, &y) == 2 && (x == 128 || x == 256) &&
+            (y == 128 || y == 256)) {
+            // rectangular tiles exist in the direct-to-LDS kernel only
+            if (x == y || dma_ok) {
+                bm = x;
+                bn = y;
+            }
             return;
         }
     }
-    // short reductions are bound by the output write, narrow outputs waste a wide tile
-    if (K < 1024 || M < 512 || N < 512) return;
-    uint64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256) * batch;
-    if (big_tiles >= 768) {
-        bm = 256;
-        bn = 256;
+    // short reductions are bound by the output write: small tiles, several per compute unit
+    if (K < 512) return;
+    if (!dma_ok) {
+        // register-staged 256x256 kernel: only pays with several full rounds of tiles
+        uint64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256) * batch;
+        if (K >= 1024 && M >= 512 && N >= 512 && big_tiles >= 768) bm = bn = 256;
+        return;
+    }
+    static tile_option_t const options[] = {
+        {256, 256, 1, 1.00}, {128, 256, 1, 0.80}, {256, 128, 1, 0.78}, {128, 128, 2, 0.66}};
+    double best = 0;
+    for (tile_option_t const& o : options) {
+        uint64_t tiles = ((M + o.bm - 1) / o.bm) * ((N + o.bn - 1) / o.bn) * batch;
+        uint64_t slots = 256ull * uint64_t(o.per_cu);
+        uint64_t rounds = (tiles + slots - 1) / slots;
+        double   t = double(rounds) * o.per_cu * double(o.bm) * double(o.bn) / o.eff;
+        if (best == 0 || t < best * 0.97) {  // near ties go to the larger tile (listed first)
+            best = t;
+            bm = o.bm;
+            bn = o.bn;
+        }
     }
 }
 
@@ -233,20 +260,24 @@ std::shared_ptr<plan_t> plan_contraction(einsummable_t const& e, int)
     a.a_mode = vec_ok(js, sA, VL) ? 0 : (vec_ok(gm, sA, VL) ? 1 : 2);
     a.b_mode = vec_ok(js, sB, VL) ? 0 : (vec_ok(gn, sB, VL) ? 1 : 2);
     a.c_mode = vec_ok(gn, sC, VL) ? 3 : (vec_ok(gn, sC, 4) ? 0 : 2);
+    a.offsets_fit_32 = e.inn_nelem(0) * dtype_size(dt) < (1ull << 32) &&
+                       e.inn_nelem(1) * dtype_size(dt) < (1ull << 32);
 
     // large tiles exist for the vector load paths (A along k; B along k or n)
-    if (a.a_mode == 0 && a.b_mode != 2) choose_tile(dt, M, N, K, Bt, p->bm, p->bn);
+    bool const dma_ok = dt == dtype_t::f16 && gemm_dma_eligible<_Float16>(a);
+    if (a.a_mode == 0 && a.b_mode != 2) choose_tile(dt, M, N, K, Bt, dma_ok, p->bm, p->bn);
     a.tiles_m = uint32_t((M + p->bm - 1) / p->bm);
     a.tiles_n = uint32_t((N + p->bn - 1) / p->bn);
     if (uint64_t(a.tiles_m) * a.tiles_n >= lim) return nullptr;
 
+    bool const dma = dma_ok && (p->bm != 128 || p->bn != 128 || K < 512);
     p->workspace_bytes = 0;
     static const char* mode_name[] = {"k", "mn", "elem"};
     p->description = std::string("contraction_mfma_") + dtype_name(dt) + " tile=" +
                      std::to_string(p->bm) + "x" + std::to_string(p->bn) + " A=" +
                      mode_name[a.a_mode] + " B=" + mode_name[a.b_mode] + " C=" +
                      (a.c_mode == 3 ? "wide" : (a.c_mode == 0 ? "vec" : "elem")) +
-                     (swapped ? " swapped" : "") +
+                     (swapped ? " swapped" : "") + (dma ? " load=direct_to_lds" : "") +
                      " M=" + std::to_string(M) + " N=" + std::to_string(N) + " K=" +
                      std::to_string(K) + " batch=" + std::to_string(Bt);
     return p;

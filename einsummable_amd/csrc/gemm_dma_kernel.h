@@ -1,0 +1,346 @@
+// 256 x 256 macro-tile GEMM whose operand slices go from global memory straight into LDS
+// (global_load_lds_dwordx4), for problems where both operands are contiguous along k.
+//
+// Why a second kernel: with 128 x 128 tiles every flop costs twice the LDS and L1 traffic of a
+// 256 x 256 tile, and both are what limits the register-staged kernel.  A 256 x 256 tile per
+// workgroup of four wavefronts needs 256 accumulator registers per lane, which leaves no room
+// for register staging of the next slice; the direct-to-LDS loads need none.
+//
+//   * 4 wavefronts, 2 x 2, each owning (BM/2) x (BN/2) of C; 128 x 128 = 4 x 4 MFMA tiles =
+//     256 accumulators for the 256 x 256 tile.
+//   * LDS: NS stages of (BM + BN) rows x 64 bytes.  Loads run NS - 1 slices ahead of the
+//     matrix work; one workgroup barrier per slice.
+//   * One load instruction moves 16 rows x 64 bytes; a wavefront's 64 x 16 bytes land
+//     contiguously in LDS (lane l at +16 l), so rows cannot be padded.  Instead the four
+//     16-byte chunks of a row are XOR-swizzled with bits 2..3 of the row number, applied on
+//     the global address of the load and again on the fragment read: sixteen consecutive rows
+//     of one k-chunk then cover all 64 banks once.
+//   * The loads are written as inline assembly so that the compiler does not serialise the
+//     pipeline with a full vmcnt wait in front of every LDS read; the waits are explicit
+//     (each lane issues 8 loads per slice, so "slice kt+1 has landed" is vmcnt <= 8 x the
+//     number of younger slices in flight).
+//   * K must be a multiple of the slice (64 bytes) and at least four slices (>= NS); rows beyond M / N
+//     are clamped on load (their results are never stored).
+#pragma once
+#include "gemm_kernel.h"
+
+namespace es
+{
+namespace gemm
+{
+
+constexpr int DMA_ROW = 64;  // bytes of k per row per stage
+
+// 64 lanes x 16 bytes from `base + voff` (per lane) to LDS at `lds_addr + 16 * lane`
+__device__ __forceinline__ void load_to_lds_16(void const* base, uint32_t voff, uint32_t lds_addr)
+{
+    asm volatile(
+        "s_mov_b32 m0, %0\n\t"
+        "s_nop 0\n\t"
+        "global_load_lds_dwordx4 %1, %2"
+        :
+        : "s"(lds_addr), "v"(voff), "s"(base)
+        : "memory");  // m0 is not kept live by the compiler across statements
+}
+
+template <int VM>
+__device__ __forceinline__ void wait_loads_and_lds()
+{
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" : : "n"(VM) : "memory");
+}
+
+template <typename T, int BM, int BN, int NS>
+__global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
+{
+    using tr = traits_t<T>;
+    constexpr int MI = tr::MI;
+    constexpr int VL = tr::VL;
+    constexpr int RB = DMA_ROW;
+    constexpr int BK = RB / int(sizeof(T));
+    constexpr int STAGE = (BM + BN) * RB;
+    constexpr int A_BYTES = BM * RB;
+    constexpr int WM = BM / 2, WN = BN / 2;
+    constexpr int TM = WM / MI, TN = WN / MI;
+    constexpr int STEPS = BK / (tr::KG * VL);
+    // load instructions per thread per slice: one moves 16 rows per wavefront
+    constexpr int NLA = BM / 64, NLB = BN / 64;
+    static_assert(MI == 32 && tr::KG == 2 && STEPS == 2, "layout below assumes 32x32 tiles");
+    static_assert(BM % 64 == 0 && BN % 64 == 0, "");
+
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    uint32_t const lds_base =
+        uint32_t(uintptr_t((__attribute__((address_space(3))) char*)lds));
+
+    int const tid = threadIdx.x;
+    int const lane = tid & 63;
+    int const wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    int const wm = wave >> 1, wn = wave & 1;
+
+    uint32_t const n_tiles = a.tiles_m * a.tiles_n;
+    uint32_t       tile = blockIdx.x;
+    {
+        uint32_t const per_xcd = n_tiles / 8;
+        if (tile < per_xcd * 8) tile = (tile % 8) * per_xcd + tile / 8;
+    }
+    constexpr uint32_t GROUP_M = 4;
+    uint32_t const     in_group = GROUP_M * a.tiles_n;
+    uint32_t const     first_m = (tile / in_group) * GROUP_M;
+    uint32_t const     rows = (a.tiles_m - first_m) < GROUP_M ? (a.tiles_m - first_m) : GROUP_M;
+    uint32_t const     tm = first_m + (tile % in_group) % rows;
+    uint32_t const     tn = (tile % in_group) / rows;
+    uint32_t const     bz = blockIdx.y;
+
+    int64_t boa, bob, boc;
+    {
+        group_offsets(a.gb, bz, boa, bob);
+        boc = 0;
+        uint32_t i = bz;
+#pragma unroll
+        for (int d = 0; d != MAXG; ++d) {
+            uint32_t q = i / a.gb.size[d];
+            boc += int64_t(i - q * a.gb.size[d]) * a.gb.sz[d];
+            i = q;
+        }
+    }
+    // the bases go into scalar registers of the load instructions
+    auto uniform = [](T const* p) {
+        uint64_t const v = reinterpret_cast<uint64_t>(p);
+        uint32_t const lo = __builtin_amdgcn_readfirstlane(uint32_t(v));
+        uint32_t const hi = __builtin_amdgcn_readfirstlane(uint32_t(v >> 32));
+        return reinterpret_cast<T const*>((uint64_t(hi) << 32) | lo);
+    };
+    T const* const A = uniform(static_cast<T const*>(a.A) + boa);
+    T const* const B = uniform(static_cast<T const*>(a.B) + bob);
+
+    // Load instruction i of this wavefront covers rows (4 i + wave) * 16 + lane / 4 of the
+    // tile; the lane's LDS slot is chunk lane % 4 of that row and holds global chunk
+    // (lane % 4) ^ bits 2..3 of the row = (lane % 4) ^ ((lane / 16) % 4).
+    uint32_t const load_chunk = uint32_t((lane & 3) ^ ((lane >> 4) & 3));
+    uint32_t       voa[NLA], vob[NLB];
+#pragma unroll
+    for (int i = 0; i != NLA; ++i) {
+        uint32_t r = tm * BM + uint32_t((4 * i + wave) * 16 + lane / 4);
+        r = r < a.M ? r : a.M - 1;
+        int64_t x, y;
+        group_offsets(a.gm, r, x, y);
+        voa[i] = uint32_t(x) * uint32_t(sizeof(T));
+    }
+#pragma unroll
+    for (int i = 0; i != NLB; ++i) {
+        uint32_t r = tn * BN + uint32_t((4 * i + wave) * 16 + lane / 4);
+        r = r < a.N ? r : a.N - 1;
+        int64_t x, y;
+        group_offsets(a.gn, r, x, y);
+        vob[i] = uint32_t(x) * uint32_t(sizeof(T));
+    }
+    // byte offsets of the lane's 16-byte chunk of slice kt within a row of A / of B
+    auto k_offsets = [&](uint32_t kt, uint32_t& ka, uint32_t& kb) {
+        uint32_t const k = kt * BK + load_chunk * VL;
+        if (a.gk.n == 1) {  // one k mode: contiguous in both operands on this path
+            ka = kb = k * uint32_t(sizeof(T));
+        } else {
+            int64_t x, y;
+            group_offsets(a.gk, k, x, y);
+            ka = uint32_t(x) * uint32_t(sizeof(T));
+            kb = uint32_t(y) * uint32_t(sizeof(T));
+        }
+    };
+    // load q of slice kt: A rows for q < NLA, B rows after that
+    auto issue = [&](uint32_t kt, int q, uint32_t ka, uint32_t kb) {
+        uint32_t const st = kt % NS;
+        if (q < NLA) {
+            load_to_lds_16(A, voa[q] + ka,
+                           lds_base + st * STAGE + uint32_t(4 * q + wave) * 1024);
+        } else {
+            load_to_lds_16(B, vob[q - NLA] + kb,
+                           lds_base + st * STAGE + A_BYTES + uint32_t(4 * (q - NLA) + wave) * 1024);
+        }
+    };
+
+    typename tr::acc_t acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i != TM; ++i) {
+#pragma unroll
+        for (int j = 0; j != TN; ++j) {
+#pragma unroll
+            for (int e = 0; e != tr::NACC; ++e) acc[i][j][e] = 0;
+        }
+    }
+
+    // Fragment of k-step s for MFMA tile row r0 + lane % 32: k-chunk 2 s + lane / 32, found
+    // in slot chunk ^ bits 2..3 of the row
+    int const f_sw = (lane >> 2) & 3;
+    int       f_off[STEPS];
+#pragma unroll
+    for (int s = 0; s != STEPS; ++s) {
+        f_off[s] = (lane % MI) * RB + (((2 * s + lane / MI) ^ f_sw) * 16);
+    }
+    int const fa_base = wm * WM * RB;
+    int const fb_base = A_BYTES + wn * WN * RB;
+
+    chunk_t fa[2][TM], fb[2][TN];
+    // read order: what the first matrix instructions of a step need comes first
+    auto read_frag = [&](char const* stage, int s, int q, chunk_t(&xa)[TM], chunk_t(&xb)[TN]) {
+        if (q == 0) {
+            xa[0] = *reinterpret_cast<chunk_t const*>(stage + fa_base + f_off[s]);
+        } else if (q <= TN) {
+            xb[q - 1] = *reinterpret_cast<chunk_t const*>(stage + fb_base + (q - 1) * MI * RB +
+                                                          f_off[s]);
+        } else {
+            xa[q - TN] = *reinterpret_cast<chunk_t const*>(stage + fa_base + (q - TN) * MI * RB +
+                                                           f_off[s]);
+        }
+    };
+    constexpr int READS = TM + TN;
+    constexpr int PAIRS = TM * TN;
+    constexpr int LOADS = NLA + NLB;
+    // side work per matrix instruction: step 0 spreads the reads over all of them, step 1
+    // over all but the first (which is followed by the barrier)
+    constexpr int R0 = (READS + PAIRS - 1) / PAIRS;
+    constexpr int R1 = (READS + PAIRS - 2) / (PAIRS - 1);
+    constexpr int L1 = (LOADS + PAIRS - 2) / (PAIRS - 1);
+
+    uint32_t const nk = a.K / BK;  // >= NS, no remainder (checked by the launcher)
+
+    // prologue: four slices in flight, the first one landed
+#pragma unroll
+    for (int s = 0; s != NS; ++s) {
+        uint32_t ka, kb;
+        k_offsets(uint32_t(s), ka, kb);
+#pragma unroll
+        for (int q = 0; q != LOADS; ++q) issue(uint32_t(s), q, ka, kb);
+    }
+    wait_loads_and_lds<LOADS*(NS - 1)>();
+    __builtin_amdgcn_s_barrier();
+#pragma unroll
+    for (int q = 0; q != READS; ++q) read_frag(lds, 0, q, fa[0], fb[0]);
+
+    // One slice.  YOUNGER = slices issued after slice kt+1 that may still be in flight when
+    // slice kt+1 is needed (-1: there is no slice kt+1); ISSUE: refill this stage with kt+4.
+    auto slice = [&](uint32_t kt, auto younger_tag, auto issue_tag) {
+        constexpr int  YOUNGER = decltype(younger_tag)::value;
+        constexpr bool ISSUE = decltype(issue_tag)::value;
+        char const*    cur = lds + (kt % NS) * STAGE;
+        char const*    nxt = lds + ((kt + 1) % NS) * STAGE;
+        uint32_t       ka = 0, kb = 0;
+        if (ISSUE) k_offsets(kt + NS, ka, kb);
+#pragma unroll
+        for (int p = 0; p != PAIRS; ++p) {
+            tr::mma(acc[p / TN][p % TN], fb[0][p % TN], fa[0][p / TN]);
+#pragma unroll
+            for (int r = p * R0; r != (p + 1) * R0; ++r) {
+                if (r < READS) read_frag(cur, 1, r, fa[1], fb[1]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int p = 0; p != PAIRS; ++p) {
+            tr::mma(acc[p / TN][p % TN], fb[1][p % TN], fa[1][p / TN]);
+            if (YOUNGER >= 0) {
+                if (p == 0) {
+                    // this wave's part of slice kt+1 has landed and its reads of this stage
+                    // are complete; after the barrier that holds for the whole workgroup
+                    wait_loads_and_lds<(YOUNGER < 0 ? 0 : YOUNGER) * LOADS>();
+                    __builtin_amdgcn_s_barrier();
+                } else {
+#pragma unroll
+                    for (int r = (p - 1) * R1; r != p * R1; ++r) {
+                        if (r < READS) read_frag(nxt, 0, r, fa[0], fb[0]);
+                    }
+#pragma unroll
+                    for (int r = (p - 1) * L1; r != p * L1; ++r) {
+                        if (ISSUE && r < LOADS) issue(kt + NS, r, ka, kb);
+                    }
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    {
+        using std::integral_constant;
+        uint32_t kt = 0;
+        for (; kt + NS < nk; ++kt) {
+            slice(kt, integral_constant<int, NS - 2>{}, std::true_type{});
+        }
+        // the last NS slices refill nothing and have ever fewer loads behind them
+        auto tail = [&](auto const& self, auto j_tag) {
+            constexpr int J = decltype(j_tag)::value;
+            slice(kt++, integral_constant<int, NS - 2 - J>{}, std::false_type{});
+            if constexpr (J + 1 < NS) self(self, integral_constant<int, J + 1>{});
+        };
+        tail(tail, integral_constant<int, 0>{});
+    }
+
+    // Epilogue: each wave turns MI rows of its tile through a private LDS strip so that the
+    // global stores are 16 bytes per lane and whole row segments per wavefront.
+    T* const C = static_cast<T*>(a.C) + boc;
+    constexpr int STRIP_PITCH = WN * int(sizeof(T)) + 16;
+    constexpr int CPR = WN * int(sizeof(T)) / 16;
+    wait_loads_and_lds<0>();
+    __builtin_amdgcn_s_barrier();
+    char* const strip = lds + wave * (MI * STRIP_PITCH);
+    typedef T quad_t __attribute__((ext_vector_type(4)));
+#pragma unroll
+    for (int i = 0; i != TM; ++i) {
+#pragma unroll
+        for (int j = 0; j != TN; ++j) {
+#pragma unroll
+            for (int e0 = 0; e0 < tr::NACC; e0 += 4) {
+                quad_t q;
+#pragma unroll
+                for (int t = 0; t != 4; ++t) q[t] = T(acc[i][j][e0 + t]);
+                int n = j * MI + tr::acc_row(e0, lane);
+                *reinterpret_cast<quad_t*>(strip + (lane % MI) * STRIP_PITCH +
+                                           n * int(sizeof(T))) = q;
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int c = 0; c != MI * CPR / 64; ++c) {
+            int      idx = c * 64 + lane;
+            int      r = idx / CPR, ch = idx % CPR;
+            uint32_t m = tm * BM + wm * WM + i * MI + uint32_t(r);
+            uint32_t n = tn * BN + wn * WN + uint32_t(ch) * VL;
+            chunk_t  v = *reinterpret_cast<chunk_t const*>(strip + r * STRIP_PITCH + ch * 16);
+            if (m < a.M && n < a.N) {
+                int64_t mo_a, mo_c, no_b, no_c;
+                group_offsets(a.gm, m, mo_a, mo_c);
+                group_offsets(a.gn, n, no_b, no_c);
+                *reinterpret_cast<chunk_t*>(C + mo_c + no_c) = v;
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+}
+
+// Whether the direct-to-LDS kernel can run this problem (both operands 16-byte vectors along
+// k, wide epilogue, K a whole number of at least four slices, operand offsets within 32 bits).
+template <typename T>
+bool gemm_dma_eligible(gemm_args_t const& a)
+{
+    constexpr uint32_t BK = DMA_ROW / sizeof(T);
+    return a.a_mode == 0 && a.b_mode == 0 && a.c_mode == 3 && a.K % BK == 0 &&
+           a.K / BK >= 4 && a.offsets_fit_32 != 0;
+}
+
+template <typename T, int BM, int BN, int NS>
+void launch_gemm_dma_kernel(gemm_args_t const& a, hipStream_t stream)
+{
+    static_assert(NS >= 2 && NS <= 4, "eligibility guarantees four slices");
+    constexpr int lds = NS * (BM + BN) * DMA_ROW;
+    static bool const raised = [] {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_dma_kernel<T, BM, BN, NS>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        return true;
+    }();
+    (void)raised;
+    dim3 grid(a.tiles_m * a.tiles_n, a.batch, 1);
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, NS>), grid, dim3(256), lds, stream, a);
+}
+
+}  // namespace gemm
+}  // namespace es

@@ -1,4 +1,5 @@
 // fp16-in / fp32-accumulate instantiations of the MFMA GEMM kernel.
+#include "gemm_dma_kernel.h"
 #include "gemm_kernel.h"
 
 namespace es
@@ -6,14 +7,26 @@ namespace es
 namespace gemm
 {
 
+// `a` arrives cut into bm x bn tiles.  A tile without a kernel for this problem's load paths
+// (they can change at run time, with the alignment of the buffers) is replaced by 128 x 128.
 void launch_gemm_f16(int bm, int bn, gemm_args_t const& a, hipStream_t stream)
 {
     using T = _Float16;
-    bool done = false;
     if (a.tiles_m == 0) return;
-    if (bm == 256 && bn == 256) done = launch_gemm_fast<T, 256, 256>(a, stream);
-    if (bm == 128 && bn == 128) done = launch_gemm_fast<T, 128, 128>(a, stream);
-    if (!done) launch_gemm_kernel<T, 128, 128, -1, -1>(a, stream);
+    if (gemm_dma_eligible<T>(a)) {
+        if (bm == 256 && bn == 256) return launch_gemm_dma_kernel<T, 256, 256, 4>(a, stream);
+        if (bm == 256 && bn == 128) return launch_gemm_dma_kernel<T, 256, 128, 4>(a, stream);
+        if (bm == 128 && bn == 256) return launch_gemm_dma_kernel<T, 128, 256, 4>(a, stream);
+        // short reductions: three stages of a small tile keep three workgroups per compute
+        // unit, whose loads, matrix work and stores overlap each other
+        if (bm == 128 && bn == 128 && a.K < 512) {
+            return launch_gemm_dma_kernel<T, 128, 128, 3>(a, stream);
+        }
+    }
+    if (bm == 256 && bn == 256 && launch_gemm_fast<T, 256, 256>(a, stream)) return;
+    gemm_args_t const b = with_tile(a, 128, 128);
+    if (launch_gemm_fast<T, 128, 128>(b, stream)) return;
+    launch_gemm_kernel<T, 128, 128, -1, -1>(b, stream);
 }
 
 // Measurement aid: matrix-core throughput with register-resident operands, i.e. the ceiling

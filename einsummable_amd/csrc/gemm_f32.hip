@@ -9,11 +9,11 @@ namespace gemm
 void launch_gemm_f32(int bm, int bn, gemm_args_t const& a, hipStream_t stream)
 {
     using T = float;
-    bool done = false;
     if (a.tiles_m == 0) return;
-    if (bm == 256 && bn == 256) done = launch_gemm_fast<T, 256, 256>(a, stream);
-    if (bm == 128 && bn == 128) done = launch_gemm_fast<T, 128, 128>(a, stream);
-    if (!done) launch_gemm_kernel<T, 128, 128, -1, -1>(a, stream);
+    if (bm == 256 && bn == 256 && launch_gemm_fast<T, 256, 256>(a, stream)) return;
+    gemm_args_t const b = with_tile(a, 128, 128);
+    if (launch_gemm_fast<T, 128, 128>(b, stream)) return;
+    launch_gemm_kernel<T, 128, 128, -1, -1>(b, stream);
 }
 
 }  // namespace gemm

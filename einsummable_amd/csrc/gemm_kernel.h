@@ -36,6 +36,7 @@ struct gemm_args_t {
     int         a_mode, b_mode;  // 0: 16-byte vectors along k, 1: along m / n, 2: elementwise
     int         c_mode;          // 0: four consecutive n per store, 2: elementwise,
                                  // 3: 16-byte row segments through LDS (tuned kernel)
+    int         offsets_fit_32;  // every byte offset into A and B (per batch entry) < 2^32
 };
 
 __device__ __forceinline__ void group_offsets(group_t const& g, uint32_t i, int64_t& ox,
@@ -832,8 +833,14 @@ void launch_gemm_f32(int bm, int bn, gemm_args_t const& a, hipStream_t stream);
 void launch_gemm_f64(int bm, int bn, gemm_args_t const& a, hipStream_t stream);
 double probe_mfma_f16(void const* operands, void* scratch, int blocks, int iters,
                       hipStream_t stream);
-// whether launch_gemm_* has a specialised kernel for this tile
-bool gemm_has_tile(int elem_size, int bm, int bn);
+
+// the same problem cut into bm x bn tiles
+inline gemm_args_t with_tile(gemm_args_t a, int bm, int bn)
+{
+    a.tiles_m = (a.M + uint32_t(bm) - 1) / uint32_t(bm);
+    a.tiles_n = (a.N + uint32_t(bn) - 1) / uint32_t(bn);
+    return a;
+}
 
 template <typename T, int BM, int BN, int AM, int BM_>
 void launch_gemm_kernel(gemm_args_t const& a, hipStream_t stream)

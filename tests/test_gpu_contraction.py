@@ -127,3 +127,58 @@ def test_misaligned_operands_fall_back_to_elementwise_loads(km):
     torch.cuda.synchronize()
     got = dc[1:1 + 4096].cpu().numpy()
     assert_close(got, oracle_einsummable(e, [a, b], oracle.WIDE), ea.F16, what="misaligned")
+
+
+@pytest.fixture()
+def km_big_tiles(km, monkeypatch):
+    """A second manager (after the session's, which initialises the device) whose planner is told to use 256 x 256 tiles wherever a kernel for them
+    exists (the planner otherwise keeps them for problems too large for the oracle)."""
+    monkeypatch.setenv("ES_KM_GEMM_TILE", "256x256")
+    return ea.KernelManager(0)
+
+
+BIG_TILE_CASES = [
+    # k-contiguous operands: the direct-to-LDS kernel (K a multiple of 32, at least 128)
+    ("ij,kj->ik", dict(i=256, j=128, k=256)),        # exactly one tile, the minimum depth
+    ("ij,kj->ik", dict(i=512, j=160, k=256)),        # five slices: one trip of the steady loop
+    ("ij,kj->ik", dict(i=264, j=448, k=520)),        # ragged m and n: clamped rows
+    ("ij,kj->ik", dict(i=40, j=256, k=24)),          # one partial tile
+    ("bij,bkj->bik", dict(b=3, i=272, j=192, k=136)),
+    ("adbe,cde->abc", dict(a=2, d=4, b=136, e=64, c=264)),   # two k modes, strided m
+    ("acbe,adbe->abcd", dict(a=1, b=2, c=264, d=136, e=128)),
+    # K not a whole number of slices, or too short: the register-staged 256 x 256 kernel
+    ("ij,kj->ik", dict(i=264, j=72, k=264)),
+    ("ij,kj->ik", dict(i=264, j=296, k=264)),
+    # B contiguous along n
+    ("ij,jk->ik", dict(i=264, j=160, k=264)),
+]
+DIRECT_TO_LDS = 7  # leading cases of the list that the direct-to-LDS kernel takes
+
+
+@pytest.mark.parametrize("case", range(len(BIG_TILE_CASES)))
+def test_big_tile_kernels(km_big_tiles, case):
+    km = km_big_tiles
+    spec, sizes = BIG_TILE_CASES[case]
+    check(km, spec, sizes, "f16", seed=20)
+    d = km.describe(contraction(spec, sizes, "f16"))
+    assert "tile=256x256" in d
+    assert ("load=direct_to_lds" in d) == (case < DIRECT_TO_LDS), d
+
+
+def test_big_tile_matches_small_tile_bitwise_on_exact_data(km, monkeypatch):
+    # small integers: every product and partial sum is exact in fp32, so both tilings must
+    # give the same bits whatever their summation order
+    e = contraction("ij,kj->ik", dict(i=520, j=256, k=392), "f16")
+    km.build(e)  # planned with the default tile rule
+    monkeypatch.setenv("ES_KM_GEMM_TILE", "256x256")
+    km_big_tiles = ea.KernelManager(0)
+    r = rng(21)
+    xs = [r.randint(-4, 5, size=520 * 256).astype(np.float16),
+          r.randint(-4, 5, size=392 * 256).astype(np.float16)]
+    a = run_einsummable(km, e, xs)
+    b = run_einsummable(km_big_tiles, e, xs)
+    assert "tile=128x128" in km.describe(e) and "tile=256x256" in km_big_tiles.describe(e)
+    want = (xs[0].astype(np.float64).reshape(520, 256) @
+            xs[1].astype(np.float64).reshape(392, 256).T).astype(np.float16)
+    np.testing.assert_array_equal(a.view(np.uint16), b.view(np.uint16))
+    np.testing.assert_array_equal(a.reshape(520, 392), want)
