@@ -63,14 +63,14 @@ void fill_group(group_t& g, std::vector<mode_info_t> const& ms,
 }
 
 // Macro tile for a problem.  Larger tiles cost less LDS and L1 traffic per flop, which is what
-// limits the kernels (measured full-chip rates on MI355X, fp16: 256x256 ~1.2 PFLOP/s,
-// 128x256 ~0.98, 128x128 ~0.8), but there are fewer of them to spread over the 256 compute
-// units.  The estimate below is rounds of resident workgroups times the time of one tile.
+// limits the fp16 kernels (measured full-chip rates on MI355X with the direct-to-LDS kernel:
+// 256x256 ~1.2 PFLOP/s, 128x256 ~0.98, 128x128 ~0.8), but there are fewer of them to spread
+// over the 256 compute units.  fp32 is bound by the matrix cores at every tile size, so only
+// the spread matters.  Estimate: tiles per compute unit, rounded up, times the time of a tile.
 // ES_KM_GEMM_TILE=128x128|128x256|256x128|256x256 overrides the choice (tuning aid).
 struct tile_option_t {
     int    bm, bn;
-    int    per_cu;  // workgroups resident on one compute unit
-    double eff;     // relative rate of one compute unit running this tile
+    double eff16, eff32;  // relative rate of a compute unit running this tile
 };
 
 void choose_tile(dtype_t dt, uint64_t M, uint64_t N, uint64_t K, uint64_t batch, bool dma_ok,
@@ -99,14 +99,24 @@ void choose_tile(dtype_t dt, uint64_t M, uint64_t N, uint64_t K, uint64_t batch,
         if (K >= 1024 && M >= 512 && N >= 512 && big_tiles >= 768) bm = bn = 256;
         return;
     }
-    static tile_option_t const options[] = {
-        {256, 256, 1, 1.00}, {128, 256, 1, 0.80}, {256, 128, 1, 0.78}, {128, 128, 2, 0.66}};
+    // Streaming shapes (one operand read once, little reuse: attention's P.V) are bound by
+    // HBM; with many rounds of tiles the small tile's extra workgroups per compute unit keep
+    // more loads in flight
+    double const elem = double(dtype_size(dt));
+    double const intensity = 2.0 * double(M) * double(N) * double(K) /
+                             ((double(M) * K + double(N) * K + double(M) * N) * elem);
+    uint64_t const small_tiles = ((M + 127) / 128) * ((N + 127) / 128) * batch;
+    if (dt == dtype_t::f16 && intensity < 150.0 && small_tiles >= 1024) return;
+    static tile_option_t const options[] = {{256, 256, 1.00, 1.00},
+                                            {128, 256, 0.80, 1.00},
+                                            {256, 128, 0.80, 1.00},
+                                            {128, 128, 0.68, 1.00}};
     double best = 0;
     for (tile_option_t const& o : options) {
         uint64_t tiles = ((M + o.bm - 1) / o.bm) * ((N + o.bn - 1) / o.bn) * batch;
-        uint64_t slots = 256ull * uint64_t(o.per_cu);
-        uint64_t rounds = (tiles + slots - 1) / slots;
-        double   t = double(rounds) * o.per_cu * double(o.bm) * double(o.bn) / o.eff;
+        uint64_t rounds = (tiles + 255) / 256;
+        double   t = double(rounds) * double(o.bm) * double(o.bn) /
+                   (dt == dtype_t::f16 ? o.eff16 : o.eff32);
         if (best == 0 || t < best * 0.97) {  // near ties go to the larger tile (listed first)
             best = t;
             bm = o.bm;
@@ -264,13 +274,14 @@ std::shared_ptr<plan_t> plan_contraction(einsummable_t const& e, int)
                        e.inn_nelem(1) * dtype_size(dt) < (1ull << 32);
 
     // large tiles exist for the vector load paths (A along k; B along k or n)
-    bool const dma_ok = dt == dtype_t::f16 && gemm_dma_eligible<_Float16>(a);
+    bool const dma_ok = (dt == dtype_t::f16 && gemm_dma_eligible<_Float16>(a)) ||
+                        (dt == dtype_t::f32 && gemm_dma_eligible<float>(a));
     if (a.a_mode == 0 && a.b_mode != 2) choose_tile(dt, M, N, K, Bt, dma_ok, p->bm, p->bn);
     a.tiles_m = uint32_t((M + p->bm - 1) / p->bm);
     a.tiles_n = uint32_t((N + p->bn - 1) / p->bn);
     if (uint64_t(a.tiles_m) * a.tiles_n >= lim) return nullptr;
 
-    bool const dma = dma_ok && (p->bm != 128 || p->bn != 128 || K < 512);
+    bool const dma = dma_ok;  // every tile has a direct-to-LDS kernel
     p->workspace_bytes = 0;
     static const char* mode_name[] = {"k", "mn", "elem"};
     p->description = std::string("contraction_mfma_") + dtype_name(dt) + " tile=" +

@@ -19,8 +19,9 @@ void launch_gemm_f16(int bm, int bn, gemm_args_t const& a, hipStream_t stream)
         if (bm == 128 && bn == 256) return launch_gemm_dma_kernel<T, 128, 256, 4>(a, stream);
         // short reductions: three stages of a small tile keep three workgroups per compute
         // unit, whose loads, matrix work and stores overlap each other
-        if (bm == 128 && bn == 128 && a.K < 512) {
-            return launch_gemm_dma_kernel<T, 128, 128, 3>(a, stream);
+        if (bm == 128 && bn == 128) {
+            return a.K < 512 ? launch_gemm_dma_kernel<T, 128, 128, 3>(a, stream)
+                             : launch_gemm_dma_kernel<T, 128, 128, 4>(a, stream);
         }
     }
     if (bm == 256 && bn == 256 && launch_gemm_fast<T, 256, 256>(a, stream)) return;

@@ -1,4 +1,5 @@
 // fp32 instantiations of the MFMA GEMM kernel.
+#include "gemm_dma_kernel.h"
 #include "gemm_kernel.h"
 
 namespace es
@@ -10,6 +11,12 @@ void launch_gemm_f32(int bm, int bn, gemm_args_t const& a, hipStream_t stream)
 {
     using T = float;
     if (a.tiles_m == 0) return;
+    if (gemm_dma_eligible<T>(a)) {
+        if (bm == 256 && bn == 256) return launch_gemm_dma_kernel<T, 256, 256, 4>(a, stream);
+        if (bm == 256 && bn == 128) return launch_gemm_dma_kernel<T, 256, 128, 4>(a, stream);
+        if (bm == 128 && bn == 256) return launch_gemm_dma_kernel<T, 128, 256, 4>(a, stream);
+        if (bm == 128 && bn == 128) return launch_gemm_dma_kernel<T, 128, 128, 4>(a, stream);
+    }
     if (bm == 256 && bn == 256 && launch_gemm_fast<T, 256, 256>(a, stream)) return;
     gemm_args_t const b = with_tile(a, 128, 128);
     if (launch_gemm_fast<T, 128, 128>(b, stream)) return;

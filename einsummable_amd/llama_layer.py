@@ -242,3 +242,19 @@ class DeviceRunner:
                 timers[i].record(launch)
             else:
                 launch()
+
+    def capture(self):
+        """Records the whole node list into a HIP graph (every node is a plain kernel launch
+        on the given stream, so stream capture sees all of it) and returns the graph; replay
+        removes the host's per-node launch cost."""
+        torch = self.torch
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            self.run(stream=side.cuda_stream)      # everything compiled and loaded
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            self.run(stream=torch.cuda.current_stream().cuda_stream)
+        return graph

@@ -129,40 +129,48 @@ def test_misaligned_operands_fall_back_to_elementwise_loads(km):
     assert_close(got, oracle_einsummable(e, [a, b], oracle.WIDE), ea.F16, what="misaligned")
 
 
-@pytest.fixture()
-def km_big_tiles(km, monkeypatch):
-    """A second manager (after the session's, which initialises the device) whose planner is told to use 256 x 256 tiles wherever a kernel for them
-    exists (the planner otherwise keeps them for problems too large for the oracle)."""
-    monkeypatch.setenv("ES_KM_GEMM_TILE", "256x256")
-    return ea.KernelManager(0)
-
-
 BIG_TILE_CASES = [
-    # k-contiguous operands: the direct-to-LDS kernel (K a multiple of 32, at least 128)
-    ("ij,kj->ik", dict(i=256, j=128, k=256)),        # exactly one tile, the minimum depth
-    ("ij,kj->ik", dict(i=512, j=160, k=256)),        # five slices: one trip of the steady loop
-    ("ij,kj->ik", dict(i=264, j=448, k=520)),        # ragged m and n: clamped rows
-    ("ij,kj->ik", dict(i=40, j=256, k=24)),          # one partial tile
-    ("bij,bkj->bik", dict(b=3, i=272, j=192, k=136)),
-    ("adbe,cde->abc", dict(a=2, d=4, b=136, e=64, c=264)),   # two k modes, strided m
-    ("acbe,adbe->abcd", dict(a=1, b=2, c=264, d=136, e=128)),
-    # K not a whole number of slices, or too short: the register-staged 256 x 256 kernel
-    ("ij,kj->ik", dict(i=264, j=72, k=264)),
-    ("ij,kj->ik", dict(i=264, j=296, k=264)),
-    # B contiguous along n
-    ("ij,jk->ik", dict(i=264, j=160, k=264)),
+    # (spec, sizes, dtype, taken by the direct-to-LDS kernel)
+    # k-contiguous operands: K a multiple of the 64-byte slice and at least four slices
+    ("ij,kj->ik", dict(i=256, j=128, k=256), "f16", True),   # one tile, the minimum depth
+    ("ij,kj->ik", dict(i=512, j=160, k=256), "f16", True),   # five slices: one steady-loop trip
+    ("ij,kj->ik", dict(i=264, j=448, k=520), "f16", True),   # ragged m and n: clamped rows
+    ("ij,kj->ik", dict(i=40, j=256, k=24), "f16", True),     # one partial tile
+    ("bij,bkj->bik", dict(b=3, i=272, j=192, k=136), "f16", True),
+    ("adbe,cde->abc", dict(a=2, d=4, b=136, e=64, c=264), "f16", True),  # two k modes
+    ("acbe,adbe->abcd", dict(a=1, b=2, c=264, d=136, e=128), "f16", True),
+    ("ij,kj->ik", dict(i=264, j=80, k=520), "f32", True),
+    # B contiguous along n: kept [k][n] in LDS, read transposed
+    ("ij,jk->ik", dict(i=264, j=160, k=264), "f16", True),
+    ("ij,jk->ik", dict(i=264, j=128, k=520), "f16", True),
+    ("ij,jk->ik", dict(i=40, j=256, k=24), "f16", True),
+    ("bhij,bhjd->bhid", dict(b=2, h=2, i=264, j=192, d=128), "f16", True),
+    ("abce,aebd->abcd", dict(a=1, b=3, c=136, e=160, d=64), "f16", True),
+    ("ij,jk->ik", dict(i=264, j=80, k=264), "f32", True),
+    ("ij,jk->ik", dict(i=130, j=64, k=520), "f32", True),
+    ("bij,bjk->bik", dict(b=2, i=40, j=112, k=72), "f32", True),
+    # K not a whole number of slices, or too short: the register-staged kernels
+    ("ij,kj->ik", dict(i=264, j=72, k=264), "f16", False),
+    ("ij,kj->ik", dict(i=264, j=296, k=264), "f16", False),
+    ("ij,jk->ik", dict(i=264, j=100, k=264), "f32", False),
 ]
-DIRECT_TO_LDS = 7  # leading cases of the list that the direct-to-LDS kernel takes
+BIG_TILES = ["256x256", "128x256", "256x128"]
 
 
+@pytest.mark.parametrize("tile", BIG_TILES)
 @pytest.mark.parametrize("case", range(len(BIG_TILE_CASES)))
-def test_big_tile_kernels(km_big_tiles, case):
-    km = km_big_tiles
-    spec, sizes = BIG_TILE_CASES[case]
-    check(km, spec, sizes, "f16", seed=20)
-    d = km.describe(contraction(spec, sizes, "f16"))
-    assert "tile=256x256" in d
-    assert ("load=direct_to_lds" in d) == (case < DIRECT_TO_LDS), d
+def test_big_tile_kernels(km, monkeypatch, case, tile):
+    # a second manager (after the session's, which initialises the device) whose planner is
+    # told which tile to use: left alone it keeps the large ones for problems too big for
+    # the oracle
+    monkeypatch.setenv("ES_KM_GEMM_TILE", tile)
+    big = ea.KernelManager(0)
+    spec, sizes, dt, direct = BIG_TILE_CASES[case]
+    check(big, spec, sizes, dt, seed=20)
+    d = big.describe(contraction(spec, sizes, dt))
+    assert ("load=direct_to_lds" in d) == direct, d
+    if direct or tile == "256x256":
+        assert "tile=" + tile in d, d
 
 
 def test_big_tile_matches_small_tile_bitwise_on_exact_data(km, monkeypatch):

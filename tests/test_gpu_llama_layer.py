@@ -84,6 +84,32 @@ def test_reduced_layer_matches_oracle_node_by_node_chain(km):
     np.testing.assert_allclose(p.sum(axis=1), 1.0, rtol=1e-5)
 
 
+def test_layer_replayed_as_hip_graph_matches_eager_launches(km):
+    """The node list captured into one HIP graph: every replay, with eager work and
+    synchronisations in between and with fresh inputs, must reproduce the eager bytes."""
+    import torch
+
+    g = LayerGraph(dim=256, n_heads=4, ffn=688, seq=128)
+    run = DeviceRunner(km, g)
+    for k, v in make_inputs(g, 1).items():
+        run.set_input(k, v)
+    graph = run.capture()
+    for seed in (2, 3, 4):
+        vals = make_inputs(g, seed)
+        for k, v in vals.items():
+            run.set_input(k, v)
+        run.run()
+        torch.cuda.synchronize()
+        eager = {name: run.get(name, np.uint8).copy() for name in ("residual2", "sm.div", "mask")}
+        for name in eager:
+            run.mem[name].zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, want in eager.items():
+            assert np.array_equal(run.get(name, np.uint8), want), (seed, name)
+
+
 def torch_layer_fp32(g, vals):
     """fp32 torch restatement of the layer, rounded to fp16 wherever the graph's tensors are
     fp16 (unscaled attention logits reach ~50, where one fp16 ulp already moves exp() by 3%,
