@@ -270,6 +270,7 @@ std::shared_ptr<plan_t> plan_contraction(einsummable_t const& e, int)
     a.a_mode = vec_ok(js, sA, VL) ? 0 : (vec_ok(gm, sA, VL) ? 1 : 2);
     a.b_mode = vec_ok(js, sB, VL) ? 0 : (vec_ok(gn, sB, VL) ? 1 : 2);
     a.c_mode = vec_ok(gn, sC, VL) ? 3 : (vec_ok(gn, sC, 4) ? 0 : 2);
+    a.c_stream = e.out_nelem() * dtype_size(dt) >= (64ull << 20);
     a.offsets_fit_32 = e.inn_nelem(0) * dtype_size(dt) < (1ull << 32) &&
                        e.inn_nelem(1) * dtype_size(dt) < (1ull << 32);
 

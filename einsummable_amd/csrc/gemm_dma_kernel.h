@@ -373,7 +373,12 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
                 int64_t mo_a, mo_c, no_b, no_c;
                 group_offsets(a.gm, m, mo_a, mo_c);
                 group_offsets(a.gn, n, no_b, no_c);
-                *reinterpret_cast<chunk_t*>(C + mo_c + no_c) = v;
+                chunk_t* const dst = reinterpret_cast<chunk_t*>(C + mo_c + no_c);
+                if (a.c_stream) {
+                    __builtin_nontemporal_store(v, dst);
+                } else {
+                    *dst = v;
+                }
             }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");

@@ -37,6 +37,7 @@ struct gemm_args_t {
     int         c_mode;          // 0: four consecutive n per store, 2: elementwise,
                                  // 3: 16-byte row segments through LDS (tuned kernel)
     int         offsets_fit_32;  // every byte offset into A and B (per batch entry) < 2^32
+    int         c_stream;        // C exceeds the caches: store it non-temporally
 };
 
 __device__ __forceinline__ void group_offsets(group_t const& g, uint32_t i, int64_t& ox,
