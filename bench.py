@@ -282,19 +282,82 @@ def run_c3(km, steps, warmup):
     return out
 
 
-def run_c4(km, steps, warmup):
+def c4_nodes(b, h, s, d):
+    """Batched attention as the apply nodes the reference's graph would hold: scores, the
+    1/sqrt(d) scale with the constant as the reference writes it (6 significant digits, then
+    fp16), the row softmax as four scalarop / reduce nodes, and P.V.  Returns
+    (name, einsummable, out buffer, input buffers, work, unit)."""
     import einsummable_amd as ea
 
-    b, h, s, d = 4, 32, 2048, 128
-    flops = 2 * b * h * s * s * d
+    E = ea.Einsummable
     mul = "*[hole|f16@0,hole|f16@1]"
-    e1 = ea.Einsummable([b, h, s, s, d], [[0, 1, 2, 4], [0, 1, 3, 4]], 4, mul, "+")
-    e2 = ea.Einsummable([b, h, s, d, s], [[0, 1, 2, 4], [0, 1, 4, 3]], 4, mul, "+")
-    r1 = run_contraction(km, "c4 scores bhid,bhjd->bhij f16", e1,
-                         [(b, h, s, d), (b, h, s, d), (b, h, s, s)], "f16", flops, steps, warmup)
-    r2 = run_contraction(km, "c4 values bhij,bhjd->bhid f16", e2,
-                         [(b, h, s, s), (b, h, s, d), (b, h, s, d)], "f16", flops, steps, warmup)
-    return [r1, r2]
+    rows, flops = b * h * s, 2 * b * h * s * s * d
+    mat = rows * s * 2
+    return [
+        ("scores bhid,bhjd->bhij", E([b, h, s, s, d], [[0, 1, 2, 4], [0, 1, 3, 4]], 4, mul, "+"),
+         "S", ["Q", "K"], flops, "flop"),
+        ("scale a->a", E([rows * s], [[0]], 1, "*[constant{f16|0.0883789},hole|f16@0]"),
+         "S", ["S"], 2 * mat, "B"),
+        ("rowmax ab->a", E([rows, s], [[0, 1]], 1, "hole|f16@0", "^"), "m", ["S"],
+         mat + rows * 2, "B"),
+        ("exp_sub ab,a->ab", E([rows, s], [[0, 1], [0]], 2, EXP_SUB), "S", ["S", "m"],
+         2 * mat + rows * 2, "B"),
+        ("rowsum ab->a", E([rows, s], [[0, 1]], 1, "hole|f16@0", "+"), "l", ["S"],
+         mat + rows * 2, "B"),
+        ("div ab,a->ab", E([rows, s], [[0, 1], [0]], 2, "*[hole|f16@0,power{-1}[hole|f16@1]]"),
+         "S", ["S", "l"], 2 * mat + rows * 2, "B"),
+        ("values bhij,bhjd->bhid", E([b, h, s, d, s], [[0, 1, 2, 4], [0, 1, 4, 3]], 4, mul, "+"),
+         "O", ["S", "V"], flops, "flop"),
+    ]
+
+
+def run_c4(km, steps, warmup):
+    """C4: b=4, h=32, s=2048, d=128, f16 with fp32 accumulation.  The elementwise nodes write
+    over their first input (the engine donates it), so the 1 GiB score tensor exists once."""
+    import torch
+
+    b, h, s, d = 4, 32, 2048, 128
+    g = torch.Generator(device="cuda").manual_seed(4)
+    mem = {k: torch.randn(b, h, s, d, device="cuda", dtype=torch.float16, generator=g)
+           for k in ("Q", "K", "V")}
+    mem["S"] = torch.empty(b, h, s, s, device="cuda", dtype=torch.float16)
+    mem["O"] = torch.empty(b, h, s, d, device="cuda", dtype=torch.float16)
+    mem["m"] = torch.empty(b * h * s, device="cuda", dtype=torch.float16)
+    mem["l"] = torch.empty(b * h * s, device="cuda", dtype=torch.float16)
+    nodes = c4_nodes(b, h, s, d)
+    for _, e, *_r in nodes:
+        assert km.build(e) == 0
+    stream = torch.cuda.current_stream().cuda_stream
+    calls = [lambda e=e, o=o, i=i: km(e, stream, mem[o].data_ptr(), [mem[x].data_ptr() for x in i])
+             for _, e, o, i, _w, _u in nodes]
+    timers = [Timed() for _ in calls]
+    for _ in range(warmup):
+        for c in calls:
+            c()
+    torch.cuda.synchronize()
+    for _ in range(steps):
+        for c, t in zip(calls, timers):
+            t.record(c)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        for c in calls:
+            c()
+    torch.cuda.synchronize()
+    chain_ms = (time.perf_counter() - t0) / steps * 1e3
+    rows = []
+    for (name, e, _o, _i, work, unit), t in zip(nodes, timers):
+        ms = t.mean_ms()
+        r = {"node": "c4 " + name, "kernel": km.describe(e), "ms": round(ms, 5)}
+        if unit == "flop":
+            r.update(flop=work, TFLOPs=round(work / ms / 1e9, 2),
+                     mfma_frac=round(work / ms / 1e9 / PEAK_TFLOPS["f16"], 4))
+        else:
+            r.update(bytes=work, GBps=round(work / ms / 1e6, 1),
+                     hbm_frac=round(work / ms / 1e6 / HBM_PEAK_GBPS, 4))
+        rows.append(r)
+    rows.append({"node": "c4 whole chain (7 nodes, no per-node events)", "ms": round(chain_ms, 4)})
+    return rows
 
 
 def run_llama_contractions(km, steps, warmup):
@@ -403,6 +466,34 @@ def run_mfma_peak(km):
     return out
 
 
+def run_read_ceiling(km, steps, warmup):
+    """What a kernel that only reads reaches on this device: the generated row max over
+    1 GiB of f16 next to the vendor library's reduction (torch.amax) over the same tensor.
+    Both stop near 4.8 TB/s, well below the 8 TB/s that mixed read + write traffic is
+    priced against."""
+    import torch
+
+    import einsummable_amd as ea
+
+    rows, n = 262144, 2048
+    x = torch.randn(rows, n, device="cuda", dtype=torch.float16)
+    m = torch.empty(rows, device="cuda", dtype=torch.float16)
+    e = ea.Einsummable([rows, n], [[0, 1]], 1, "hole|f16@0", "^")
+    assert km.build(e) == 0
+    stream = torch.cuda.current_stream().cuda_stream
+    ours, lib = Timed(), Timed()
+    for i in range(warmup + steps):
+        t = ours if i >= warmup else Timed()
+        t.record(lambda: km(e, stream, m.data_ptr(), [x.data_ptr()]))
+    for i in range(warmup + steps):
+        t = lib if i >= warmup else Timed()
+        t.record(lambda: torch.amax(x, dim=1, out=m))
+    torch.cuda.synchronize()
+    nbytes = rows * n * 2 + rows * 2
+    return {"bytes": nbytes, "es_rowmax_GBps": round(nbytes / ours.mean_ms() / 1e6, 1),
+            "torch_amax_GBps": round(nbytes / lib.mean_ms() / 1e6, 1)}
+
+
 def run_copy(km, steps, warmup):
     """A plain copy of known size (1-D touch without castable, 512 MiB in, 512 MiB out): the
     yardstick the FETCH_SIZE / WRITE_SIZE counters are scaled by."""
@@ -474,6 +565,7 @@ def main():
         torch.cuda.empty_cache()
     if args.workload == "all":
         others["mfma_f16_register_ceiling"] = run_mfma_peak(km)
+        others["read_only_1GiB"] = run_read_ceiling(km, args.steps, args.warmup)
     if args.workload in ("llama", "all"):
         others["llama7b_contractions"] = run_llama_contractions(km, max(args.steps // 5, 3),
                                                                 max(args.warmup // 5, 1))

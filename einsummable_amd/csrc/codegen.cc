@@ -656,8 +656,13 @@ cg_kernel_t gen_reduce_row(einsummable_t const& e, int max_vec)
     s << "                const idx_t vv = v0 + (idx_t)u * TEAM;\n";
     s << "                if (vv < nvec) {\n";
     s << "                    idx_t ar = vv * V;\n";
-    s << "                    const idx_t g" << (R - 1) << " = ar % " << g.P(p_shape[R - 1]) << ";\n";
-    if (R - 1 > O) s << "                    ar /= " << g.P(p_shape[R - 1]) << ";\n";
+    if (R - 1 > O) {
+        s << "                    const idx_t g" << (R - 1) << " = ar % " << g.P(p_shape[R - 1]) << ";\n";
+        s << "                    ar /= " << g.P(p_shape[R - 1]) << ";\n";
+    } else {
+        // a single aggregated mode: the flat index is the mode's index
+        s << "                    const idx_t g" << (R - 1) << " = ar;\n";
+    }
     for (int m = R - 2; m > O; --m) {
         s << "                    const idx_t g" << m << " = ar % " << g.P(p_shape[m]) << ";\n";
         s << "                    ar /= " << g.P(p_shape[m]) << ";\n";

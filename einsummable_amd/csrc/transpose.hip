@@ -36,6 +36,98 @@ struct transpose_args_t {
     int64_t     bsi[MAXB], bso[MAXB];
 };
 
+// Tile origin and batch offsets of a workgroup; false when the workgroup has no tile.
+template <int EDGE>
+__device__ __forceinline__ bool locate(transpose_args_t const& a, uint32_t& i0, uint32_t& o0,
+                                       int64_t& off_i, int64_t& off_o)
+{
+    uint64_t const linear = uint64_t(blockIdx.y) * gridDim.x + blockIdx.x;
+    if (linear >= a.n_blocks) return false;  // uniform over the workgroup
+    uint32_t t = uint32_t(linear);
+    uint32_t const ti = t % a.tiles_i;
+    t /= a.tiles_i;
+    uint32_t const to = t % a.tiles_o;
+    uint32_t bidx = t / a.tiles_o;
+    off_i = 0;
+    off_o = 0;
+#pragma unroll
+    for (int d = 0; d != MAXB; ++d) {
+        if (d < int(a.nb)) {
+            uint32_t q = bidx / a.bsize[d];
+            uint32_t r = bidx - q * a.bsize[d];
+            off_i += int64_t(r) * a.bsi[d];
+            off_o += int64_t(r) * a.bso[d];
+            bidx = q;
+        }
+    }
+    i0 = ti * EDGE;
+    o0 = to * EDGE;
+    return true;
+}
+
+// The same tile with 16-byte global accesses on both sides: a lane loads V = 16 / sizeof(T)
+// consecutive elements of an input row and, after the turn through LDS, stores V consecutive
+// elements of an output row.  Needs every row start on both sides 16-byte aligned (strides,
+// batch offsets, extents and base pointers: checked on the host).
+// The tile edge is 128 for 2-byte elements (256-byte row segments), 64 otherwise.
+template <typename T>
+struct vec_tile_t {
+    static constexpr int edge = sizeof(T) == 2 ? 128 : 64;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_vec_kernel(transpose_args_t a)
+{
+    constexpr int TT = vec_tile_t<T>::edge;
+    constexpr int V = 16 / int(sizeof(T));
+    constexpr int LPR = TT / V;      // lanes per tile row
+    constexpr int RPP = 256 / LPR;   // tile rows per pass of the workgroup
+    // pitch: an odd number of 4-byte words, so that a column walks over all banks
+    constexpr int PITCH = sizeof(T) == 2 ? TT + 2 : TT + 1;
+    typedef T vecT __attribute__((ext_vector_type(V)));
+    __shared__ T tile[TT * PITCH];
+
+    uint32_t i0, o0;
+    int64_t  off_i, off_o;
+    if (!locate<TT>(a, i0, o0, off_i, off_o)) return;
+    T const* const in = static_cast<T const*>(a.in) + off_i;
+    T* const       out = static_cast<T*>(a.out) + off_o;
+    uint32_t const col = (threadIdx.x % LPR) * V;
+    uint32_t const row = threadIdx.x / LPR;
+
+#pragma unroll
+    for (int p = 0; p != TT / RPP; ++p) {
+        uint32_t const ol = row + p * RPP;
+        uint32_t const o = o0 + ol, i = i0 + col;
+        if (o < a.n_o && i < a.n_i) {  // n_i is a multiple of V: a started vector is whole
+            vecT v = __builtin_nontemporal_load(
+                reinterpret_cast<vecT const*>(in + int64_t(o) * a.si_o + i));
+            if constexpr (sizeof(T) == 2) {
+                typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+                u32x4 w = __builtin_bit_cast(u32x4, v);
+                uint32_t* dst = reinterpret_cast<uint32_t*>(&tile[ol * PITCH + col]);
+#pragma unroll
+                for (int j = 0; j != 4; ++j) dst[j] = w[j];
+            } else {
+#pragma unroll
+                for (int j = 0; j != V; ++j) tile[ol * PITCH + col + j] = v[j];
+            }
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int p = 0; p != TT / RPP; ++p) {
+        uint32_t const il = row + p * RPP;
+        uint32_t const i = i0 + il, o = o0 + col;
+        if (i < a.n_i && o < a.n_o) {
+            vecT v;
+#pragma unroll
+            for (int j = 0; j != V; ++j) v[j] = tile[(col + j) * PITCH + il];
+            __builtin_nontemporal_store(v, reinterpret_cast<vecT*>(out + int64_t(i) * a.so_i + o));
+        }
+    }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void transpose_kernel(transpose_args_t a)
 {
@@ -87,28 +179,50 @@ __global__ __launch_bounds__(256) void transpose_kernel(transpose_args_t a)
 struct transpose_plan_t : plan_t {
     transpose_args_t args;
     int              elem_size;
-    uint64_t         blocks;
+    uint64_t         batch;
+    bool             vec_ok;  // extents, strides and batch offsets keep rows 16-byte aligned
 
     void run(hipStream_t stream, void* out, void const* const* inns, void*, uint64_t) const override
     {
         transpose_args_t a = args;
         a.in = inns[0];
         a.out = out;
+        bool const aligned = reinterpret_cast<uintptr_t>(a.in) % 16 == 0 &&
+                             reinterpret_cast<uintptr_t>(a.out) % 16 == 0;
+        bool const vec = vec_ok && aligned;
+        uint32_t const edge = vec && elem_size == 2 ? 128 : 64;
+        a.tiles_i = (a.n_i + edge - 1) / edge;
+        a.tiles_o = (a.n_o + edge - 1) / edge;
+        uint64_t const blocks = uint64_t(a.tiles_i) * a.tiles_o * batch;
         a.n_blocks = blocks;
         // a grid dimension times the block size must stay below 2^32
         unsigned gx = unsigned(std::min<uint64_t>(blocks, 1ull << 22));
         unsigned gy = unsigned((blocks + gx - 1) / gx);
         dim3     grid(gx, gy), block(256);
-        switch (elem_size) {
-            case 2:
-                hipLaunchKernelGGL((transpose_kernel<uint16_t>), grid, block, 0, stream, a);
-                break;
-            case 4:
-                hipLaunchKernelGGL((transpose_kernel<uint32_t>), grid, block, 0, stream, a);
-                break;
-            default:
-                hipLaunchKernelGGL((transpose_kernel<uint64_t>), grid, block, 0, stream, a);
-                break;
+        if (vec) {
+            switch (elem_size) {
+                case 2:
+                    hipLaunchKernelGGL((transpose_vec_kernel<uint16_t>), grid, block, 0, stream, a);
+                    break;
+                case 4:
+                    hipLaunchKernelGGL((transpose_vec_kernel<uint32_t>), grid, block, 0, stream, a);
+                    break;
+                default:
+                    hipLaunchKernelGGL((transpose_vec_kernel<uint64_t>), grid, block, 0, stream, a);
+                    break;
+            }
+        } else {
+            switch (elem_size) {
+                case 2:
+                    hipLaunchKernelGGL((transpose_kernel<uint16_t>), grid, block, 0, stream, a);
+                    break;
+                case 4:
+                    hipLaunchKernelGGL((transpose_kernel<uint32_t>), grid, block, 0, stream, a);
+                    break;
+                default:
+                    hipLaunchKernelGGL((transpose_kernel<uint64_t>), grid, block, 0, stream, a);
+                    break;
+            }
         }
         hipError_t err = hipGetLastError();
         if (err != hipSuccess) {
@@ -173,11 +287,22 @@ std::shared_ptr<plan_t> plan_transpose(einsummable_t const& e, int)
         batch *= e.join_shape[m];
         ++a.nb;
     }
-    p->blocks = uint64_t(a.tiles_i) * a.tiles_o * batch;
-    if (p->blocks >= (1ull << 31) || batch >= (1ull << 31)) return nullptr;
+    p->batch = batch;
+    if (uint64_t(a.tiles_i) * a.tiles_o * batch >= (1ull << 31) || batch >= (1ull << 31)) {
+        return nullptr;
+    }
     p->elem_size = int(dtype_size(e.out_dtype()));
+    {
+        int64_t const V = 16 / p->elem_size;
+        bool ok = a.n_i % V == 0 && a.n_o % V == 0 && a.si_o % V == 0 && a.so_i % V == 0;
+        for (uint32_t d = 0; d != a.nb; ++d) ok = ok && a.bsi[d] % V == 0 && a.bso[d] % V == 0;
+        p->vec_ok = ok;
+    }
     p->workspace_bytes = 0;
-    p->description = "transpose_lds tile=64x64 batch=" + std::to_string(batch);
+    p->description = std::string("transpose_lds tile=") +
+                     (p->vec_ok && p->elem_size == 2 ? "128x128 " : "64x64 ") +
+                     (p->vec_ok ? "vec16 " : "") +
+                     "batch=" + std::to_string(batch);
     return p;
 }
 

@@ -54,3 +54,35 @@ def test_kernel_choice(km):
     km.build(e2)
     assert km.describe(e1).startswith("elementwise")
     assert km.describe(e2).startswith("transpose_lds")
+
+
+@pytest.mark.parametrize("dt,npdt", [("f16", np.float16), ("f32", np.float32), ("f64", np.float64),
+                                     ("c64", np.complex64)])
+def test_transposes_with_16_byte_rows_use_vector_accesses(km, dt, npdt):
+    r = rng(51)
+    v = 16 // np.dtype(npdt).itemsize
+    for shape, perm in [((9 * v, 17 * v), (1, 0)), ((3, 9 * v, 17 * v), (0, 2, 1)),
+                        ((8 * v, 3, 5, 8 * v), (3, 1, 2, 0)), ((2 * v, 7, 11 * v), (2, 1, 0)),
+                        ((64, 64), (1, 0)), ((128, 192), (1, 0))]:
+        x = normal(r, int(np.prod(shape)), npdt).reshape(shape)
+        e = permute_einsummable(shape, perm, dt)
+        got = run_einsummable(km, e, [x])
+        assert "vec16" in km.describe(e), km.describe(e)
+        want = np.ascontiguousarray(np.transpose(x, perm)).reshape(-1)
+        assert_bits_equal(got, want, "permute %s %s" % (shape, perm))
+
+
+def test_vector_transpose_falls_back_when_a_buffer_is_misaligned(km):
+    import torch
+    from helpers import stream_handle
+
+    x = normal(rng(52), 72 * 136, np.float16).reshape(72, 136)
+    e = permute_einsummable((72, 136), (1, 0), "f16")
+    km.build(e)
+    din = torch.zeros(72 * 136 + 8, dtype=torch.float16, device="cuda")
+    dout = torch.zeros(72 * 136 + 8, dtype=torch.float16, device="cuda")
+    din[1:1 + 72 * 136] = torch.from_numpy(x.reshape(-1)).cuda()
+    km(e, stream_handle(), dout.data_ptr() + 6, [din.data_ptr() + 2])
+    torch.cuda.synchronize()
+    got = dout[3:3 + 72 * 136].cpu().numpy()
+    assert_bits_equal(got, np.ascontiguousarray(x.T).reshape(-1), "misaligned transpose")
