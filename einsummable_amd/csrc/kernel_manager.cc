@@ -257,65 +257,162 @@ void kernel_manager_t::touch_batch(std::vector<touch_t> const& touches_, hipStre
             s *= ts[0].selection[d].d_out;
         }
     }
-    for (size_t first = 0; first < n; first += TOUCH_BATCH_MAX) {
-        size_t const  cnt = std::min<size_t>(TOUCH_BATCH_MAX, n - first);
-        touch_batch_t b;
-        b.n = int(cnt);
-        b.vec = wide ? vmax : 1;
-        b.aligned = (wide && aligned) ? 1 : 0;
-        b.any_castable = 0;
-        uint64_t lo[4] = {0, 0, 0, 0}, hi[4] = {1, 1, 1, 1};
-        for (int s = 0; s != 4; ++s) {
-            int d = r - 4 + s;
-            if (d < 0) continue;
-            lo[s] = ~0ull;
-            hi[s] = 0;
+    // every touch as a four-dimensional window of the output
+    std::vector<touch_item_t> items(n);
+    for (size_t i = 0; i != n; ++i) {
+        touch_t const& t = ts[i];
+        touch_item_t&  it = items[i];
+        it.inn = inns[i];
+        it.op = t.castable ? 1 + int(t.castable.value()) : 0;
+        it.base_inn = 0;
+        uint64_t si = 1;
+        uint64_t str_i[4] = {0, 0, 0, 0};
+        for (int d = r - 1; d >= 0; --d) {
+            str_i[d] = si;
+            it.base_inn += t.selection[d].offset_inn * si;
+            si *= t.selection[d].d_inn;
         }
-        for (size_t i = 0; i != cnt; ++i) {
-            touch_t const& t = ts[first + i];
-            touch_item_t&  it = b.items[i];
-            it.inn = inns[first + i];
-            it.op = t.castable ? 1 + int(t.castable.value()) : 0;
-            it.pad_ = 0;
-            if (it.op) b.any_castable = 1;
-            it.base_inn = 0;
-            uint64_t si = 1;
-            uint64_t str_i[4] = {0, 0, 0, 0};
-            for (int d = r - 1; d >= 0; --d) {
-                str_i[d] = si;
-                it.base_inn += t.selection[d].offset_inn * si;
-                si *= t.selection[d].d_inn;
+        for (int s = 0; s != 4; ++s) {
+            int d = r - 4 + s;  // dimension feeding slot s
+            if (d >= 0) {
+                it.lo[s] = uint32_t(t.selection[d].offset_out);
+                it.size[s] = uint32_t(t.selection[d].size);
+                if (s < 3) it.str_inn[s] = str_i[d];
+            } else {
+                it.lo[s] = 0;
+                it.size[s] = 1;
+                if (s < 3) it.str_inn[s] = 0;
             }
+        }
+        // input vectors line up with output vectors when the window's origin has the same
+        // phase in both tensors and every input row starts on a vector boundary
+        bool v = wide && reinterpret_cast<uintptr_t>(inns[i]) % 16 == 0 &&
+                 it.base_inn % uint64_t(vmax) == it.lo[3] % uint32_t(vmax);
+        for (int s = 0; s != 3; ++s) v = v && (it.size[s] == 1 || it.str_inn[s] % uint64_t(vmax) == 0);
+        it.vec_inn = v ? 1 : 0;
+    }
+    uint64_t out_str4[3];
+    for (int s = 0; s != 3; ++s) {
+        int d = r - 4 + s;
+        out_str4[s] = d >= 0 ? out_str[d] : 0;
+    }
+    auto overlap = [](touch_item_t const& x, touch_item_t const& y) {
+        for (int s = 0; s != 4; ++s) {
+            if (x.lo[s] + uint64_t(x.size[s]) <= y.lo[s] || y.lo[s] + uint64_t(y.size[s]) <= x.lo[s]) {
+                return false;
+            }
+        }
+        return true;
+    };
+
+    // Two ways to keep the sequential result.  Windows that mostly lie side by side are
+    // sorted into levels (a touch goes one level above the last earlier touch it overlaps);
+    // a level's windows are disjoint and run as one launch, each streaming at full width.
+    // Windows stacked on top of each other (the fan-in of partial sums) are folded by the
+    // owner of each output vector instead, which reads and writes the output once per launch.
+    constexpr size_t SPAN = 2048;  // the level search is quadratic: bounded spans of the list
+    for (size_t span0 = 0; span0 < n; span0 += SPAN) {
+        size_t const span_n = std::min(SPAN, n - span0);
+        uint64_t     blo[4], bhi[4];
+        for (int s = 0; s != 4; ++s) {
+            blo[s] = ~0ull;
+            bhi[s] = 0;
+        }
+        double span_volume = 0;
+        for (size_t i = span0; i != span0 + span_n; ++i) {
+            double vol = 1;
             for (int s = 0; s != 4; ++s) {
-                int d = r - 4 + s;  // dimension feeding slot s
-                if (d >= 0) {
-                    it.lo[s] = uint32_t(t.selection[d].offset_out);
-                    it.size[s] = uint32_t(t.selection[d].size);
-                    if (s < 3) it.str_inn[s] = str_i[d];
-                    lo[s] = std::min<uint64_t>(lo[s], t.selection[d].offset_out);
-                    hi[s] = std::max<uint64_t>(hi[s], t.selection[d].offset_out + t.selection[d].size);
-                } else {
-                    it.lo[s] = 0;
-                    it.size[s] = 1;
-                    if (s < 3) it.str_inn[s] = 0;
+                blo[s] = std::min<uint64_t>(blo[s], items[i].lo[s]);
+                bhi[s] = std::max<uint64_t>(bhi[s], items[i].lo[s] + uint64_t(items[i].size[s]));
+                vol *= double(items[i].size[s]);
+            }
+            span_volume += vol;
+        }
+        double box_volume = 1;
+        for (int s = 0; s != 4; ++s) box_volume *= double(bhi[s] - blo[s]);
+        bool const stacked = span_volume >= 4.0 * box_volume;
+
+        if (!stacked) {
+            std::vector<int> level(span_n, 0);
+            int              top = 0;
+            for (size_t i = 0; i != span_n; ++i) {
+                for (size_t j = 0; j != i; ++j) {
+                    if (level[j] >= level[i] && overlap(items[span0 + i], items[span0 + j])) {
+                        level[i] = level[j] + 1;
+                    }
+                }
+                top = std::max(top, level[i]);
+            }
+            for (int l = 0; l <= top; ++l) {
+                touch_level_t b;
+                b.vec = wide ? vmax : 1;
+                for (int s = 0; s != 3; ++s) b.out_str[s] = out_str4[s];
+                b.n = 0;
+                b.max_vec = 0;
+                bool castable = false;
+                auto flush = [&]() {
+                    if (b.n == 0) return;
+                    launch_touch_level(b, esz, int(dt), castable, stream, out);
+                    hip_check(hipGetLastError(), "touch_batch launch");
+                    b.n = 0;
+                    b.max_vec = 0;
+                    castable = false;
+                };
+                for (size_t i = 0; i != span_n; ++i) {
+                    if (level[i] != l) continue;
+                    touch_item_t const& it = items[span0 + i];
+                    uint64_t const v = uint64_t(b.vec);
+                    uint64_t const vpr = (it.lo[3] + uint64_t(it.size[3]) - 1) / v - it.lo[3] / v + 1;
+                    uint64_t const nv = uint64_t(it.size[0]) * it.size[1] * it.size[2] * vpr;
+                    if (nv >= (1ull << 39)) {
+                        throw km_error(km_status::invalid, "touch_batch: window too large");
+                    }
+                    b.items[b.n++] = it;
+                    b.max_vec = std::max(b.max_vec, nv);
+                    castable = castable || it.op != 0;
+                    if (b.n == TOUCH_BATCH_MAX) flush();
+                }
+                flush();
+            }
+            continue;
+        }
+
+        for (size_t first = span0; first < span0 + span_n; first += TOUCH_BATCH_MAX) {
+            size_t const  cnt = std::min<size_t>(TOUCH_BATCH_MAX, span0 + span_n - first);
+            touch_batch_t b;
+            b.n = int(cnt);
+            b.vec = wide ? vmax : 1;
+            b.aligned = (wide && aligned) ? 1 : 0;
+            b.any_castable = 0;
+            uint64_t lo[4], hi[4];
+            for (int s = 0; s != 4; ++s) {
+                lo[s] = ~0ull;
+                hi[s] = 0;
+            }
+            for (size_t i = 0; i != cnt; ++i) {
+                touch_item_t const& it = items[first + i];
+                b.items[i] = it;
+                if (it.op) b.any_castable = 1;
+                for (int s = 0; s != 4; ++s) {
+                    lo[s] = std::min<uint64_t>(lo[s], it.lo[s]);
+                    hi[s] = std::max<uint64_t>(hi[s], it.lo[s] + uint64_t(it.size[s]));
                 }
             }
+            lo[3] = lo[3] / uint64_t(b.vec) * uint64_t(b.vec);
+            hi[3] = (hi[3] + uint64_t(b.vec) - 1) / uint64_t(b.vec) * uint64_t(b.vec);
+            b.n_vec = 1;
+            for (int s = 0; s != 4; ++s) {
+                b.box_lo[s] = uint32_t(lo[s]);
+                b.box_size[s] = uint32_t(hi[s] - lo[s]);
+                b.n_vec *= (s == 3) ? (hi[s] - lo[s]) / uint64_t(b.vec) : (hi[s] - lo[s]);
+                if (s < 3) b.out_str[s] = out_str4[s];
+            }
+            if (b.n_vec >= (1ull << 40)) {
+                throw km_error(km_status::invalid, "touch_batch: bounding box too large");
+            }
+            launch_touch_batch(b, esz, int(dt), stream, out);
+            hip_check(hipGetLastError(), "touch_batch launch");
         }
-        lo[3] = lo[3] / uint64_t(b.vec) * uint64_t(b.vec);
-        hi[3] = (hi[3] + uint64_t(b.vec) - 1) / uint64_t(b.vec) * uint64_t(b.vec);
-        b.n_vec = 1;
-        for (int s = 0; s != 4; ++s) {
-            b.box_lo[s] = uint32_t(lo[s]);
-            b.box_size[s] = uint32_t(hi[s] - lo[s]);
-            b.n_vec *= (s == 3) ? (hi[s] - lo[s]) / uint64_t(b.vec) : (hi[s] - lo[s]);
-            int d = r - 4 + s;
-            if (s < 3) b.out_str[s] = d >= 0 ? out_str[d] : 0;
-        }
-        if (b.n_vec >= (1ull << 40)) {
-            throw km_error(km_status::invalid, "touch_batch: bounding box too large");
-        }
-        launch_touch_batch(b, esz, int(dt), stream, out);
-        hip_check(hipGetLastError(), "touch_batch launch");
     }
 }
 

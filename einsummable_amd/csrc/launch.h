@@ -35,7 +35,8 @@ struct touch_item_t {
     uint32_t    lo[4];       // window origin in the output
     uint32_t    size[4];     // window extents
     int         op;          // 0 copy, 1 add, 2 mul, 3 min, 4 max
-    int         pad_;
+    int         vec_inn;     // level kernel: the input can be read as 16-byte vectors that
+                             // line up with the output's vectors
 };
 
 constexpr int TOUCH_BATCH_MAX = 32;  // items per launch (kernel-argument budget)
@@ -54,6 +55,21 @@ struct touch_batch_t {
 
 void launch_touch_batch(touch_batch_t const& b, int elem_size, int dtype_code, hipStream_t stream,
                         void* out);
+
+// A set of touches into one output tensor whose windows are pairwise disjoint: one launch,
+// blockIdx.y selects the touch, every touch streams through its own window.  Output vectors
+// that a window covers only in part are written element by element, so that windows sharing
+// a vector never write each other's elements.
+struct touch_level_t {
+    int          n;
+    int          vec;         // elements per output vector
+    uint64_t     out_str[3];  // element strides of the output's outer dimensions
+    uint64_t     max_vec;     // largest number of vectors any item covers
+    touch_item_t items[TOUCH_BATCH_MAX];
+};
+
+void launch_touch_level(touch_level_t const& b, int elem_size, int dtype_code, bool any_castable,
+                        hipStream_t stream, void* out);
 
 void launch_fill_constant(int elem_size, uint64_t bits, uint64_t nelem, hipStream_t stream,
                           void* out);

@@ -303,6 +303,91 @@ void launch_touch_batch_t(touch_batch_t const& b, hipStream_t stream, void* out)
     }
 }
 
+// ---- touches with pairwise disjoint windows, one per blockIdx.y
+
+template <typename T>
+__device__ __forceinline__ T apply_dyn(int op, T out, T inn)
+{
+    switch (op) {
+        case OP_COPY:
+            return inn;
+        case OP_ADD:
+            return apply<OP_ADD, T>(out, inn);
+        case OP_MUL:
+            return apply<OP_MUL, T>(out, inn);
+        case OP_MIN:
+            if constexpr (!(sizeof(T) == 8 && alignof(T) == 4)) return apply<OP_MIN, T>(out, inn);
+            return inn;
+        default:
+            if constexpr (!(sizeof(T) == 8 && alignof(T) == 4)) return apply<OP_MAX, T>(out, inn);
+            return inn;
+    }
+}
+
+template <typename T, int V>
+__global__ __launch_bounds__(256) void touch_level_kernel(touch_level_t b, T* __restrict__ out)
+{
+    using vt = vec_t<T, V>;
+    touch_item_t const& it = b.items[blockIdx.y];  // uniform index: scalar loads
+    uint32_t const lo3 = it.lo[3], sz3 = it.size[3];
+    // the output vectors that the window's rows overlap
+    uint32_t const v_first = lo3 / V;
+    uint32_t const vpr = (lo3 + sz3 - 1) / V - v_first + 1;
+    uint64_t const n_vec = uint64_t(it.size[0]) * it.size[1] * it.size[2] * vpr;
+    uint64_t const idx = uint64_t(blockIdx.x) * 256 + threadIdx.x;
+    if (idx >= n_vec) return;
+    uint64_t       r = idx / vpr;
+    uint32_t const c3 = (v_first + uint32_t(idx - r * vpr)) * V;
+    uint32_t const d2 = uint32_t(r % it.size[2]);
+    r /= it.size[2];
+    uint32_t const d1 = uint32_t(r % it.size[1]);
+    uint32_t const d0 = uint32_t(r / it.size[1]);
+    uint64_t const oo = (it.lo[0] + d0) * b.out_str[0] + (it.lo[1] + d1) * b.out_str[1] +
+                        (it.lo[2] + d2) * b.out_str[2] + c3;
+    T const* const src = static_cast<T const*>(it.inn) + it.base_inn + d0 * it.str_inn[0] +
+                         d1 * it.str_inn[1] + d2 * it.str_inn[2];
+    int const  op = it.op;
+    bool const full = c3 >= lo3 && c3 + V <= lo3 + sz3;
+    if (full) {
+        vt x;
+        if (it.vec_inn) {
+            x = *reinterpret_cast<vt const*>(src + (c3 - lo3));
+        } else {
+#pragma unroll
+            for (int j = 0; j != V; ++j) x.v[j] = src[c3 - lo3 + uint32_t(j)];
+        }
+        if (op != OP_COPY) {
+            vt const y = *reinterpret_cast<vt const*>(out + oo);
+#pragma unroll
+            for (int j = 0; j != V; ++j) x.v[j] = apply_dyn<T>(op, y.v[j], x.v[j]);
+        }
+        *reinterpret_cast<vt*>(out + oo) = x;
+    } else {
+#pragma unroll
+        for (int j = 0; j != V; ++j) {
+            uint32_t const d3 = c3 + uint32_t(j) - lo3;  // wraps below the window
+            if (d3 < sz3) {
+                T const x = src[d3];
+                out[oo + j] = op == OP_COPY ? x : apply_dyn<T>(op, out[oo + j], x);
+            }
+        }
+    }
+}
+
+template <typename T>
+void launch_touch_level_t(touch_level_t const& b, hipStream_t stream, void* out)
+{
+    constexpr int VMAX = 16 / sizeof(T);
+    dim3          grid(unsigned((b.max_vec + 255) / 256), unsigned(b.n));
+    if (b.vec == VMAX) {
+        hipLaunchKernelGGL((touch_level_kernel<T, VMAX>), grid, dim3(256), 0, stream, b,
+                           static_cast<T*>(out));
+    } else {
+        hipLaunchKernelGGL((touch_level_kernel<T, 1>), grid, dim3(256), 0, stream, b,
+                           static_cast<T*>(out));
+    }
+}
+
 // ---- fills
 
 template <int V>
@@ -418,6 +503,32 @@ void launch_touch_batch(touch_batch_t const& b, int elem_size, int dtype_code, h
             return launch_touch_batch_t<double>(b, stream, out);
         default:
             return launch_touch_batch_t<c64_t>(b, stream, out);
+    }
+}
+
+void launch_touch_level(touch_level_t const& b, int elem_size, int dtype_code, bool any_castable,
+                        hipStream_t stream, void* out)
+{
+    if (b.n == 0 || b.max_vec == 0) return;
+    if (!any_castable) {
+        switch (elem_size) {
+            case 2:
+                return launch_touch_level_t<uint16_t>(b, stream, out);
+            case 4:
+                return launch_touch_level_t<uint32_t>(b, stream, out);
+            default:
+                return launch_touch_level_t<uint64_t>(b, stream, out);
+        }
+    }
+    switch (dtype_code) {
+        case 0:
+            return launch_touch_level_t<_Float16>(b, stream, out);
+        case 1:
+            return launch_touch_level_t<float>(b, stream, out);
+        case 2:
+            return launch_touch_level_t<double>(b, stream, out);
+        default:
+            return launch_touch_level_t<c64_t>(b, stream, out);
     }
 }
 

@@ -174,6 +174,48 @@ def test_touch_batch_memory_movement_configuration(km):
     assert_bits_equal(to_host(d_out, np.float16), want, "64 accumulate touches, batched")
 
 
+@pytest.mark.parametrize("dt", [ea.F16, ea.F32, ea.C64])
+def test_touch_batch_disjoint_windows_that_share_output_vectors(km, dt):
+    """Windows laid side by side with odd widths: neighbours meet inside 16-byte output
+    vectors, and being disjoint they run in the same launch.  Each must leave the other's
+    elements alone."""
+    r = rng(60 + dt)
+    rows, cols = 37, 256
+    touches, blocks = [], []
+    c = 0
+    while c < cols:
+        w = min(int(r.randint(1, 23)), cols - c)
+        h = int(r.randint(1, rows + 1))
+        r0 = int(r.randint(0, rows - h + 1))
+        oi = int(r.randint(0, 5))
+        touches.append(ea.Touch([(h, rows, 0, r0, h), (w + oi + 2, cols, oi, c, w)],
+                                [None, "+", "x"][int(r.randint(0, 3))], dt))
+        blocks.append(normal(r, h * (w + oi + 2), NP[dt], 0.5))
+        c += w
+    out0 = normal(r, rows * cols, NP[dt], 0.5)
+    want = _apply_sequentially(touches, blocks, out0)
+    d_out = to_device(out0)
+    d_blocks = [to_device(b) for b in blocks]
+    km.touch_batch(touches, stream_handle(), d_out.data_ptr(), [b.data_ptr() for b in d_blocks])
+    assert_bits_equal(to_host(d_out, NP[dt]), want, "side-by-side windows")
+
+
+@pytest.mark.parametrize("dt", [ea.F16, ea.F32])
+def test_touch_batch_stacked_partial_sums(km, dt):
+    """The fan-in of partial sums: 40 inputs accumulated into the same window, in order."""
+    r = rng(70 + dt)
+    n, b = 96, 64
+    touches = [ea.Touch([(b, n, 0, 16, b), (b, n, 0, 8, b)], None if i == 0 else "+", dt)
+               for i in range(40)]
+    blocks = [normal(r, b * b, NP[dt]) for _ in touches]
+    out0 = normal(r, n * n, NP[dt])
+    want = _apply_sequentially(touches, blocks, out0)
+    d_out = to_device(out0)
+    d_blocks = [to_device(x) for x in blocks]
+    km.touch_batch(touches, stream_handle(), d_out.data_ptr(), [x.data_ptr() for x in d_blocks])
+    assert_bits_equal(to_host(d_out, NP[dt]), want, "stacked partial sums")
+
+
 def test_touch_batch_errors(km):
     d = to_device(np.zeros(64, np.float32))
     a = ea.Touch([(4, 8, 0, 0, 4)], None, ea.F32)
