@@ -394,9 +394,17 @@ template <int V>
 __global__ __launch_bounds__(256) void fill_constant_kernel(uint64_t n_vec, vec_t<uint32_t, V> pat,
                                                             vec_t<uint32_t, V>* __restrict__ out)
 {
-    uint64_t i = uint64_t(blockIdx.x) * 256 + threadIdx.x;
-    uint64_t stride = uint64_t(gridDim.x) * 256;
-    for (; i < n_vec; i += stride) out[i] = pat;
+    // one vector per thread; fills larger than the caches bypass them
+    uint64_t const i = uint64_t(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= n_vec) return;
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    static_assert(V == 4, "16-byte pattern");
+    u32x4 const v = {pat.v[0], pat.v[1], pat.v[2], pat.v[3]};
+    if (n_vec >= (4u << 20)) {
+        __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(out) + i);
+    } else {
+        reinterpret_cast<u32x4*>(out)[i] = v;
+    }
 }
 
 template <typename T>
@@ -563,7 +571,8 @@ void launch_fill_constant(int elem_size, uint64_t bits, uint64_t nelem, hipStrea
     };
     edge(0, head_bytes / uint64_t(elem_size));
     if (body_vec) {
-        unsigned blocks = (unsigned)std::min<uint64_t>((body_vec + 255) / 256, 16384);
+        if (body_vec >= (1ull << 39)) return;  // beyond any device memory
+        unsigned blocks = unsigned((body_vec + 255) / 256);
         hipLaunchKernelGGL((fill_constant_kernel<4>), dim3(blocks), dim3(256), 0, stream, body_vec,
                            pat,
                            reinterpret_cast<vec_t<uint32_t, 4>*>(static_cast<char*>(out) +
