@@ -261,9 +261,13 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
     constexpr int LOADS = NLA + NLB;
     // side work per matrix instruction: step 0 spreads the reads over all of them, step 1
     // over all but the first (which is followed by the barrier)
-    constexpr int R0 = (READS + PAIRS - 1) / PAIRS;
-    constexpr int R1 = (READS + PAIRS - 2) / (PAIRS - 1);
-    constexpr int L1 = (LOADS + PAIRS - 2) / (PAIRS - 1);
+    // A 16-byte chunk feeds tr::SUB matrix instructions (4 for 4-byte elements).  They go
+    // round the accumulator tiles, so that consecutive instructions never depend on each
+    // other, and each carries its share of the side work.
+    constexpr int MMAS = PAIRS * tr::SUB;
+    constexpr int R0 = (READS + MMAS - 1) / MMAS;
+    constexpr int R1 = (READS + MMAS - 2) / (MMAS - 1);
+    constexpr int L1 = (LOADS + MMAS - 2) / (MMAS - 1);
 
     uint32_t const nk = a.K / BK;  // >= NS, no remainder (checked by the launcher)
 
@@ -290,30 +294,32 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
         uint32_t       ka = 0, kb = 0;
         if (ISSUE) k_offsets(kt + NS, ka, kb);
 #pragma unroll
-        for (int p = 0; p != PAIRS; ++p) {
-            tr::mma(acc[p / TN][p % TN], fb[0][p % TN], fa[0][p / TN]);
+        for (int q = 0; q != MMAS; ++q) {
+            int const p = q % PAIRS;
+            tr::mma_sub(acc[p / TN][p % TN], fb[0][p % TN], fa[0][p / TN], q / PAIRS);
 #pragma unroll
-            for (int r = p * R0; r != (p + 1) * R0; ++r) {
+            for (int r = q * R0; r != (q + 1) * R0; ++r) {
                 if (r < READS) read_frag(cur, 1, r, fa[1], fb[1]);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
-        for (int p = 0; p != PAIRS; ++p) {
-            tr::mma(acc[p / TN][p % TN], fb[1][p % TN], fa[1][p / TN]);
+        for (int q = 0; q != MMAS; ++q) {
+            int const p = q % PAIRS;
+            tr::mma_sub(acc[p / TN][p % TN], fb[1][p % TN], fa[1][p / TN], q / PAIRS);
             if (YOUNGER >= 0) {
-                if (p == 0) {
+                if (q == 0) {
                     // this wave's part of slice kt+1 has landed and its reads of this stage
                     // are complete; after the barrier that holds for the whole workgroup
                     wait_loads_and_lds<(YOUNGER < 0 ? 0 : YOUNGER) * LOADS>();
                     __builtin_amdgcn_s_barrier();
                 } else {
 #pragma unroll
-                    for (int r = (p - 1) * R1; r != p * R1; ++r) {
+                    for (int r = (q - 1) * R1; r != q * R1; ++r) {
                         if (r < READS) read_frag(nxt, 0, r, fa[0], fb[0]);
                     }
 #pragma unroll
-                    for (int r = (p - 1) * L1; r != p * L1; ++r) {
+                    for (int r = (q - 1) * L1; r != q * L1; ++r) {
                         if (ISSUE && r < LOADS) issue(kt + NS, r, ka, kb);
                     }
                 }

@@ -107,6 +107,13 @@ struct traits_t<_Float16> {
         return (i / 4) * 8 + (lane / 32) * 4 + (i % 4);
     }
     static constexpr bool QUAD = true;  // registers 4q..4q+3 hold four consecutive rows
+    // matrix instructions per 16-byte operand chunk, and the t-th of them
+    static constexpr int SUB = 1;
+    __device__ static __forceinline__ void mma_sub(acc_t& acc, chunk_t const& row,
+                                                   chunk_t const& col, int)
+    {
+        mma(acc, row, col);
+    }
 };
 
 template <>
@@ -131,6 +138,14 @@ struct traits_t<float> {
         return (i / 4) * 8 + (lane / 32) * 4 + (i % 4);
     }
     static constexpr bool QUAD = true;  // registers 4q..4q+3 hold four consecutive rows
+    static constexpr int SUB = 4;
+    __device__ static __forceinline__ void mma_sub(acc_t& acc, chunk_t const& row,
+                                                   chunk_t const& col, int t)
+    {
+        float4_t r = __builtin_bit_cast(float4_t, row);
+        float4_t c = __builtin_bit_cast(float4_t, col);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(r[t], c[t], acc, 0, 0, 0);
+    }
 };
 
 template <>
