@@ -432,6 +432,29 @@ def run_c5(km, steps, warmup):
         graph.replay()
     torch.cuda.synchronize()
     graph_ms = (time.perf_counter() - t0) / steps * 1e3
+    # the same layer through the exec-node layer: one arena, dependencies from the memory
+    # ranges, nodes placed on 1 / 2 / 4 streams, one burst of launches per layer
+    del graph
+    exec_ms = {}
+    state = {name: run.mem[name].clone() for name in g.inputs}
+    for ns in (1, 2, 4):
+        del run
+        torch.cuda.empty_cache()
+        run = None
+        from einsummable_amd.llama_layer import ArenaRunner
+        par = ArenaRunner(km, g, ns)
+        for name, t in state.items():
+            par.view(name).copy_(t)
+        for _ in range(max(warmup, 2)):
+            par.run()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            par.run()
+        torch.cuda.synchronize()
+        exec_ms[str(ns)] = round((time.perf_counter() - t0) / steps * 1e3, 4)
+        run = par
+    del par, run, state
     rows = []
     for n, t in zip(g.nodes, timers):
         rows.append((n["label"], n["kind"], t.mean_ms(), n.get("flops", 0)))
@@ -439,6 +462,7 @@ def run_c5(km, steps, warmup):
     top = sorted(rows, key=lambda r: -r[2])[:12]
     return {"node": "c5 LLaMA-7B decoder layer, b=1 s=2048 f16", "layer_ms": round(wall_ms, 4),
             "layer_hipgraph_ms": round(graph_ms, 4),
+            "layer_exec_graph_ms_by_streams": exec_ms,
             "layer_with_node_events_ms": round(timed_wall_ms, 4), "nodes": len(rows), "sum_node_ms": round(sum(r[2] for r in rows), 4),
             "contraction_ms": round(gemm_ms, 4),
             "contraction_TFLOPs": round(g.contraction_flops() / gemm_ms / 1e9, 1),

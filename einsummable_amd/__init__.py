@@ -8,6 +8,7 @@ nothing of its own: every call goes straight to the library and fails loudly whe
 library is missing.
 """
 from .km import (  # noqa: F401
+    ApplyGraph,
     C64,
     F16,
     F32,

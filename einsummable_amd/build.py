@@ -19,6 +19,7 @@ SOURCES = [
     "ir.cc",
     "kernel_manager.cc",
     "c_api.cc",
+    "exec_graph.cc",
     "codegen.cc",
     "touch.hip",
     "transpose.hip",

@@ -4,6 +4,7 @@
 #include "../../include/es_km.h"
 
 #include "codegen.h"
+#include "exec_graph.h"
 #include "gemm_kernel.h"
 #include "kernel_manager.h"
 
@@ -12,6 +13,11 @@
 struct es_km {
     std::unique_ptr<es::kernel_manager_t> km;
     std::string                           last_error;
+};
+
+struct es_km_graph {
+    es_km_t*                            owner;  // may be null (plan-only graph)
+    std::unique_ptr<es::apply_graph_t> graph;
 };
 
 namespace
@@ -351,4 +357,159 @@ double es_km_probe_mfma_f16(es_km_t* h, const void* operands, void* scratch, int
     return es::gemm::probe_mfma_f16(operands, scratch, blocks, iters,
                                     static_cast<hipStream_t>(stream));
 }
+
+// ---- exec-node layer (see exec_graph.h)
+
+es_km_graph_t* es_km_graph_create(es_km_t* h)
+{
+    try {
+        auto* g = new es_km_graph;
+        g->owner = h;
+        g->graph = std::make_unique<es::apply_graph_t>(h ? h->km.get() : nullptr);
+        return g;
+    } catch (std::exception const& e) {
+        err_slot(h) = e.what();
+        return nullptr;
+    }
+}
+
+void es_km_graph_destroy(es_km_graph_t* g) { delete g; }
+
+namespace
+{
+std::vector<es::mem_t> make_mems(const uint64_t* offsets, const uint64_t* sizes, int n)
+{
+    if (!offsets || !sizes || n < 1) throw es::ir_error("graph node: bad memory ranges");
+    std::vector<es::mem_t> m;
+    for (int i = 0; i != n; ++i) m.push_back(es::mem_t{offsets[i], sizes[i]});
+    return m;
+}
+std::vector<int> make_deps(const int* deps, int n)
+{
+    if (n < 0 || (n > 0 && !deps)) throw es::ir_error("graph node: bad dependency list");
+    return std::vector<int>(deps, deps + n);
+}
+}  // namespace
+
+int es_km_graph_add_einsummable(es_km_graph_t* g, const uint64_t* join_shape, int join_rank,
+                                const int* inns_flat, const int* inns_offsets, int n_inns,
+                                int out_rank, const char* join_text, char castable,
+                                const uint64_t* mem_offsets, const uint64_t* mem_sizes, int n_mems,
+                                const int* deps, int n_deps)
+{
+    return guarded(g ? g->owner : nullptr, [&]() -> int {
+        if (!g) throw es::ir_error("null graph");
+        check_descriptor(join_shape, join_rank, inns_flat, inns_offsets, n_inns, out_rank,
+                         join_text);
+        es::einsummable_t e = make_einsummable(join_shape, join_rank, inns_flat, inns_offsets,
+                                               n_inns, out_rank, join_text, castable);
+        return g->graph->add_einsummable(e, make_mems(mem_offsets, mem_sizes, n_mems),
+                                         make_deps(deps, n_deps));
+    });
+}
+
+int es_km_graph_add_touch(es_km_graph_t* g, const uint64_t* touchdims, int rank, char castable,
+                          int dtype, int group, const uint64_t* mem_offsets,
+                          const uint64_t* mem_sizes, const int* deps, int n_deps)
+{
+    return guarded(g ? g->owner : nullptr, [&]() -> int {
+        if (!g) throw es::ir_error("null graph");
+        if (!touchdims || rank < 1 || rank > 64) throw es::ir_error("touch: bad selection");
+        if (dtype < 0 || dtype > 3) throw es::ir_error("touch: bad dtype");
+        es::touch_t t;
+        t.dtype = es::dtype_t(dtype);
+        t.castable = es::castable_from_char(castable);
+        t.selection.resize(size_t(rank));
+        for (int i = 0; i != rank; ++i) {
+            const uint64_t* d = touchdims + 5 * i;
+            t.selection[size_t(i)] = es::touchdim_t{d[0], d[1], d[2], d[3], d[4]};
+        }
+        return g->graph->add_touch(t, group, make_mems(mem_offsets, mem_sizes, 2),
+                                   make_deps(deps, n_deps));
+    });
+}
+
+int es_km_graph_add_fill_constant(es_km_graph_t* g, int dtype, uint64_t value_bits,
+                                  uint64_t nelem, uint64_t offset, uint64_t size, const int* deps,
+                                  int n_deps)
+{
+    return guarded(g ? g->owner : nullptr, [&]() -> int {
+        if (!g) throw es::ir_error("null graph");
+        if (dtype < 0 || dtype > 3) throw es::ir_error("fill: bad dtype");
+        return g->graph->add_constant_fill(es::dtype_t(dtype), value_bits, nelem,
+                                           es::mem_t{offset, size}, make_deps(deps, n_deps));
+    });
+}
+
+int es_km_graph_add_fill_lowertri(es_km_graph_t* g, int dtype, uint64_t lower_bits,
+                                  uint64_t upper_bits, uint64_t nrow, uint64_t ncol, int64_t start,
+                                  uint64_t offset, uint64_t size, const int* deps, int n_deps)
+{
+    return guarded(g ? g->owner : nullptr, [&]() -> int {
+        if (!g) throw es::ir_error("null graph");
+        if (dtype < 0 || dtype > 3) throw es::ir_error("fill: bad dtype");
+        return g->graph->add_lowertri_fill(es::dtype_t(dtype), lower_bits, upper_bits, nrow, ncol,
+                                           start, es::mem_t{offset, size},
+                                           make_deps(deps, n_deps));
+    });
+}
+
+int es_km_graph_add_copy(es_km_graph_t* g, uint64_t dst_offset, uint64_t src_offset, uint64_t size,
+                         const int* deps, int n_deps)
+{
+    return guarded(g ? g->owner : nullptr, [&]() -> int {
+        if (!g) throw es::ir_error("null graph");
+        return g->graph->add_copy(es::mem_t{dst_offset, size}, es::mem_t{src_offset, size},
+                                  make_deps(deps, n_deps));
+    });
+}
+
+int es_km_graph_add_memory_dependencies(es_km_graph_t* g)
+{
+    return guarded(g ? g->owner : nullptr, [&]() -> int {
+        if (!g) throw es::ir_error("null graph");
+        g->graph->add_memory_dependencies();
+        return ES_KM_OK;
+    });
+}
+
+int es_km_graph_finalize(es_km_graph_t* g, int n_streams)
+{
+    return guarded(g ? g->owner : nullptr, [&]() -> int {
+        if (!g) throw es::ir_error("null graph");
+        g->graph->finalize(n_streams);
+        return ES_KM_OK;
+    });
+}
+
+int es_km_graph_run(es_km_graph_t* g, void* stream, void* arena)
+{
+    return guarded(g ? g->owner : nullptr, [&]() -> int {
+        if (!g) throw es::ir_error("null graph");
+        if (!arena) throw es::ir_error("graph run: null arena");
+        g->graph->run(static_cast<hipStream_t>(stream), arena);
+        return ES_KM_OK;
+    });
+}
+
+int es_km_graph_node_info(es_km_graph_t* g, int id, int* position, int* stream, int* deps, int cap,
+                          int* n_deps)
+{
+    return guarded(g ? g->owner : nullptr, [&]() -> int {
+        if (!g) throw es::ir_error("null graph");
+        if (id < 0 || id >= g->graph->n_nodes()) throw es::ir_error("graph: no such node");
+        if (position) *position = g->graph->position_of(id);
+        if (stream) *stream = g->graph->stream_of(id);
+        std::vector<int> const& d = g->graph->deps_of(id);
+        if (n_deps) *n_deps = int(d.size());
+        for (int i = 0; deps && i < cap && i < int(d.size()); ++i) deps[i] = d[size_t(i)];
+        return ES_KM_OK;
+    });
+}
+
+int es_km_graph_cross_stream_waits(es_km_graph_t* g)
+{
+    return g ? g->graph->n_cross_stream_waits() : ES_KM_ERR_INVALID;
+}
+
 }

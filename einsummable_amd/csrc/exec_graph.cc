@@ -1,0 +1,307 @@
+#include "exec_graph.h"
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+
+namespace es
+{
+namespace
+{
+
+void check(hipError_t err, const char* what)
+{
+    if (err != hipSuccess) {
+        throw km_error(km_status::device, std::string(what) + ": " + hipGetErrorString(err));
+    }
+}
+
+bool overlaps(mem_t const& a, mem_t const& b)
+{
+    return a.size != 0 && b.size != 0 && a.offset < b.offset + b.size &&
+           b.offset < a.offset + a.size;
+}
+
+}  // namespace
+
+apply_graph_t::apply_graph_t(kernel_manager_t* km) : km_(km) {}
+
+apply_graph_t::~apply_graph_t()
+{
+    for (size_t s = 1; s < streams_.size(); ++s) (void)hipStreamDestroy(streams_[s]);
+    for (hipEvent_t e : events_) (void)hipEventDestroy(e);
+    for (hipEvent_t e : joins_) (void)hipEventDestroy(e);
+    if (fork_) (void)hipEventDestroy(fork_);
+}
+
+int apply_graph_t::insert(node_t&& n, std::vector<int> const& deps)
+{
+    if (finalized_) throw km_error(km_status::invalid, "apply graph: already finalized");
+    int const id = int(nodes_.size());
+    for (int d : deps) {
+        // insertion order is the launch order, so a node can only wait for earlier ones
+        if (d < 0 || d >= id) {
+            throw km_error(km_status::invalid,
+                           "apply graph: node " + std::to_string(id) + " depends on node " +
+                               std::to_string(d) + ", which is not an earlier node");
+        }
+    }
+    n.deps = deps;
+    std::sort(n.deps.begin(), n.deps.end());
+    n.deps.erase(std::unique(n.deps.begin(), n.deps.end()), n.deps.end());
+    nodes_.push_back(std::move(n));
+    return id;
+}
+
+int apply_graph_t::add_einsummable(einsummable_t const& e, std::vector<mem_t> const& mems,
+                                   std::vector<int> const& deps)
+{
+    if (mems.size() != e.inns.size() + 1) {
+        throw km_error(km_status::inputs, "apply graph: einsummable with " +
+                                              std::to_string(e.inns.size()) + " inputs given " +
+                                              std::to_string(mems.size()) + " memory ranges");
+    }
+    node_t n;
+    n.kind = kind_t::einsummable;
+    n.e = e;
+    n.mems = mems;
+    return insert(std::move(n), deps);
+}
+
+int apply_graph_t::add_touch(touch_t const& t, int group, std::vector<mem_t> const& mems,
+                             std::vector<int> const& deps_)
+{
+    if (mems.size() != 2) {
+        throw km_error(km_status::inputs, "apply graph: a touch takes an output and an input");
+    }
+    t.validate();
+    node_t n;
+    n.kind = kind_t::touch;
+    n.touch = t;
+    n.group = group;
+    n.mems = mems;
+    std::vector<int> deps = deps_;
+    // A touch outside any group is the only writer of its bytes: a copy.  Inside a group
+    // the touches are serialised in insertion order and the first one initialises.
+    int previous = -1;
+    if (group >= 0) {
+        for (int i = int(nodes_.size()) - 1; i >= 0 && previous < 0; --i) {
+            if (nodes_[i].kind == kind_t::touch && nodes_[i].group == group) previous = i;
+        }
+    }
+    if (previous < 0) {
+        n.touch.castable = std::nullopt;
+    } else {
+        deps.push_back(previous);
+    }
+    return insert(std::move(n), deps);
+}
+
+int apply_graph_t::add_constant_fill(dtype_t dtype, uint64_t value_bits, uint64_t nelem,
+                                     mem_t out, std::vector<int> const& deps)
+{
+    node_t n;
+    n.kind = kind_t::constant;
+    n.dtype = dtype;
+    n.bits0 = value_bits;
+    n.n0 = nelem;
+    n.mems = {out};
+    return insert(std::move(n), deps);
+}
+
+int apply_graph_t::add_lowertri_fill(dtype_t dtype, uint64_t lower_bits, uint64_t upper_bits,
+                                     uint64_t nrow, uint64_t ncol, int64_t start, mem_t out,
+                                     std::vector<int> const& deps)
+{
+    node_t n;
+    n.kind = kind_t::lowertri;
+    n.dtype = dtype;
+    n.bits0 = lower_bits;
+    n.bits1 = upper_bits;
+    n.n0 = nrow;
+    n.n1 = ncol;
+    n.start = start;
+    n.mems = {out};
+    return insert(std::move(n), deps);
+}
+
+int apply_graph_t::add_copy(mem_t dst, mem_t src, std::vector<int> const& deps)
+{
+    if (dst.size != src.size) {
+        throw km_error(km_status::invalid, "apply graph: copy between ranges of different size");
+    }
+    node_t n;
+    n.kind = kind_t::copy;
+    n.mems = {dst, src};
+    return insert(std::move(n), deps);
+}
+
+void apply_graph_t::add_memory_dependencies()
+{
+    if (finalized_) throw km_error(km_status::invalid, "apply graph: already finalized");
+    for (size_t v = 0; v != nodes_.size(); ++v) {
+        node_t& nv = nodes_[v];
+        for (size_t u = 0; u != v; ++u) {
+            node_t const& nu = nodes_[u];
+            bool dep = false;
+            // v reads or rewrites what u wrote; v overwrites what u read
+            for (mem_t const& m : nv.mems) dep = dep || overlaps(nu.mems[0], m);
+            for (size_t k = 1; k < nu.mems.size(); ++k) dep = dep || overlaps(nv.mems[0], nu.mems[k]);
+            if (dep) nv.deps.push_back(int(u));
+        }
+        std::sort(nv.deps.begin(), nv.deps.end());
+        nv.deps.erase(std::unique(nv.deps.begin(), nv.deps.end()), nv.deps.end());
+    }
+}
+
+void apply_graph_t::finalize(int n_streams)
+{
+    if (finalized_) throw km_error(km_status::invalid, "apply graph: already finalized");
+    if (n_streams < 1 || n_streams > 16) {
+        throw km_error(km_status::invalid, "apply graph: between 1 and 16 streams");
+    }
+    int const n = int(nodes_.size());
+    if (km_) {
+        for (node_t const& nd : nodes_) {
+            if (nd.kind != kind_t::einsummable) continue;
+            if (!km_->build(nd.e)) {
+                throw km_error(km_status::invalid, "apply graph: no kernel for an einsummable "
+                                                   "(build returned unsupported)");
+            }
+        }
+    }
+
+    // Placement, in launch order.  A node continues the stream of a dependency that is
+    // still the last node of its stream (the most recent such dependency): that needs no
+    // wait at all.  Otherwise it takes the stream whose last node is oldest, and independent
+    // branches spread over the pool.
+    std::vector<int> last(size_t(n_streams), -1);
+    std::vector<std::vector<int>> synced(size_t(n_streams), std::vector<int>(size_t(n_streams), -1));
+    order_.resize(size_t(n));
+    n_waits_ = 0;
+    for (int v = 0; v != n; ++v) {
+        node_t& nv = nodes_[v];
+        nv.position = v;
+        order_[size_t(v)] = v;
+        int best = -1;
+        for (int d : nv.deps) {
+            int s = nodes_[d].stream;
+            if (last[size_t(s)] == d && (best < 0 || d > last[size_t(best)])) best = s;
+        }
+        if (best < 0) {
+            best = 0;
+            for (int s = 1; s != n_streams; ++s) {
+                if (last[size_t(s)] < last[size_t(best)]) best = s;
+            }
+        }
+        nv.stream = best;
+        last[size_t(best)] = v;
+        // waits: a stream runs in order, so waiting for a node covers everything its stream
+        // launched before it
+        nv.waits.clear();
+        std::vector<int> deps = nv.deps;
+        std::sort(deps.begin(), deps.end(), [](int x, int y) { return x > y; });
+        for (int d : deps) {
+            int sd = nodes_[d].stream;
+            if (sd == best) continue;
+            if (synced[size_t(best)][size_t(sd)] >= d) continue;
+            synced[size_t(best)][size_t(sd)] = d;
+            nv.waits.push_back(d);
+            nodes_[d].record = true;
+            ++n_waits_;
+        }
+    }
+
+    if (km_) {
+        check(hipSetDevice(km_->device()), "hipSetDevice");
+        streams_.assign(size_t(n_streams), nullptr);  // slot 0 is the caller's stream
+        for (int s = 1; s != n_streams; ++s) {
+            check(hipStreamCreateWithFlags(&streams_[size_t(s)], hipStreamNonBlocking),
+                  "hipStreamCreateWithFlags");
+        }
+        event_of_.assign(size_t(n), -1);
+        for (int v = 0; v != n; ++v) {
+            if (!nodes_[v].record) continue;
+            hipEvent_t e;
+            check(hipEventCreateWithFlags(&e, hipEventDisableTiming), "hipEventCreateWithFlags");
+            event_of_[size_t(v)] = int(events_.size());
+            events_.push_back(e);
+        }
+        check(hipEventCreateWithFlags(&fork_, hipEventDisableTiming), "hipEventCreateWithFlags");
+        for (int s = 1; s != n_streams; ++s) {
+            hipEvent_t e;
+            check(hipEventCreateWithFlags(&e, hipEventDisableTiming), "hipEventCreateWithFlags");
+            joins_.push_back(e);
+        }
+    }
+    finalized_ = true;
+}
+
+void apply_graph_t::launch(node_t const& n, hipStream_t stream, char* arena) const
+{
+    void* const out = arena + n.mems[0].offset;
+    switch (n.kind) {
+        case kind_t::einsummable: {
+            plan_t const* p = km_->plan_of(n.e);
+            if (!p) throw km_error(km_status::not_built, "apply graph: einsummable not built");
+            void const* inns[8];
+            std::vector<void const*> many;
+            void const** ptrs = inns;
+            size_t const k = n.mems.size() - 1;
+            if (k > 8) {
+                many.resize(k);
+                ptrs = many.data();
+            }
+            for (size_t i = 0; i != k; ++i) ptrs[i] = arena + n.mems[i + 1].offset;
+            km_->run_plan(*p, stream, out, ptrs, int(k), nullptr, 0);
+            break;
+        }
+        case kind_t::touch:
+            (*km_)(n.touch, stream, out, arena + n.mems[1].offset);
+            break;
+        case kind_t::constant:
+            km_->constant_fill(n.dtype, n.bits0, n.n0, stream, out);
+            break;
+        case kind_t::lowertri:
+            km_->lowerTri_fill(n.dtype, n.bits0, n.bits1, n.n0, n.n1, n.start, stream, out);
+            break;
+        case kind_t::copy:
+            check(hipMemcpyAsync(out, arena + n.mems[1].offset, n.mems[0].size,
+                                 hipMemcpyDeviceToDevice, stream),
+                  "hipMemcpyAsync");
+            break;
+    }
+}
+
+void apply_graph_t::run(hipStream_t main, void* arena_) const
+{
+    if (!finalized_) throw km_error(km_status::not_built, "apply graph: run before finalize");
+    if (!km_) throw km_error(km_status::device, "apply graph: planned without a kernel manager");
+    char* const arena = static_cast<char*>(arena_);
+    size_t const ns = streams_.size();
+    auto stream_at = [&](int s) { return s == 0 ? main : streams_[size_t(s)]; };
+    if (ns > 1) {
+        check(hipEventRecord(fork_, main), "hipEventRecord");
+        for (size_t s = 1; s != ns; ++s) {
+            check(hipStreamWaitEvent(streams_[s], fork_, 0), "hipStreamWaitEvent");
+        }
+    }
+    for (int v : order_) {
+        node_t const&     n = nodes_[size_t(v)];
+        hipStream_t const st = stream_at(n.stream);
+        for (int d : n.waits) {
+            check(hipStreamWaitEvent(st, events_[size_t(event_of_[size_t(d)])], 0),
+                  "hipStreamWaitEvent");
+        }
+        launch(n, st, arena);
+        if (n.record) {
+            check(hipEventRecord(events_[size_t(event_of_[size_t(v)])], st), "hipEventRecord");
+        }
+    }
+    for (size_t s = 1; s != ns; ++s) {
+        check(hipEventRecord(joins_[s - 1], streams_[s]), "hipEventRecord");
+        check(hipStreamWaitEvent(main, joins_[s - 1], 0), "hipStreamWaitEvent");
+    }
+}
+
+}  // namespace es

@@ -1,0 +1,111 @@
+// The exec-node layer over the kernel manager: a dependency graph of apply (einsummable /
+// touch) and fill nodes addressed by offsets into one device arena, run on one GPU.
+//
+// It plays the part of the reference's GPU exec graph for these node kinds
+// (src/engine/exec_graph.h:17-80; gpu_einsummable_t, gpu_touch_t, gpu_constant_t,
+// gpu_lowerTri_t, gpu_copy_t in src/engine/gpu/exec_nodes.h and
+// src/engine/gpu/exec_graph.cc:258-404, 600-690).  The reference drives its graph from a host
+// event loop: every node takes a stream from a pool, launches, and reports back through
+// cudaStreamAddCallback, after which the loop releases the node's dependents
+// (src/engine/exec_state.cc).  That is one host round trip per node.  Here the order is fixed
+// once, at finalize(): nodes are placed on a small pool of streams and every dependency that
+// crosses streams becomes an event wait on the device, so run() is a burst of launches with
+// no host synchronisation at all.  (A single-stream placement can also be captured into a
+// HIP graph; capturing the fork / join of pool streams crashed the ROCm 7.2 runtime and is
+// not supported.)
+//
+// Touch groups keep the reference's meaning (src/engine/managers.cc:3-21,
+// gpu/exec_graph.cc:354-378): touches of one group are serialised, and the first of a group
+// to run has its castable cleared (it initialises the output).  With a fixed order "first to
+// run" is the first one inserted.  A touch without a group is a plain copy
+// (gpu/exec_graph.cc:176-181).
+#pragma once
+#include "kernel_manager.h"
+
+#include <cstdint>
+#include <string>
+#include <vector>
+
+namespace es
+{
+
+struct mem_t {
+    uint64_t offset;
+    uint64_t size;
+};
+
+class apply_graph_t
+{
+public:
+    // `km` may be null: the graph can then be planned and inspected but not run
+    explicit apply_graph_t(kernel_manager_t* km);
+    ~apply_graph_t();
+    apply_graph_t(apply_graph_t const&) = delete;
+    apply_graph_t& operator=(apply_graph_t const&) = delete;
+
+    // mems[0] is the output, the rest are the inputs in order (memgraph.h:252-263).
+    // `deps` are ids of nodes that must complete first.  Each returns the new node's id.
+    int add_einsummable(einsummable_t const& e, std::vector<mem_t> const& mems,
+                        std::vector<int> const& deps);
+    int add_touch(touch_t const& t, int group, std::vector<mem_t> const& mems,
+                  std::vector<int> const& deps);
+    int add_constant_fill(dtype_t dtype, uint64_t value_bits, uint64_t nelem, mem_t out,
+                          std::vector<int> const& deps);
+    int add_lowertri_fill(dtype_t dtype, uint64_t lower_bits, uint64_t upper_bits, uint64_t nrow,
+                          uint64_t ncol, int64_t start, mem_t out, std::vector<int> const& deps);
+    int add_copy(mem_t dst, mem_t src, std::vector<int> const& deps);
+
+    // Adds, between every pair of nodes in insertion order, the dependency their memory
+    // ranges imply (read after write, write after write, write after read).
+    void add_memory_dependencies();
+
+    // Builds every einsummable on the kernel manager (throws km_error when one has no
+    // kernel), fixes the launch order and places the nodes on `n_streams` streams.
+    void finalize(int n_streams);
+
+    // Enqueues the whole graph.  Work is ordered after what `main` holds at the call and
+    // `main` is ordered after all of it on return; nothing synchronises with the host.
+    void run(hipStream_t main, void* arena) const;
+
+    int n_nodes() const { return int(nodes_.size()); }
+    // after finalize: launch position, stream and dependencies (own + implied) of a node
+    int                     position_of(int id) const { return nodes_[id].position; }
+    int                     stream_of(int id) const { return nodes_[id].stream; }
+    std::vector<int> const& deps_of(int id) const { return nodes_[id].deps; }
+    // number of event waits run() enqueues (dependencies that cross streams)
+    int n_cross_stream_waits() const { return n_waits_; }
+
+private:
+    enum class kind_t { einsummable, touch, constant, lowertri, copy };
+    struct node_t {
+        kind_t             kind;
+        einsummable_t      e;
+        touch_t            touch;
+        int                group = -1;
+        dtype_t            dtype = dtype_t::f32;
+        uint64_t           bits0 = 0, bits1 = 0, n0 = 0, n1 = 0;
+        int64_t            start = 0;
+        std::vector<mem_t> mems;
+        std::vector<int>   deps;
+        std::vector<int>   waits;  // dependencies on other streams, reduced
+        int                position = -1;
+        int                stream = -1;
+        bool               record = false;  // some dependent waits for this node's event
+    };
+
+    int  insert(node_t&& n, std::vector<int> const& deps);
+    void launch(node_t const& n, hipStream_t stream, char* arena) const;
+
+    kernel_manager_t*        km_;
+    std::vector<node_t>      nodes_;
+    std::vector<int>         order_;
+    std::vector<hipStream_t> streams_;
+    std::vector<hipEvent_t>  events_;  // one per node that records
+    std::vector<int>         event_of_;
+    hipEvent_t               fork_ = nullptr;
+    std::vector<hipEvent_t>  joins_;
+    int                      n_waits_ = 0;
+    bool                     finalized_ = false;
+};
+
+}  // namespace es

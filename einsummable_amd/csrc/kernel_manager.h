@@ -76,6 +76,10 @@ public:
                            void const* const* inns, int n_inns, void* workspace,
                            uint64_t workspace_bytes) const;
 
+    // the plan build() made for this einsummable, or null (for callers that launch the
+    // same node many times and do not want the lookup on their hot path)
+    plan_t const* plan_of(einsummable_t const& e) const { return find(e.merge_adjacent_dims()); }
+
     int device() const { return device_; }
 
 private:

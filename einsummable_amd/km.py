@@ -25,6 +25,18 @@ EXPORTS = [
     "es_km_scalarop_roundtrip",
     "es_km_merge_adjacent_dims",
     "es_km_probe_mfma_f16",
+    "es_km_graph_create",
+    "es_km_graph_destroy",
+    "es_km_graph_add_einsummable",
+    "es_km_graph_add_touch",
+    "es_km_graph_add_fill_constant",
+    "es_km_graph_add_fill_lowertri",
+    "es_km_graph_add_copy",
+    "es_km_graph_add_memory_dependencies",
+    "es_km_graph_finalize",
+    "es_km_graph_run",
+    "es_km_graph_node_info",
+    "es_km_graph_cross_stream_waits",
 ]
 
 
@@ -127,6 +139,21 @@ def load_library():
     lib.es_km_merge_adjacent_dims.argtypes = desc + [ctypes.c_void_p, ctypes.c_void_p,
                                                      ctypes.c_void_p, ctypes.c_void_p,
                                                      ctypes.c_void_p, ctypes.c_size_t]
+    V, I, U64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_uint64
+    lib.es_km_graph_create.restype = V
+    lib.es_km_graph_create.argtypes = [V]
+    lib.es_km_graph_destroy.argtypes = [V]
+    lib.es_km_graph_add_einsummable.argtypes = [V] + desc + [V, V, I, V, I]
+    lib.es_km_graph_add_touch.argtypes = [V, V, I, ctypes.c_char, I, I, V, V, V, I]
+    lib.es_km_graph_add_fill_constant.argtypes = [V, I, U64, U64, U64, U64, V, I]
+    lib.es_km_graph_add_fill_lowertri.argtypes = [V, I, U64, U64, U64, U64, ctypes.c_int64, U64,
+                                                  U64, V, I]
+    lib.es_km_graph_add_copy.argtypes = [V, U64, U64, U64, V, I]
+    lib.es_km_graph_add_memory_dependencies.argtypes = [V]
+    lib.es_km_graph_finalize.argtypes = [V, I]
+    lib.es_km_graph_run.argtypes = [V, V, V]
+    lib.es_km_graph_node_info.argtypes = [V, I, V, V, V, I, V]
+    lib.es_km_graph_cross_stream_waits.argtypes = [V]
     _lib = lib
     return lib
 
@@ -343,3 +370,95 @@ class KernelManager:
                                            start, stream, out)
         if rc != OK:
             self._fail(rc)
+
+
+class ApplyGraph:
+    """The exec-node layer (include/es_km.h, es_km_graph_*): apply / fill / copy nodes over
+    one device arena with dependencies, placed on a pool of streams at finalize() and
+    enqueued by run() without any host synchronisation.  `km=None` gives a graph that can be
+    planned and inspected without a device."""
+
+    def __init__(self, km=None):
+        self._lib = load_library()
+        self._km = km
+        self._g = self._lib.es_km_graph_create(km._h if km is not None else None)
+        if not self._g:
+            raise KmError(ERR_DEVICE, "es_km_graph_create failed")
+
+    def close(self):
+        if self._g:
+            self._lib.es_km_graph_destroy(self._g)
+            self._g = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def _check(self, rc):
+        if rc < 0:
+            h = self._km._h if self._km is not None else None
+            raise KmError(rc, self._lib.es_km_last_error(h).decode())
+        return rc
+
+    @staticmethod
+    def _mems(mems):
+        offs = (ctypes.c_uint64 * len(mems))(*[int(m[0]) for m in mems])
+        sizes = (ctypes.c_uint64 * len(mems))(*[int(m[1]) for m in mems])
+        return offs, sizes
+
+    @staticmethod
+    def _deps(deps):
+        deps = list(deps or [])
+        return (ctypes.c_int * max(len(deps), 1))(*deps), len(deps)
+
+    def add_einsummable(self, e, mems, deps=None):
+        """mems: [(offset, size)] with the output first, then the inputs."""
+        offs, sizes = self._mems(mems)
+        d, nd = self._deps(deps)
+        return self._check(self._lib.es_km_graph_add_einsummable(
+            self._g, *e._args, offs, sizes, len(mems), d, nd))
+
+    def add_touch(self, t, group, mems, deps=None):
+        offs, sizes = self._mems(mems)
+        d, nd = self._deps(deps)
+        return self._check(self._lib.es_km_graph_add_touch(
+            self._g, ctypes.cast(t._dims, ctypes.c_void_p), len(t.selection),
+            _castable_char(t.castable), t.dtype, int(group), offs, sizes, d, nd))
+
+    def add_constant_fill(self, dtype, value_bits, nelem, mem, deps=None):
+        d, nd = self._deps(deps)
+        return self._check(self._lib.es_km_graph_add_fill_constant(
+            self._g, dtype, value_bits, nelem, int(mem[0]), int(mem[1]), d, nd))
+
+    def add_lowertri_fill(self, dtype, lower_bits, upper_bits, nrow, ncol, start, mem, deps=None):
+        d, nd = self._deps(deps)
+        return self._check(self._lib.es_km_graph_add_fill_lowertri(
+            self._g, dtype, lower_bits, upper_bits, nrow, ncol, start, int(mem[0]), int(mem[1]),
+            d, nd))
+
+    def add_copy(self, dst_offset, src_offset, size, deps=None):
+        d, nd = self._deps(deps)
+        return self._check(self._lib.es_km_graph_add_copy(self._g, dst_offset, src_offset, size,
+                                                          d, nd))
+
+    def add_memory_dependencies(self):
+        self._check(self._lib.es_km_graph_add_memory_dependencies(self._g))
+
+    def finalize(self, n_streams=1):
+        self._check(self._lib.es_km_graph_finalize(self._g, int(n_streams)))
+
+    def run(self, stream, arena):
+        self._check(self._lib.es_km_graph_run(self._g, stream, arena))
+
+    def node_info(self, node):
+        """(launch position, stream index, [dependencies]) after finalize."""
+        pos, st, n = ctypes.c_int(-1), ctypes.c_int(-1), ctypes.c_int(0)
+        deps = (ctypes.c_int * 4096)()
+        self._check(self._lib.es_km_graph_node_info(self._g, node, ctypes.byref(pos),
+                                                    ctypes.byref(st), deps, 4096, ctypes.byref(n)))
+        return pos.value, st.value, list(deps[:min(n.value, 4096)])
+
+    def cross_stream_waits(self):
+        return self._check(self._lib.es_km_graph_cross_stream_waits(self._g))

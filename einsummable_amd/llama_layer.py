@@ -258,3 +258,83 @@ class DeviceRunner:
         with torch.cuda.graph(graph):
             self.run(stream=torch.cuda.current_stream().cuda_stream)
         return graph
+
+
+class ArenaRunner:
+    """The same node list through the exec-node layer: every buffer is a range of ONE device
+    arena (as in the engine: `arena + mems[i].offset`, src/engine/gpu/exec_graph.cc:295-301),
+    the dependencies follow from the ranges, the nodes are placed on `n_streams` streams at
+    construction and run() enqueues the whole layer with no host synchronisation."""
+
+    ALIGN = 256
+
+    def __init__(self, km, graph, n_streams=4):
+        import struct
+
+        import torch
+
+        from .km import ApplyGraph
+
+        self.km, self.g, self.torch = km, graph, torch
+        self.ranges, off = {}, 0
+        for name, nbytes in graph.buffers.items():
+            self.ranges[name] = (off, nbytes)
+            off += (nbytes + self.ALIGN - 1) // self.ALIGN * self.ALIGN
+        self.arena = torch.empty(max(off, 1), dtype=torch.uint8, device="cuda")
+        ag = ApplyGraph(km)
+        self.ids = []
+        for n in graph.nodes:
+            if n["kind"] == "einsummable":
+                i = ag.add_einsummable(n["e"], [self.ranges[n["out"]]] +
+                                       [self.ranges[b] for b in n["inns"]])
+            elif n["kind"] == "touch":
+                i = ag.add_touch(n["t"], -1, [self.ranges[n["out"]], self.ranges[n["inn"]]])
+            else:
+                assert n["dtype"] == F16
+                lo = struct.unpack("<H", struct.pack("<e", n["lower"]))[0]
+                up = struct.unpack("<H", struct.pack("<e", n["upper"]))[0]
+                i = ag.add_lowertri_fill(n["dtype"], lo, up, n["nrow"], n["ncol"], n["start"],
+                                         self.ranges[n["out"]])
+            self.ids.append(i)
+        ag.add_memory_dependencies()
+        ag.finalize(n_streams)
+        self.graph = ag
+        self.n_streams = n_streams
+
+    def view(self, name):
+        off, nbytes = self.ranges[name]
+        return self.arena[off:off + nbytes]
+
+    def set_input(self, name, array):
+        import numpy as np
+
+        t = self.torch.from_numpy(np.ascontiguousarray(array).view(np.uint8).reshape(-1))
+        assert t.numel() == self.view(name).numel(), name
+        self.view(name).copy_(t)
+
+    def get(self, name, np_dtype):
+        return self.view(name).cpu().numpy().view(np_dtype)
+
+    def run(self, stream=None):
+        stream = stream if stream is not None else self.torch.cuda.current_stream().cuda_stream
+        self.graph.run(stream, self.arena.data_ptr())
+
+    def capture(self):
+        """The burst captured into one HIP graph.  Only for a single-stream placement:
+        capturing a run whose pool streams fork from and join the capturing stream crashed
+        inside the HIP runtime on ROCm 7.2 (host-side segmentation fault during capture),
+        so that combination is refused here."""
+        if self.n_streams != 1:
+            raise NotImplementedError("HIP graph capture of a multi-stream exec graph is "
+                                      "switched off (the runtime crashed during capture)")
+        torch = self.torch
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            self.run(stream=side.cuda_stream)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            self.run(stream=torch.cuda.current_stream().cuda_stream)
+        return graph

@@ -150,6 +150,68 @@ int es_km_merge_adjacent_dims(const uint64_t* join_shape, int join_rank, const i
 double es_km_probe_mfma_f16(es_km_t* km, const void* operands, void* scratch, int blocks, int iters,
                             void* stream);
 
+/* ---------------------------------------------------------------------------------------
+ * Exec-node layer: a dependency graph of apply / fill / copy nodes over ONE device arena.
+ *
+ * Replaces, for one GPU, the reference's GPU exec graph and its node types
+ *   exec_graph_t::insert / node_t                   src/engine/exec_graph.h:53-80
+ *   gpu_einsummable_t::launch                       src/engine/gpu/exec_graph.cc:276-332
+ *   gpu_touch_t::launch (group semantics)           src/engine/gpu/exec_graph.cc:354-404
+ *   gpu_constant_t / gpu_lowerTri_t / gpu_copy_t    src/engine/gpu/exec_nodes.h:112-160
+ *   streampool_manager_t, group_manager_t           src/engine/gpu/stream_pool.cc,
+ *                                                   src/engine/managers.cc:3-21
+ * Memory ranges are (offset, size) into the arena passed to run (mem_t, memgraph.h:44-60;
+ * mems[0] is the output, memgraph.h:252-263).  A node may only depend on nodes added before
+ * it: insertion order is the launch order.  Where the reference reports every node's
+ * completion to a host event loop through a stream callback, finalize fixes the order and
+ * the stream of every node once and run enqueues everything, cross-stream dependencies as
+ * event waits on the device; nothing synchronises with the host.  A graph finalized on one
+ * stream may be captured into a HIP graph; do not capture a multi-stream run (the fork /
+ * join of pool streams inside a capture crashed the HIP runtime of ROCm 7.2).
+ * `add_*` return the node id (>= 0) or a negative error code.
+ * Touches: group < 0 makes the touch a copy (exec_graph.cc:176-181); touches of one group
+ * run in insertion order and the first has its castable cleared (exec_graph.cc:368-378).
+ * es_km_graph_create(NULL) gives a graph that can be planned and inspected but not run. */
+typedef struct es_km_graph es_km_graph_t;
+
+es_km_graph_t* es_km_graph_create(es_km_t* km);
+void           es_km_graph_destroy(es_km_graph_t* g);
+
+int es_km_graph_add_einsummable(es_km_graph_t* g, const uint64_t* join_shape, int join_rank,
+                                const int* inns_flat, const int* inns_offsets, int n_inns,
+                                int out_rank, const char* join_text, char castable,
+                                const uint64_t* mem_offsets, const uint64_t* mem_sizes, int n_mems,
+                                const int* deps, int n_deps);
+int es_km_graph_add_touch(es_km_graph_t* g, const uint64_t* touchdims, int rank, char castable,
+                          int dtype, int group, const uint64_t* mem_offsets,
+                          const uint64_t* mem_sizes, const int* deps, int n_deps);
+int es_km_graph_add_fill_constant(es_km_graph_t* g, int dtype, uint64_t value_bits,
+                                  uint64_t nelem, uint64_t offset, uint64_t size, const int* deps,
+                                  int n_deps);
+int es_km_graph_add_fill_lowertri(es_km_graph_t* g, int dtype, uint64_t lower_bits,
+                                  uint64_t upper_bits, uint64_t nrow, uint64_t ncol, int64_t start,
+                                  uint64_t offset, uint64_t size, const int* deps, int n_deps);
+int es_km_graph_add_copy(es_km_graph_t* g, uint64_t dst_offset, uint64_t src_offset, uint64_t size,
+                         const int* deps, int n_deps);
+
+/* Adds the dependencies the nodes' memory ranges imply (read after write, write after
+ * write, write after read), for callers that hold no explicit edge list. */
+int es_km_graph_add_memory_dependencies(es_km_graph_t* g);
+
+/* Builds every einsummable (an unsupported one is an error here), places the nodes on
+ * n_streams (1..16) streams.  The graph is immutable afterwards. */
+int es_km_graph_finalize(es_km_graph_t* g, int n_streams);
+
+/* Enqueues the whole graph: ordered after what `stream` holds at the call, and `stream` is
+ * ordered after all of it on return.  Calls on one graph must not overlap in time. */
+int es_km_graph_run(es_km_graph_t* g, void* stream, void* arena);
+
+/* After finalize: launch position, stream index and dependencies of a node (deps receives
+ * at most cap ids, *n_deps the full count); number of event waits one run enqueues. */
+int es_km_graph_node_info(es_km_graph_t* g, int id, int* position, int* stream, int* deps, int cap,
+                          int* n_deps);
+int es_km_graph_cross_stream_waits(es_km_graph_t* g);
+
 #ifdef __cplusplus
 }
 #endif

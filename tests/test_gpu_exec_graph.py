@@ -1,0 +1,179 @@
+"""The exec-node layer (es_km_graph_*): dependency graphs of apply / fill / copy nodes over
+one arena, placed on several streams.  Kernels are deterministic, so whatever the placement
+the arena must end up with exactly the bytes of the same nodes run one after the other."""
+import numpy as np
+import pytest
+
+import einsummable_amd as ea
+from einsummable_amd.llama_layer import ArenaRunner, DeviceRunner, LayerGraph
+from helpers import NP, normal, rng, stream_handle
+from test_gpu_llama_layer import make_inputs
+
+pytestmark = pytest.mark.gpu
+
+E = ea.Einsummable
+SLOT = 64 * 1024          # bytes per arena slot in the random graphs
+N = SLOT // 4             # f32 elements per slot
+
+
+def random_graph(r, n_nodes, n_slots):
+    """Node descriptions over arena slots: unary / binary elementwise, row reductions into
+    the head of a slot, copies, touches (grouped accumulations included) and fills."""
+    nodes = []
+    group_of_slot = {}
+    for _ in range(n_nodes):
+        kind = r.choice(["unary", "binary", "reduce", "copy", "touch", "group", "fill"],
+                        p=[0.3, 0.25, 0.1, 0.1, 0.1, 0.1, 0.05])
+        out = int(r.randint(1, n_slots))
+        a, b = int(r.randint(0, n_slots)), int(r.randint(0, n_slots))
+        if kind in ("unary", "copy", "touch", "group", "reduce") and a == out:
+            a = (a + 1) % n_slots
+        if kind == "binary" and (a == out or b == out):
+            kind = "fill"
+        nodes.append((kind, out, a, b))
+    return nodes
+
+
+def add_nodes(g, nodes):
+    ids = []
+    groups = {}
+    for kind, out, a, b in nodes:
+        mo, ma, mb = (out * SLOT, SLOT), (a * SLOT, SLOT), (b * SLOT, SLOT)
+        if kind == "unary":
+            i = g.add_einsummable(E([N], [[0]], 1, "*[constant{f32|0.5},hole|f32@0]"), [mo, ma])
+        elif kind == "binary":
+            i = g.add_einsummable(E([N], [[0], [0]], 1, "+[hole|f32@0,hole|f32@1]"), [mo, ma, mb])
+        elif kind == "reduce":
+            i = g.add_einsummable(E([64, N // 64], [[0, 1]], 1, "hole|f32@0", "^"),
+                                  [(out * SLOT, 64 * 4), ma])
+        elif kind == "copy":
+            i = g.add_copy(out * SLOT, a * SLOT, SLOT)
+        elif kind == "touch":
+            t = ea.Touch([(128, 128, 0, 0, 128), (N // 128, N // 128, 3, 5, 40)], "+", ea.F32)
+            i = g.add_touch(t, -1, [mo, ma])       # no group: runs as a copy
+        elif kind == "group":
+            t = ea.Touch([(N, N, 0, 0, N)], "+", ea.F32)
+            i = g.add_touch(t, groups.setdefault(out, len(groups)), [mo, ma])
+        else:
+            i = g.add_constant_fill(ea.F32, int(np.float32(1.25).view(np.uint32)), N, mo)
+        ids.append(i)
+    return ids
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_graphs_give_the_sequential_bytes_on_any_number_of_streams(km, seed):
+    import torch
+
+    r = rng(100 + seed)
+    n_slots = 12
+    nodes = random_graph(r, 60, n_slots)
+    init = normal(r, n_slots * N, np.float32)
+    results = []
+    for n_streams in (1, 2, 5):
+        g = ea.ApplyGraph(km)
+        ids = add_nodes(g, nodes)
+        g.add_memory_dependencies()
+        g.finalize(n_streams)
+        arena = torch.from_numpy(init.copy()).cuda()
+        g.run(stream_handle(), arena.data_ptr())
+        torch.cuda.synchronize()
+        results.append(arena.cpu().numpy())
+        streams = {g.node_info(i)[1] for i in ids}
+        assert max(streams) < n_streams
+        if n_streams == 1:
+            assert g.cross_stream_waits() == 0
+    assert np.array_equal(results[0].view(np.uint32), results[1].view(np.uint32))
+    assert np.array_equal(results[0].view(np.uint32), results[2].view(np.uint32))
+    assert not np.array_equal(results[0], init)
+
+
+def test_touch_groups_first_member_initialises_then_members_accumulate_in_order(km):
+    import torch
+
+    r = rng(120)
+    n = 4096
+    parts = [normal(r, n, np.float16) for _ in range(5)]
+    arena = torch.zeros(6 * n, dtype=torch.float16, device="cuda")
+    arena[:n] = 777.0                                   # stale bytes the first touch must replace
+    for k, p in enumerate(parts):
+        arena[(k + 1) * n:(k + 2) * n] = torch.from_numpy(p).cuda()
+    g = ea.ApplyGraph(km)
+    t = ea.Touch([(n, n, 0, 0, n)], "+", ea.F16)
+    for k in range(5):
+        g.add_touch(t, 7, [(0, 2 * n), ((k + 1) * 2 * n, 2 * n)])
+    g.finalize(3)
+    g.run(stream_handle(), arena.data_ptr())
+    torch.cuda.synchronize()
+    want = parts[0].copy()
+    for p in parts[1:]:
+        want = (want + p).astype(np.float16)            # fp16 rounding after every touch
+    assert np.array_equal(arena[:n].cpu().numpy().view(np.uint16), want.view(np.uint16))
+
+
+@pytest.mark.parametrize("n_streams", [1, 2, 4])
+def test_llama_layer_through_the_exec_graph_equals_node_by_node_launches(km, n_streams):
+    import torch
+
+    g = LayerGraph(dim=256, n_heads=4, ffn=688, seq=128)
+    vals = make_inputs(g, 3)
+    seq = DeviceRunner(km, g)
+    par = ArenaRunner(km, g, n_streams)
+    for k, v in vals.items():
+        seq.set_input(k, v)
+        par.set_input(k, v)
+    seq.run()
+    par.run()
+    torch.cuda.synchronize()
+    for name in g.buffers:
+        assert np.array_equal(seq.get(name, np.uint8), par.get(name, np.uint8)), name
+    if n_streams > 1:
+        assert par.graph.cross_stream_waits() > 0
+        assert len({par.graph.node_info(i)[1] for i in par.ids}) > 1
+
+
+@pytest.mark.parametrize("n_streams", [
+    1,
+    pytest.param(4, marks=pytest.mark.skip(
+        reason="capturing a run that forks to and joins from pool streams ended in a "
+               "host-side segmentation fault inside the HIP runtime (ROCm 7.2); no cause "
+               "found in this code, so the combination is refused by ArenaRunner.capture")),
+])
+def test_exec_graph_captured_into_a_hip_graph_replays_the_eager_bytes(km, n_streams):
+    import torch
+
+    g = LayerGraph(dim=256, n_heads=4, ffn=688, seq=128)
+    par = ArenaRunner(km, g, n_streams)
+    for k, v in make_inputs(g, 5).items():
+        par.set_input(k, v)
+    hip_graph = par.capture()
+    for seed in (6, 7, 8):
+        for k, v in make_inputs(g, seed).items():
+            par.set_input(k, v)
+        par.run()
+        torch.cuda.synchronize()
+        eager = {n: par.get(n, np.uint8).copy() for n in ("residual2", "sm.div", "mask")}
+        for n in eager:
+            par.view(n).zero_()
+        torch.cuda.synchronize()
+        hip_graph.replay()
+        torch.cuda.synchronize()
+        for n, want in eager.items():
+            assert np.array_equal(par.get(n, np.uint8), want), (seed, n)
+
+
+def test_exec_graph_errors(km):
+    g = ea.ApplyGraph(km)
+    e = E([16], [[0]], 1, "hole|f32@0")
+    with pytest.raises(ea.KmError) as ei:
+        g.add_einsummable(e, [(0, 64), (64, 64)], deps=[0])      # depends on itself / later
+    assert ei.value.code == -1
+    with pytest.raises(ea.KmError) as ei:
+        g.add_einsummable(e, [(0, 64)])                           # an input range is missing
+    assert ei.value.code == -4
+    a = g.add_einsummable(e, [(0, 64), (64, 64)])
+    with pytest.raises(ea.KmError) as ei:
+        g.run(0, 1)                                               # run before finalize
+    assert ei.value.code == -2
+    g.finalize(2)
+    with pytest.raises(ea.KmError):
+        g.add_einsummable(e, [(0, 64), (64, 64)], deps=[a])      # immutable after finalize

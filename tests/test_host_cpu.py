@@ -131,3 +131,63 @@ def test_descriptor_errors_map_to_codes():
         with pytest.raises(ea.KmError) as ei:
             ea.codegen_source(e)
         assert ei.value.code == -1, e.join
+
+
+# ---- exec-node layer: planning needs no device
+
+def _plan_only_graph():
+    import einsummable_amd as ea
+
+    g = ea.ApplyGraph(None)
+    E = ea.Einsummable
+    unary = E([1024], [[0]], 1, "hole|f32@0")
+    add = E([1024], [[0], [0]], 1, "+[hole|f32@0,hole|f32@1]")
+    m = lambda slot: (slot * 4096, 4096)
+    return g, unary, add, m
+
+
+def test_exec_graph_memory_dependencies_and_stream_placement():
+    g, unary, add, m = _plan_only_graph()
+    a = g.add_einsummable(unary, [m(1), m(0)])
+    b = g.add_einsummable(unary, [m(2), m(1)])            # reads a's output
+    c = g.add_einsummable(unary, [m(3), m(1)])            # reads a's output
+    d = g.add_einsummable(add, [m(4), m(2), m(3)])        # joins b and c
+    e = g.add_einsummable(unary, [m(6), m(5)])            # independent
+    f = g.add_einsummable(unary, [m(1), m(5)])            # overwrites what b and c read
+    g.add_memory_dependencies()
+    g.finalize(3)
+    info = {k: g.node_info(k) for k in (a, b, c, d, e, f)}
+    assert [info[k][0] for k in (a, b, c, d, e, f)] == [0, 1, 2, 3, 4, 5]   # launch order
+    assert info[b][2] == [a] and info[c][2] == [a] and info[d][2] == [b, c]
+    assert info[e][2] == []
+    assert set(info[f][2]) == {a, b, c}                   # write after write / after read
+    # a chain stays on its stream, a fork takes another one, an independent node a third
+    assert info[b][1] == info[a][1]
+    assert info[c][1] != info[b][1]
+    assert info[d][1] in (info[b][1], info[c][1])
+    assert info[e][1] not in (info[b][1], info[c][1])
+    assert g.cross_stream_waits() >= 2
+
+
+def test_exec_graph_single_stream_needs_no_events_and_groups_chain():
+    import einsummable_amd as ea
+
+    g, unary, add, m = _plan_only_graph()
+    t = ea.Touch([(1024, 1024, 0, 0, 1024)], "+", ea.F32)
+    x = g.add_touch(t, 3, [m(0), m(1)])
+    y = g.add_touch(t, 3, [m(0), m(2)])
+    z = g.add_touch(t, 4, [m(5), m(2)])
+    g.finalize(1)
+    assert g.cross_stream_waits() == 0
+    assert g.node_info(y)[2] == [x]                       # same group: serialised
+    assert g.node_info(z)[2] == []
+
+
+def test_exec_graph_rejects_forward_dependencies():
+    import pytest as _pytest
+
+    import einsummable_amd as ea
+
+    g, unary, add, m = _plan_only_graph()
+    with _pytest.raises(ea.KmError):
+        g.add_einsummable(unary, [m(1), m(0)], deps=[3])
