@@ -208,6 +208,104 @@ private:
     }
 
     es_km_t* h_;
+    friend class exec_graph_t;
+};
+
+// mem_t of the memgraph (src/einsummable/memgraph.h:44-60): a byte range of the arena
+struct mem_t {
+    uint64_t offset, size;
+};
+
+// The exec-node layer: what exec_graph_t::make_gpu_exec_graph builds out of a memgraph's
+// apply / constant / copy nodes (src/engine/gpu/exec_graph.cc:60-256) and what
+// exec_state_t::event_loop then drives (src/engine/exec_state.cc).  insert_* mirror the op
+// types of src/engine/gpu/exec_nodes.h; `inns` are the ids of the nodes to wait for, as in
+// exec_graph_t::insert (src/engine/exec_graph.h:53).
+class exec_graph_t
+{
+public:
+    explicit exec_graph_t(kernel_manager_t& km) : km_(km), g_(es_km_graph_create(km.h_))
+    {
+        if (!g_) throw std::runtime_error("exec_graph_t: could not create the graph");
+    }
+    ~exec_graph_t() { es_km_graph_destroy(g_); }
+    exec_graph_t(exec_graph_t const&) = delete;
+    exec_graph_t& operator=(exec_graph_t const&) = delete;
+
+    // gpu_einsummable_t: mems[0] is the output
+    int insert_einsummable(einsummable_t const& e, std::vector<mem_t> const& mems,
+                           std::vector<int> const& inns = {})
+    {
+        std::vector<int> flat, offs{0};
+        for (auto const& inn : e.inns) {
+            flat.insert(flat.end(), inn.begin(), inn.end());
+            offs.push_back(int(flat.size()));
+        }
+        std::vector<uint64_t> mo, ms;
+        split(mems, mo, ms);
+        return id(es_km_graph_add_einsummable(
+            g_, e.join_shape.data(), int(e.join_shape.size()), flat.data(), offs.data(),
+            int(e.inns.size()), e.out_rank, e.join.c_str(), castable_char(e.castable), mo.data(),
+            ms.data(), int(mems.size()), inns.data(), int(inns.size())));
+    }
+    // gpu_touch_t: group < 0 makes it a copy, the first touch of a group initialises
+    int insert_touch(touch_t const& t, int group, mem_t out, mem_t inn,
+                     std::vector<int> const& inns = {})
+    {
+        uint64_t mo[2] = {out.offset, inn.offset}, ms[2] = {out.size, inn.size};
+        return id(es_km_graph_add_touch(
+            g_, reinterpret_cast<uint64_t const*>(t.selection.data()), int(t.selection.size()),
+            castable_char(t.castable), int(t.dtype), group, mo, ms, inns.data(), int(inns.size())));
+    }
+    // gpu_constant_t / gpu_lowerTri_t
+    int insert_constant(fill_t::constant_t const& c, mem_t out, std::vector<int> const& inns = {})
+    {
+        uint64_t n = 1;
+        for (uint64_t d : c.shape) n *= d;
+        return id(es_km_graph_add_fill_constant(g_, int(c.value.dtype), c.value.bits(), n,
+                                                out.offset, out.size, inns.data(),
+                                                int(inns.size())));
+    }
+    int insert_lowertri(fill_t::lowertri_t const& l, mem_t out, std::vector<int> const& inns = {})
+    {
+        return id(es_km_graph_add_fill_lowertri(g_, int(l.lower.dtype), l.lower.bits(),
+                                                l.upper.bits(), l.nrow, l.ncol, l.start, out.offset,
+                                                out.size, inns.data(), int(inns.size())));
+    }
+    // gpu_copy_t within the device
+    int insert_copy(mem_t dst, mem_t src, std::vector<int> const& inns = {})
+    {
+        if (dst.size != src.size) throw std::runtime_error("exec_graph_t: copy sizes differ");
+        return id(es_km_graph_add_copy(g_, dst.offset, src.offset, dst.size, inns.data(),
+                                       int(inns.size())));
+    }
+    void add_memory_dependencies() { check(es_km_graph_add_memory_dependencies(g_)); }
+    void finalize(int n_streams) { check(es_km_graph_finalize(g_, n_streams)); }
+    // the whole graph, ordered after and before `stream`; no host synchronisation
+    void run(void* stream, void* arena) const { check(es_km_graph_run(g_, stream, arena)); }
+
+private:
+    static void split(std::vector<mem_t> const& m, std::vector<uint64_t>& o,
+                      std::vector<uint64_t>& s)
+    {
+        for (auto const& x : m) {
+            o.push_back(x.offset);
+            s.push_back(x.size);
+        }
+    }
+    int id(int rc) const
+    {
+        if (rc < 0) check(rc);
+        return rc;
+    }
+    void check(int rc) const
+    {
+        if (rc < 0) {
+            throw std::runtime_error(std::string("exec_graph_t: ") + es_km_last_error(km_.h_));
+        }
+    }
+    kernel_manager_t& km_;
+    es_km_graph_t*    g_;
 };
 
 }  // namespace eskm

@@ -188,6 +188,37 @@ int main()
         expect(threw, "wrong input count throws");
     }
 
+    {  // exec-node layer: out = relu(x) + relu(y) as three dependent nodes over one arena,
+       // a grouped pair of touches, on two streams (src/engine/gpu/exec_graph.cc:258-404)
+        uint64_t const n = 4096, B = n * 4;
+        std::string const relu = "ite_>=[constant{f32|0},hole|f32@0,constant{f32|0},hole|f32@0]";
+        einsummable_t e_relu{{n}, {{0}}, 1, relu, std::nullopt};
+        einsummable_t e_add{{n}, {{0}, {0}}, 1, "+[hole|f32@0,hole|f32@1]", std::nullopt};
+        auto x = random_f32(gen, n, -1, 1), y = random_f32(gen, n, -1, 1);
+        device_buffer_t arena(6 * B);
+        std::vector<float> host(6 * n, 9.0f), got(6 * n);
+        std::copy(x.begin(), x.end(), host.begin());
+        std::copy(y.begin(), y.end(), host.begin() + n);
+        arena.upload(host.data());
+        exec_graph_t g(km);
+        int a = g.insert_einsummable(e_relu, {{2 * B, B}, {0, B}});
+        int b = g.insert_einsummable(e_relu, {{3 * B, B}, {B, B}});
+        int c = g.insert_einsummable(e_add, {{4 * B, B}, {2 * B, B}, {3 * B, B}}, {a, b});
+        touch_t t{{{n, n, 0, 0, n}}, castable_t::add, dtype_t::f32};
+        g.insert_touch(t, 0, {5 * B, B}, {0, B});          // first of its group: initialises
+        g.insert_touch(t, 0, {5 * B, B}, {4 * B, B}, {c});  // accumulates
+        g.finalize(2);
+        g.run(stream, arena.ptr);
+        HIP_OK(hipStreamSynchronize(stream));
+        arena.download(got.data());
+        bool ok = true;
+        for (uint64_t i = 0; i != n; ++i) {
+            float s = std::max(x[i], 0.0f) + std::max(y[i], 0.0f);
+            ok = ok && got[4 * n + i] == s && got[5 * n + i] == x[i] + s;
+        }
+        expect(ok, "exec graph: dependent nodes and a touch group on two streams");
+    }
+
     HIP_OK(hipStreamDestroy(stream));
     std::printf("PASS\n");
     return 0;
