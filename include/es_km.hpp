@@ -13,7 +13,8 @@
 // The descriptor structs carry the same fields as the reference's einsummable_t
 // (src/einsummable/einsummable.h:8-20), touch_t (touch.h:8-29) and fill_t (fill.h:11-30); the
 // join travels as the text `operator<<(ostream&, scalarop_t)` writes.  Inside the reference
-// tree the adapter is three lines per call: see INTEGRATION.md.
+// tree the adapter is three lines per call: flatten `inns`, print `join` and the castable
+// with write_with_ss, forward to the C entry point.
 #pragma once
 #include "es_km.h"
 
