@@ -518,6 +518,43 @@ def run_read_ceiling(km, steps, warmup):
             "torch_amax_GBps": round(nbytes / lib.mean_ms() / 1e6, 1)}
 
 
+def run_col_reductions(km, steps, warmup):
+    """Reductions whose aggregated mode is not the innermost one (column sums and the like):
+    few outputs and a long aggregation run as two passes over a workspace."""
+    import torch
+
+    import einsummable_amd as ea
+
+    E = ea.Einsummable
+    cases = [
+        ("ab->b 8192x8192 f16 add", E([8192, 8192], [[1, 0]], 1, "hole|f16@0", "+"),
+         8192 * 8192, 8192, torch.float16),
+        ("ab->b 65536x1024 f32 add", E([1024, 65536], [[1, 0]], 1, "hole|f32@0", "+"),
+         65536 * 1024, 1024, torch.float32),
+        ("abc->ac 64x2048x1024 f16 max", E([64, 1024, 2048], [[0, 2, 1]], 2, "hole|f16@0", "^"),
+         64 * 2048 * 1024, 64 * 1024, torch.float16),
+    ]
+    stream = torch.cuda.current_stream().cuda_stream
+    rows = []
+    for name, e, n_in, n_out, dt in cases:
+        ws = km.build(e)
+        w = torch.empty(max(ws, 1), dtype=torch.uint8, device="cuda")
+        x = torch.randn(n_in, device="cuda", dtype=dt)
+        y = torch.empty(n_out, device="cuda", dtype=dt)
+        t = Timed()
+        for i in range(warmup + steps):
+            (t if i >= warmup else Timed()).record(
+                lambda: km(e, stream, y.data_ptr(), [x.data_ptr()],
+                           (w.data_ptr(), ws) if ws else None))
+        torch.cuda.synchronize()
+        nbytes = (n_in + n_out) * x.element_size()
+        rows.append({"node": name, "kernel": km.describe(e), "workspace_bytes": ws,
+                     "bytes": nbytes, "ms": round(t.mean_ms(), 5),
+                     "GBps": round(nbytes / t.mean_ms() / 1e6, 1),
+                     "hbm_frac": round(nbytes / t.mean_ms() / 1e6 / HBM_PEAK_GBPS, 4)})
+    return rows
+
+
 def run_copy(km, steps, warmup):
     """A plain copy of known size (1-D touch without castable, 512 MiB in, 512 MiB out): the
     yardstick the FETCH_SIZE / WRITE_SIZE counters are scaled by."""
@@ -590,6 +627,7 @@ def main():
     if args.workload == "all":
         others["mfma_f16_register_ceiling"] = run_mfma_peak(km)
         others["read_only_1GiB"] = run_read_ceiling(km, args.steps, args.warmup)
+        others["column_reductions"] = run_col_reductions(km, args.steps, args.warmup)
     if args.workload in ("llama", "all"):
         others["llama7b_contractions"] = run_llama_contractions(km, max(args.steps // 5, 3),
                                                                 max(args.warmup // 5, 1))

@@ -326,12 +326,14 @@ struct gen_t {
         src << ")\n{\n" << em.body.str() << "    return " << r << ";\n}\n";
     }
 
-    void args_struct()
+    // `with_ws`: a pointer to partial results (in the accumulator type) follows the inputs
+    void args_struct(bool with_ws = false)
     {
         src << "struct args_t {\n    " << storage_type(e.out_dtype()) << "* out;\n";
         for (int i = 0; i != L.NI; ++i) {
             src << "    const " << storage_type(e.inn_dtype(i)) << "* in" << i << ";\n";
         }
+        if (with_ws) src << "    " << compute_type(e.out_dtype()) << "* ws;\n";
         src << "    idx_t p[" << std::max(n_params, 1) << "];\n};\n";
     }
 
@@ -764,8 +766,27 @@ cg_kernel_t gen_reduce_col(einsummable_t const& e, int max_vec)
     int const V = any_vec ? pow2_divisor(L.shape[O - 1], vcap) : 1;
     uint64_t const n_vec = n_out / uint64_t(V);
     g.k.vec = V;
+    // Few outputs and a long aggregation: one thread per output vector leaves the device
+    // idle.  The outermost aggregated mode is then cut into slices that run side by side
+    // (grid z), each leaving partial results in the workspace; a second kernel folds the
+    // slices in order, so the result does not depend on scheduling.
+    uint64_t const outer = L.shape[O];
+    uint64_t const want_threads = 1ull << 16;  // measured: 32-64 K threads with 4 rows in flight each
+    uint64_t       S = 1;
+    if (n_vec * 2 <= want_threads && outer >= 16) {
+        S = std::min<uint64_t>({(want_threads + n_vec - 1) / n_vec, outer / 8, 1024});
+        S = uint64_t(std::max(1, env_int("ES_KM_RED_SPLITS", int(S))));
+        S = std::min<uint64_t>(S, outer);
+    }
+    uint64_t const chunk = (outer + S - 1) / S;
+    S = (outer + chunk - 1) / chunk;  // no empty slice
+    bool const split = S > 1;
+    g.k.splits = int(S);
+    g.k.ws_bytes = split ? S * n_out * dtype_size(od == dtype_t::f16 ? dtype_t::f32 : od) : 0;
 
     int p_nvec = g.param(n_vec);
+    int p_nout = g.param(n_out);
+    int p_chunk = g.param(chunk);
     int p_vpr = g.param(L.shape[O - 1] / uint64_t(V));
     std::vector<int> p_shape(R);
     for (int m = 0; m != R; ++m) p_shape[m] = g.param(L.shape[m]);
@@ -777,12 +798,33 @@ cg_kernel_t gen_reduce_col(einsummable_t const& e, int max_vec)
     }
 
     g.header();
-    g.args_struct();
+    g.args_struct(split);
     auto& s = g.src;
     std::string ACC = compute_type(od);
     s << "#define V " << V << "\n";
     s << "__device__ __forceinline__ " << ACC << " comb(" << ACC << " x, " << ACC
       << " y) { return " << combine_expr(cast, od, "x", "y") << "; }\n";
+    if (split) {
+        // second pass: fold the slices' partial results, in slice order
+        g.k.entry2 = g.k.entry + "_fold";
+        s << "extern \"C\" __global__ __launch_bounds__(256) void " << g.k.entry2
+          << "(args_t a)\n{\n";
+        s << "    const idx_t vid = ((idx_t)blockIdx.y * gridDim.x + blockIdx.x) * 256 + threadIdx.x;\n";
+        s << "    if (vid >= " << g.P(p_nvec) << ") return;\n";
+        s << "    " << ACC << " acc[V];\n";
+        s << "#pragma unroll\n    for (int j = 0; j != V; ++j) acc[j] = "
+          << identity_of(cast, od) << ";\n";
+        s << "    for (unsigned z = 0; z != " << S << "u; ++z) {\n";
+        s << "        const " << ACC << "* part = a.ws + (size_t)z * " << g.P(p_nout)
+          << " + (size_t)vid * V;\n";
+        s << "#pragma unroll\n        for (int j = 0; j != V; ++j) acc[j] = comb(acc[j], part[j]);\n";
+        s << "    }\n";
+        s << "    vec_t<" << storage_type(od) << ", V> res;\n";
+        s << "#pragma unroll\n    for (int j = 0; j != V; ++j) res.v[j] = "
+          << g.store_cast("acc[j]") << ";\n";
+        s << "    *reinterpret_cast<vec_t<" << storage_type(od)
+          << ", V>*>(a.out + vid * V) = res;\n}\n";
+    }
     s << "extern \"C\" __global__ __launch_bounds__(256) void " << g.k.entry << "(args_t a)\n{\n";
     s << "    const idx_t vid = ((idx_t)blockIdx.y * gridDim.x + blockIdx.x) * 256 + threadIdx.x;\n";
     s << "    if (vid >= " << g.P(p_nvec) << ") return;\n";
@@ -807,8 +849,19 @@ cg_kernel_t gen_reduce_col(einsummable_t const& e, int max_vec)
       << ";\n";
     std::string indent = "    ";
     for (int m = O; m != R; ++m) {
-        s << indent << "for (idx_t g" << m << " = 0; g" << m << " != " << g.P(p_shape[m]) << "; ++g"
-          << m << ") {\n";
+        if (m == O && split) {
+            s << indent << "const idx_t lo" << m << " = (idx_t)blockIdx.z * " << g.P(p_chunk) << ";\n";
+            s << indent << "const idx_t hi" << m << " = lo" << m << " + " << g.P(p_chunk) << " < "
+              << g.P(p_shape[m]) << " ? lo" << m << " + " << g.P(p_chunk) << " : "
+              << g.P(p_shape[m]) << ";\n";
+            if (m == R - 1) s << "#pragma unroll 4\n";  // several rows' loads in flight
+            s << indent << "for (idx_t g" << m << " = lo" << m << "; g" << m << " < hi" << m
+              << "; ++g" << m << ") {\n";
+        } else {
+            if (m == R - 1) s << "#pragma unroll 4\n";
+            s << indent << "for (idx_t g" << m << " = 0; g" << m << " != " << g.P(p_shape[m])
+              << "; ++g" << m << ") {\n";
+        }
         indent += "    ";
     }
     for (int k = 0; k != L.NI; ++k) {
@@ -843,10 +896,17 @@ cg_kernel_t gen_reduce_col(einsummable_t const& e, int max_vec)
         indent.resize(indent.size() - 4);
         s << indent << "}\n";
     }
-    s << "    vec_t<" << storage_type(od) << ", V> res;\n";
-    s << "#pragma unroll\n    for (int j = 0; j != V; ++j) res.v[j] = " << g.store_cast("acc[j]")
-      << ";\n";
-    s << "    *reinterpret_cast<vec_t<" << storage_type(od) << ", V>*>(a.out + vid * V) = res;\n";
+    if (split) {
+        s << "    " << ACC << "* part = a.ws + (size_t)blockIdx.z * " << g.P(p_nout)
+          << " + (size_t)vid * V;\n";
+        s << "#pragma unroll\n    for (int j = 0; j != V; ++j) part[j] = acc[j];\n";
+    } else {
+        s << "    vec_t<" << storage_type(od) << ", V> res;\n";
+        s << "#pragma unroll\n    for (int j = 0; j != V; ++j) res.v[j] = "
+          << g.store_cast("acc[j]") << ";\n";
+        s << "    *reinterpret_cast<vec_t<" << storage_type(od)
+          << ", V>*>(a.out + vid * V) = res;\n";
+    }
     s << "}\n";
 
     g.k.source = s.str();
@@ -917,8 +977,8 @@ namespace
 {
 
 struct module_cache_t {
-    std::mutex                                                    mu;
-    std::unordered_map<std::string, std::pair<hipModule_t, hipFunction_t>> by_source;
+    std::mutex                                   mu;
+    std::unordered_map<std::string, hipModule_t> by_source;
 };
 
 module_cache_t& module_cache()
@@ -927,33 +987,42 @@ module_cache_t& module_cache()
     return c;
 }
 
-hipFunction_t load_kernel(cg_kernel_t const& k)
-{
-    auto&                       cache = module_cache();
-    std::lock_guard<std::mutex> lock(cache.mu);
-    auto                        it = cache.by_source.find(k.source);
-    if (it != cache.by_source.end()) return it->second.second;
-    std::vector<char> code = compile_hip_source(k.source, "es_generated.hip", "gfx950");
-    hipModule_t       mod;
-    hipError_t        err = hipModuleLoadData(&mod, code.data());
-    if (err != hipSuccess) {
-        throw km_error(km_status::device,
-                       std::string("hipModuleLoadData: ") + hipGetErrorString(err));
-    }
-    hipFunction_t fn;
-    err = hipModuleGetFunction(&fn, mod, k.entry.c_str());
-    if (err != hipSuccess) {
-        throw km_error(km_status::device,
-                       std::string("hipModuleGetFunction: ") + hipGetErrorString(err));
-    }
-    cache.by_source.emplace(k.source, std::make_pair(mod, fn));
-    return fn;
-}
-
 struct variant_t {
     cg_kernel_t   k;
     hipFunction_t fn = nullptr;
+    hipFunction_t fn2 = nullptr;  // second pass of a split reduction
 };
+
+// Compiles (once per distinct source) and resolves the variant's entry points.
+void load_kernel(variant_t& v)
+{
+    auto&                       cache = module_cache();
+    std::lock_guard<std::mutex> lock(cache.mu);
+    hipModule_t                 mod;
+    auto                        it = cache.by_source.find(v.k.source);
+    if (it != cache.by_source.end()) {
+        mod = it->second;
+    } else {
+        std::vector<char> code = compile_hip_source(v.k.source, "es_generated.hip", "gfx950");
+        hipError_t        err = hipModuleLoadData(&mod, code.data());
+        if (err != hipSuccess) {
+            throw km_error(km_status::device,
+                           std::string("hipModuleLoadData: ") + hipGetErrorString(err));
+        }
+        cache.by_source.emplace(v.k.source, mod);
+    }
+    auto get = [&](std::string const& name) {
+        hipFunction_t fn;
+        hipError_t    err = hipModuleGetFunction(&fn, mod, name.c_str());
+        if (err != hipSuccess) {
+            throw km_error(km_status::device,
+                           std::string("hipModuleGetFunction: ") + hipGetErrorString(err));
+        }
+        return fn;
+    };
+    v.fn = get(v.k.entry);
+    if (v.k.splits > 1) v.fn2 = get(v.k.entry2);
+}
 
 struct codegen_plan_t : plan_t {
     einsummable_t     e;
@@ -963,15 +1032,20 @@ struct codegen_plan_t : plan_t {
 
     explicit codegen_plan_t(einsummable_t const& e_) : e(e_) {}
 
-    static void launch(variant_t const& v, hipStream_t stream, void* out, void const* const* inns)
+    static void launch(variant_t const& v, hipStream_t stream, void* out, void const* const* inns,
+                       void* workspace)
     {
-        // argument block: out pointer, input pointers, then idx_t parameters
+        // argument block: out pointer, input pointers, (partial results,) idx_t parameters
         unsigned char buf[1024];
         size_t        n = 0;
         std::memcpy(buf + n, &out, 8);
         n += 8;
         for (int i = 0; i != v.k.n_inns; ++i) {
             std::memcpy(buf + n, &inns[i], 8);
+            n += 8;
+        }
+        if (v.k.splits > 1) {
+            std::memcpy(buf + n, &workspace, 8);
             n += 8;
         }
         if (v.k.idx64) {
@@ -994,8 +1068,12 @@ struct codegen_plan_t : plan_t {
         uint64_t const gx_max = 1ull << 22;
         unsigned gx = unsigned(std::min<uint64_t>(v.k.grid, gx_max));
         unsigned gy = unsigned((v.k.grid + gx - 1) / gx);
-        hipError_t err = hipModuleLaunchKernel(v.fn, gx, gy, 1, v.k.block, 1, 1, 0, stream,
-                                               nullptr, config);
+        hipError_t err = hipModuleLaunchKernel(v.fn, gx, gy, unsigned(v.k.splits), v.k.block, 1, 1,
+                                               0, stream, nullptr, config);
+        if (err == hipSuccess && v.k.splits > 1) {
+            err = hipModuleLaunchKernel(v.fn2, gx, gy, 1, v.k.block, 1, 1, 0, stream, nullptr,
+                                        config);
+        }
         if (err != hipSuccess) {
             throw km_error(km_status::device,
                            std::string("hipModuleLaunchKernel: ") + hipGetErrorString(err));
@@ -1016,20 +1094,18 @@ struct codegen_plan_t : plan_t {
         return true;
     }
 
-    void run(hipStream_t stream, void* out, void const* const* inns, void*, uint64_t) const override
+    void run(hipStream_t stream, void* out, void const* const* inns, void* workspace,
+             uint64_t) const override
     {
         if (aligned(wide, out, inns)) {
-            launch(wide, stream, out, inns);
+            launch(wide, stream, out, inns, workspace);
             return;
         }
         {
             std::lock_guard<std::mutex> lock(mu);
-            if (!narrow.fn) {
-                narrow.k = generate_kernel(e, 1);
-                narrow.fn = load_kernel(narrow.k);
-            }
+            if (!narrow.fn) load_kernel(narrow);  // generated at plan time, compiled here
         }
-        launch(narrow, stream, out, inns);
+        launch(narrow, stream, out, inns, workspace);
     }
 };
 
@@ -1047,7 +1123,10 @@ std::shared_ptr<plan_t> plan_codegen(einsummable_t const& e, int)
     if (8 * (1 + k.n_inns) + 8 * k.params.size() > 1000) return nullptr;
     auto p = std::make_shared<codegen_plan_t>(e);
     p->wide.k = std::move(k);
-    p->wide.fn = load_kernel(p->wide.k);
+    load_kernel(p->wide);
+    // the scalar variant is only compiled if a misaligned buffer ever shows up, but its
+    // workspace need is part of what build() reports
+    p->narrow.k = generate_kernel(e, 1);
     switch (p->wide.k.kind) {
         case cg_kind::elementwise:
             p->description = "elementwise";
@@ -1060,7 +1139,8 @@ std::shared_ptr<plan_t> plan_codegen(einsummable_t const& e, int)
             break;
     }
     p->description += " vec=" + std::to_string(p->wide.k.vec);
-    p->workspace_bytes = 0;
+    if (p->wide.k.splits > 1) p->description += " splits=" + std::to_string(p->wide.k.splits);
+    p->workspace_bytes = std::max(p->wide.k.ws_bytes, p->narrow.k.ws_bytes);
     return p;
 }
 

@@ -30,6 +30,11 @@ struct cg_kernel_t {
     std::vector<uint64_t> params;        // written after the pointers as idx_t values
     // byte alignment every pointer must satisfy for this variant
     std::vector<int> out_inn_align;      // [0] = out, [1+k] = input k
+    // Two-pass reductions: `splits` > 1 slices of the aggregated range run side by side
+    // (grid z) and leave partial results in the workspace, which `entry2` then folds.
+    int         splits = 1;
+    std::string entry2;
+    uint64_t    ws_bytes = 0;
 };
 
 // Generate the kernel for a (merged) einsummable.  `max_vec` caps the vector width (1 forces

@@ -29,6 +29,9 @@ apply_graph_t::apply_graph_t(kernel_manager_t* km) : km_(km) {}
 apply_graph_t::~apply_graph_t()
 {
     for (size_t s = 1; s < streams_.size(); ++s) (void)hipStreamDestroy(streams_[s]);
+    for (void* w : workspace_) {
+        if (w) (void)hipFree(w);
+    }
     for (hipEvent_t e : events_) (void)hipEventDestroy(e);
     for (hipEvent_t e : joins_) (void)hipEventDestroy(e);
     if (fork_) (void)hipEventDestroy(fork_);
@@ -227,6 +230,17 @@ void apply_graph_t::finalize(int n_streams)
             event_of_[size_t(v)] = int(events_.size());
             events_.push_back(e);
         }
+        workspace_.assign(size_t(n_streams), nullptr);
+        workspace_bytes_.assign(size_t(n_streams), 0);
+        for (node_t const& nd : nodes_) {
+            if (nd.kind != kind_t::einsummable) continue;
+            uint64_t& need = workspace_bytes_[size_t(nd.stream)];
+            need = std::max(need, km_->workspace_size(nd.e));
+        }
+        for (int s = 0; s != n_streams; ++s) {
+            if (workspace_bytes_[size_t(s)] == 0) continue;
+            check(hipMalloc(&workspace_[size_t(s)], workspace_bytes_[size_t(s)]), "hipMalloc");
+        }
         check(hipEventCreateWithFlags(&fork_, hipEventDisableTiming), "hipEventCreateWithFlags");
         for (int s = 1; s != n_streams; ++s) {
             hipEvent_t e;
@@ -253,7 +267,8 @@ void apply_graph_t::launch(node_t const& n, hipStream_t stream, char* arena) con
                 ptrs = many.data();
             }
             for (size_t i = 0; i != k; ++i) ptrs[i] = arena + n.mems[i + 1].offset;
-            km_->run_plan(*p, stream, out, ptrs, int(k), nullptr, 0);
+            km_->run_plan(*p, stream, out, ptrs, int(k), workspace_[size_t(n.stream)],
+                          workspace_bytes_[size_t(n.stream)]);
             break;
         }
         case kind_t::touch:

@@ -102,6 +102,11 @@ private:
     std::vector<hipStream_t> streams_;
     std::vector<hipEvent_t>  events_;  // one per node that records
     std::vector<int>         event_of_;
+    // scratch for kernels that need it: one buffer per stream (a stream runs its nodes one
+    // after the other), sized for the stream's hungriest node; the reference takes these
+    // from a pool per launch (src/engine/gpu/workspace.cc:48-91)
+    std::vector<void*>       workspace_;
+    std::vector<uint64_t>    workspace_bytes_;
     hipEvent_t               fork_ = nullptr;
     std::vector<hipEvent_t>  joins_;
     int                      n_waits_ = 0;

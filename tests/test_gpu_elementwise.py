@@ -230,3 +230,62 @@ def test_error_contract(km):
         km.build(E([4, 4], [[0, 1]], 1, "hole|f32@0"))
     # scalar variables must be substituted by the caller: unsupported, not an error
     assert km.build(E([4], [[0]], 1, "*[variable{lr|f32},hole|f32@0]")) is None
+
+
+SPLIT_REDUCTIONS = [
+    # few outputs, long aggregation over an outer mode: slices of the aggregated range run
+    # side by side and a second kernel folds their partial results (needs a workspace)
+    (E([64, 4096], [[1, 0]], 1, "hole|f32@0", "+"), False),                 # ba->a
+    (E([256, 1000], [[1, 0]], 1, "hole|f16@0", "+"), False),
+    (E([256, 1000], [[1, 0]], 1, "hole|f16@0", "^"), True),
+    (E([3, 40, 777], [[0, 2, 1]], 2, "hole|f32@0", "v"), True),             # acb->ab
+    (E([24, 300, 5], [[1, 2, 0]], 1, "hole|f32@0", "+"), False),            # two aggregated modes
+    (E([128, 513], [[1, 0], [0]], 1, "*[hole|f32@0,hole|f32@1]", "+"), False),  # ba,a->a
+    (E([16, 3000], [[1, 0]], 1, "hole|f64@0", "+"), False),
+    (E([8, 2048], [[1, 0]], 1, "hole|c64@0", "+"), False),
+]
+
+
+@pytest.mark.parametrize("case", range(len(SPLIT_REDUCTIONS)))
+def test_split_column_reductions(km, case):
+    e, exact = SPLIT_REDUCTIONS[case]
+    ws = km.build(e)
+    assert ws is not None and ws > 0, "expected a two-pass plan"
+    assert "splits=" in km.describe(e) and km.workspace_size(e) == ws
+    check(km, e, seed=60 + case, exact=exact)
+
+
+def test_workspace_contract_of_a_two_pass_reduction(km):
+    import torch
+
+    e = E([64, 4096], [[1, 0]], 1, "hole|f32@0", "+")
+    ws = km.build(e)
+    assert ws > 0
+    x = torch.zeros(64 * 4096, device="cuda")
+    y = torch.zeros(64, device="cuda")
+    w = torch.zeros(ws, dtype=torch.uint8, device="cuda")
+    with pytest.raises(ea.KmError) as ei:          # no workspace
+        km(e, 0, y.data_ptr(), [x.data_ptr()])
+    assert ei.value.code == -3
+    with pytest.raises(ea.KmError) as ei:          # too small
+        km(e, 0, y.data_ptr(), [x.data_ptr()], (w.data_ptr(), ws - 1))
+    assert ei.value.code == -3
+    km(e, 0, y.data_ptr(), [x.data_ptr()], (w.data_ptr(), ws))
+    torch.cuda.synchronize()
+
+
+def test_two_pass_reduction_inside_an_exec_graph(km):
+    import torch
+
+    e = E([64, 4096], [[1, 0]], 1, "hole|f32@0", "+")
+    r = rng(70)
+    x = normal(r, 64 * 4096, np.float32)
+    arena = torch.zeros(64 * 4096 + 64, device="cuda")
+    arena[:64 * 4096] = torch.from_numpy(x).cuda()
+    g = ea.ApplyGraph(km)
+    g.add_einsummable(e, [(64 * 4096 * 4, 256), (0, 64 * 4096 * 4)])
+    g.finalize(2)
+    g.run(0, arena.data_ptr())
+    torch.cuda.synchronize()
+    want = x.reshape(4096, 64).astype(np.float64).sum(axis=0)
+    assert_close(arena[64 * 4096:].cpu().numpy(), want, ea.F32, what="exec graph two-pass")
