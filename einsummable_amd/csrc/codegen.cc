@@ -586,9 +586,24 @@ cg_kernel_t gen_reduce_row(einsummable_t const& e, int max_vec)
     int const U = env_int("ES_KM_RED_UNROLL",
                           (nvecA >= uint64_t(TEAM) * 4) ? 4 : ((nvecA >= uint64_t(TEAM) * 2) ? 2 : 1));
     g.k.vec = V;
+    // A handful of very long rows: one team per row leaves the device idle.  Each row is
+    // then cut into slices on grid z; a second kernel folds the slices' partial results in
+    // order (needs a workspace of slices x rows accumulators).
+    uint64_t S = 1, chunk = nvecA;
+    if (TEAM == 256 && n_out < 1024 && nvecA >= uint64_t(TEAM) * U * 16) {
+        S = std::min<uint64_t>({(2048 + n_out - 1) / n_out, nvecA / (uint64_t(TEAM) * U * 8), 4096});
+        S = uint64_t(std::max(1, env_int("ES_KM_RED_SPLITS", int(S))));
+        uint64_t const step = uint64_t(TEAM) * U;
+        chunk = ((nvecA + S - 1) / S + step - 1) / step * step;
+        S = (nvecA + chunk - 1) / chunk;
+    }
+    bool const split = S > 1;
+    g.k.splits = int(S);
+    g.k.ws_bytes = split ? S * n_out * dtype_size(od == dtype_t::f16 ? dtype_t::f32 : od) : 0;
 
     int p_nout = g.param(n_out);
     int p_nvec = g.param(nvecA);
+    int p_chunk = g.param(chunk);
     std::vector<int> p_shape(R);
     for (int m = 0; m != R; ++m) p_shape[m] = g.param(L.shape[m]);
     std::vector<std::vector<int>> p_str(L.NI, std::vector<int>(R, -1));
@@ -599,15 +614,34 @@ cg_kernel_t gen_reduce_row(einsummable_t const& e, int max_vec)
     }
 
     g.header();
-    g.args_struct();
+    g.args_struct(split);
     auto& s = g.src;
     std::string ACC = compute_type(od);
     s << "#define V " << V << "\n#define U " << U << "\n#define TEAM " << TEAM << "\n";
     s << "__device__ __forceinline__ " << ACC << " comb(" << ACC << " x, " << ACC
       << " y) { return " << combine_expr(cast, od, "x", "y") << "; }\n";
+    if (split) {
+        g.k.entry2 = g.k.entry + "_fold";
+        s << "extern \"C\" __global__ __launch_bounds__(" << BLOCK << ") void " << g.k.entry2
+          << "(args_t a)\n{\n";
+        s << "    const idx_t row = ((idx_t)blockIdx.y * gridDim.x + blockIdx.x) * " << BLOCK
+          << " + threadIdx.x;\n";
+        s << "    if (row >= " << g.P(p_nout) << ") return;\n";
+        s << "    " << ACC << " acc = " << identity_of(cast, od) << ";\n";
+        s << "    for (unsigned z = 0; z != " << S << "u; ++z) acc = comb(acc, a.ws[(size_t)z * "
+          << g.P(p_nout) << " + row]);\n";
+        s << "    a.out[row] = " << g.store_cast("acc") << ";\n}\n";
+    }
     s << "extern \"C\" __global__ __launch_bounds__(" << BLOCK << ") void " << g.k.entry << "(args_t a)\n{\n";
     s << "    const idx_t n_out = " << g.P(p_nout) << ";\n";
-    s << "    const idx_t nvec = " << g.P(p_nvec) << ";\n";
+    if (split) {
+        s << "    const idx_t v_lo = (idx_t)blockIdx.z * " << g.P(p_chunk) << ";\n";
+        s << "    const idx_t nvec = v_lo + " << g.P(p_chunk) << " < " << g.P(p_nvec) << " ? v_lo + "
+          << g.P(p_chunk) << " : " << g.P(p_nvec) << ";  // end of this slice\n";
+    } else {
+        s << "    const idx_t v_lo = 0;\n";
+        s << "    const idx_t nvec = " << g.P(p_nvec) << ";\n";
+    }
     s << "    const unsigned lane = threadIdx.x % TEAM;\n";
     s << "    const idx_t row = ((idx_t)blockIdx.y * gridDim.x + blockIdx.x) * (" << BLOCK << " / TEAM) + threadIdx.x / TEAM;\n";
     // min / max of f16 values is exact in f16: keep V packed half accumulators per lane
@@ -644,7 +678,7 @@ cg_kernel_t gen_reduce_row(einsummable_t const& e, int max_vec)
               << k << "[b" << k << "]);\n";
         }
     }
-    s << "        for (idx_t v0 = lane; v0 < nvec; v0 += (idx_t)TEAM * U) {\n";
+    s << "        for (idx_t v0 = v_lo + lane; v0 < nvec; v0 += (idx_t)TEAM * U) {\n";
     for (int k = 0; k != L.NI; ++k) {
         if (row_const[k]) continue;
         std::string T = storage_type(e.inn_dtype(k));
@@ -720,7 +754,11 @@ cg_kernel_t gen_reduce_row(einsummable_t const& e, int max_vec)
         s << "    __syncthreads();\n";
         s << "    if (threadIdx.x == 0 && row < n_out) {\n";
         s << "        acc = comb(comb(part[0], part[1]), comb(part[2], part[3]));\n";
-        s << "        a.out[row] = " << g.store_cast("acc") << ";\n    }\n";
+        if (split) {
+            s << "        a.ws[(size_t)blockIdx.z * n_out + row] = acc;\n    }\n";
+        } else {
+            s << "        a.out[row] = " << g.store_cast("acc") << ";\n    }\n";
+        }
     } else {
         s << "    if (lane == 0 && row < n_out) a.out[row] = " << g.store_cast("acc") << ";\n";
     }

@@ -289,3 +289,23 @@ def test_two_pass_reduction_inside_an_exec_graph(km):
     torch.cuda.synchronize()
     want = x.reshape(4096, 64).astype(np.float64).sum(axis=0)
     assert_close(arena[64 * 4096:].cpu().numpy(), want, ea.F32, what="exec graph two-pass")
+
+
+SPLIT_ROW_REDUCTIONS = [
+    # a handful of very long rows: each row is cut into slices that run side by side
+    (E([3, 131072], [[0, 1]], 1, "hole|f16@0", "+"), False),
+    (E([1, 262144], [[0, 1]], 1, "hole|f32@0", "^"), True),
+    (E([5, 70000], [[0, 1]], 1, "hole|f32@0", "+"), False),                      # ragged last slice
+    (E([2, 64, 2048], [[0, 1, 2]], 1, "hole|f16@0", "v"), True),                 # two aggregated modes
+    (E([2, 131072], [[0, 1], [0]], 1, "exp[+[hole|f16@0,*[constant{f16|-1},hole|f16@1]]]", "+"),
+     False),                                                                      # ab,a->a
+    (E([3, 40000], [[0, 1]], 1, "hole|f64@0", "+"), False),
+]
+
+
+@pytest.mark.parametrize("case", range(len(SPLIT_ROW_REDUCTIONS)))
+def test_split_row_reductions(km, case):
+    e, exact = SPLIT_ROW_REDUCTIONS[case]
+    ws = km.build(e)
+    assert ws is not None and ws > 0 and "splits=" in km.describe(e), km.describe(e)
+    check(km, e, seed=80 + case, exact=exact, sd=0.5)
