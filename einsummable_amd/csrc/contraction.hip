@@ -131,6 +131,7 @@ struct contraction_plan_t : plan_t {
     gemm_args_t args;
     dtype_t     dtype;
     bool        swapped;
+    bool        planned_dma = false;
     int         bm, bn;
 
     void run(hipStream_t stream, void* out, void const* const* inns, void*, uint64_t) const override
@@ -141,11 +142,20 @@ struct contraction_plan_t : plan_t {
         a.C = out;
         // vector paths need 16-byte aligned operands
         auto mis = [](void const* p) { return reinterpret_cast<uintptr_t>(p) % 16 != 0; };
+        bool const misaligned = mis(a.A) || mis(a.B) || mis(a.C);
         if (mis(a.A) && a.a_mode != 2) a.a_mode = 2;
         if (mis(a.B) && a.b_mode != 2) a.b_mode = 2;
         if (mis(a.C) && a.c_mode != 2) a.c_mode = 2;
-        // the wide epilogue lives in the tuned kernel (A along k, B along k or n)
-        if (a.c_mode == 3 && !(a.a_mode == 0 && a.b_mode != 2)) a.c_mode = 0;
+        // the wide epilogue lives in the direct-to-LDS kernel and in the register-staged
+        // one (A along k, B along k or n)
+        bool const dma = (dtype == dtype_t::f16 && gemm_dma_eligible<_Float16>(a)) ||
+                         (dtype == dtype_t::f32 && gemm_dma_eligible<float>(a));
+        if (a.c_mode == 3 && !dma && !(a.a_mode == 0 && a.b_mode != 2)) a.c_mode = 0;
+        // what build() described is what runs, unless a buffer's alignment forbids it
+        if (planned_dma && !dma && !misaligned) {
+            throw km_error(km_status::device,
+                           "contraction: the planned direct-to-LDS kernel cannot be launched");
+        }
         launch(a, stream);
         hipError_t err = hipGetLastError();
         if (err != hipSuccess) {
@@ -274,15 +284,20 @@ std::shared_ptr<plan_t> plan_contraction(einsummable_t const& e, int)
     a.offsets_fit_32 = e.inn_nelem(0) * dtype_size(dt) < (1ull << 32) &&
                        e.inn_nelem(1) * dtype_size(dt) < (1ull << 32);
 
-    // large tiles exist for the vector load paths (A along k; B along k or n)
     bool const dma_ok = (dt == dtype_t::f16 && gemm_dma_eligible<_Float16>(a)) ||
                         (dt == dtype_t::f32 && gemm_dma_eligible<float>(a));
-    if (a.a_mode == 0 && a.b_mode != 2) choose_tile(dt, M, N, K, Bt, dma_ok, p->bm, p->bn);
+    // large tiles exist in the direct-to-LDS kernel (both operands on a vector path) and, for
+    // A along k, in the register-staged one
+    if (dma_ok || (a.a_mode == 0 && a.b_mode != 2)) {
+        choose_tile(dt, M, N, K, Bt, dma_ok, p->bm, p->bn);
+    }
     a.tiles_m = uint32_t((M + p->bm - 1) / p->bm);
     a.tiles_n = uint32_t((N + p->bn - 1) / p->bn);
     if (uint64_t(a.tiles_m) * a.tiles_n >= lim) return nullptr;
 
     bool const dma = dma_ok;  // every tile has a direct-to-LDS kernel
+    p->planned_dma = dma && (dt == dtype_t::f16 ? gemm_dma_eligible<_Float16>(a)
+                                                : gemm_dma_eligible<float>(a));
     p->workspace_bytes = 0;
     static const char* mode_name[] = {"k", "mn", "elem"};
     p->description = std::string("contraction_mfma_") + dtype_name(dt) + " tile=" +

@@ -1,5 +1,6 @@
 // 256 x 256 macro-tile GEMM whose operand slices go from global memory straight into LDS
-// (global_load_lds_dwordx4), for problems where A is contiguous along k and B along k or n.
+// (global_load_lds_dwordx4), for problems where each operand is contiguous along k or along
+// its own m / n mode (all four matmul transposes and their batched / multi-mode relatives).
 //
 // Why a second kernel: with 128 x 128 tiles every flop costs twice the LDS and L1 traffic of a
 // 256 x 256 tile, and both are what limits the register-staged kernel.  A 256 x 256 tile per
@@ -49,7 +50,7 @@ __device__ __forceinline__ void wait_loads_and_lds()
     asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" : : "n"(VM) : "memory");
 }
 
-template <typename T, int BM, int BN, int NS, int BMODE>
+template <typename T, int BM, int BN, int NS, int AMODE, int BMODE>
 __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
 {
     using tr = traits_t<T>;
@@ -66,9 +67,13 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
     constexpr int NLA = BM / 64, NLB = BN / 64;
     static_assert(MI == 32 && tr::KG == 2 && STEPS == 2, "layout below assumes 32x32 tiles");
     static_assert(BM % 64 == 0 && BN % 64 == 0, "");
-    // B contiguous along n (BMODE 1) stays [k][n] in LDS: BK rows of BN elements
-    constexpr int RBN = BN * int(sizeof(T));  // bytes of one k row
-    constexpr int RPI = 1024 / RBN;           // k rows per load instruction
+    // An operand contiguous along m / n (mode 1) stays [k][m] / [k][n] in LDS: BK rows of
+    // BM / BN elements
+    constexpr int RAM = BM * int(sizeof(T));  // bytes of one k row of A
+    constexpr int RPIA = 1024 / RAM;          // k rows per load instruction
+    constexpr int RBN = BN * int(sizeof(T));
+    constexpr int RPI = 1024 / RBN;
+    static_assert(AMODE == 0 || (RAM <= 1024 && 1024 % RAM == 0), "");
     static_assert(BMODE == 0 || (RBN <= 1024 && 1024 % RBN == 0), "");
 
     extern __shared__ __attribute__((aligned(16))) char lds[];
@@ -121,21 +126,31 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
     // (lane % 4) ^ bits 2..3 of the row = (lane % 4) ^ ((lane / 16) % 4).
     uint32_t const load_chunk = uint32_t((lane & 3) ^ ((lane >> 4) & 3));
     uint32_t       voa[NLA], vob[NLB];
-#pragma unroll
-    for (int i = 0; i != NLA; ++i) {
-        uint32_t r = tm * BM + uint32_t((4 * i + wave) * 16 + lane / 4);
-        r = r < a.M ? r : a.M - 1;
-        int64_t x, y;
-        group_offsets(a.gm, r, x, y);
-        voa[i] = uint32_t(x) * uint32_t(sizeof(T));
-    }
-    // [k][n] rows of B: the 16-byte chunks of a row are permuted so that the fragment reads
-    // (which walk down k for a fixed n) spread over the banks; bits of the k row select which
-    // 64-byte (2-byte elements: rows k..k+3 are read together) or 128-byte (4-byte elements:
-    // rows k and k+4) segment a chunk lands in
+    // [k][m] / [k][n] rows: the 16-byte chunks of a row are permuted so that the fragment
+    // reads (which walk down k for a fixed m / n) spread over the banks; bits of the k row
+    // select which 64-byte (2-byte elements: rows k..k+3 are read together) or 128-byte
+    // (4-byte elements: rows k and k+4) segment a chunk lands in
     auto kn_swizzle = [](uint32_t r) {
         return sizeof(T) == 2 ? (r & 3) << 2 : ((r >> 2) & 1) << 3;
     };
+#pragma unroll
+    for (int i = 0; i != NLA; ++i) {
+        int64_t x, y;
+        if constexpr (AMODE == 0) {
+            uint32_t r = tm * BM + uint32_t((4 * i + wave) * 16 + lane / 4);
+            r = r < a.M ? r : a.M - 1;
+            group_offsets(a.gm, r, x, y);
+            voa[i] = uint32_t(x) * uint32_t(sizeof(T));
+        } else {
+            // this lane's slot: k row r of the slice, chunk c of that row
+            uint32_t const r = uint32_t(4 * i + wave) * RPIA + uint32_t(lane * 16) / RAM;
+            uint32_t const c = (uint32_t(lane * 16) % RAM) / 16;
+            uint32_t       m = tm * BM + (c ^ kn_swizzle(r)) * VL;
+            m = m < a.M ? m : a.M - VL;  // M is a multiple of VL on this path
+            group_offsets(a.gm, m, x, y);
+            voa[i] = (uint32_t(x) + r * uint32_t(a.gk.sx[0])) * uint32_t(sizeof(T));
+        }
+    }
 #pragma unroll
     for (int i = 0; i != NLB; ++i) {
         int64_t x, y;
@@ -157,9 +172,11 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
     // byte offsets of the lane's 16-byte chunk of slice kt within a row of A / of B
     auto k_offsets = [&](uint32_t kt, uint32_t& ka, uint32_t& kb) {
         uint32_t const k = kt * BK + load_chunk * VL;
-        if constexpr (BMODE == 1) {  // one k mode (checked by the launcher)
-            ka = k * uint32_t(sizeof(T));
-            kb = kt * BK * uint32_t(a.gk.sy[0]) * uint32_t(sizeof(T));
+        if constexpr (AMODE == 1 || BMODE == 1) {  // one k mode (checked by the launcher)
+            ka = AMODE == 1 ? kt * BK * uint32_t(a.gk.sx[0]) * uint32_t(sizeof(T))
+                            : k * uint32_t(sizeof(T));
+            kb = BMODE == 1 ? kt * BK * uint32_t(a.gk.sy[0]) * uint32_t(sizeof(T))
+                            : k * uint32_t(sizeof(T));
         } else if (a.gk.n == 1) {  // contiguous in both operands on this path
             ka = kb = k * uint32_t(sizeof(T));
         } else {
@@ -201,7 +218,25 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
     }
     int const fa_base = wm * WM * RB;
     int const fb_base = A_BYTES + wn * WN * RB;
-    // [k][n] B: byte offset of the lane's first element of MFMA tile j at k-step 0
+    // [k][m] A / [k][n] B: byte offset of the lane's first element of MFMA tile i / j at
+    // k-step 0.  ds_read_b64_tr_b16: within 16 lanes, lane i addresses 4 consecutive m (n) of
+    // k row i / 4 (column group i % 4) and receives, for its own m (n), 4 consecutive k.
+    int f_km[TM];
+    if constexpr (AMODE == 1) {
+#pragma unroll
+        for (int i = 0; i != TM; ++i) {
+            if constexpr (sizeof(T) == 2) {
+                int const i16 = lane & 15, blk = lane >> 4;
+                int const m0 = wm * WM + i * MI + (blk & 1) * 16 + 4 * (i16 & 3);
+                int const k0 = (blk >> 1) * VL + (i16 >> 2);
+                f_km[i] = k0 * RAM + ((m0 * 2) ^ int(kn_swizzle(uint32_t(k0)) * 16));
+            } else {
+                int const m0 = wm * WM + i * MI + lane % MI;
+                int const k0 = (lane / MI) * VL;
+                f_km[i] = k0 * RAM + ((m0 * 4) ^ int(kn_swizzle(uint32_t(k0)) * 16));
+            }
+        }
+    }
     int f_kn[TN];
     if constexpr (BMODE == 1) {
 #pragma unroll
@@ -222,38 +257,50 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
     }
 
     chunk_t fa[2][TM], fb[2][TN];
+    // a fragment of an operand kept [k][row] in LDS: transposing read (2-byte elements) or
+    // one element per k row (4-byte elements); rows k..k+3 and k+4..k+7 share their low two
+    // bits, rows k0..k0+3 of one lane share bit 2, hence their swizzle
+    auto read_transposed = [&](char const* p, int row_bytes) {
+        if constexpr (sizeof(T) == 2) {
+            typedef short tr_t __attribute__((ext_vector_type(4)));
+            typedef short tr8_t __attribute__((ext_vector_type(8)));
+            tr_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (__attribute__((address_space(3))) tr_t*)(p));
+            tr_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (__attribute__((address_space(3))) tr_t*)(p + 4 * row_bytes));
+            tr8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            return __builtin_bit_cast(chunk_t, both);
+        } else {
+            chunk_t v;
+#pragma unroll
+            for (int t = 0; t != VL; ++t) {
+                v[t] = *reinterpret_cast<uint32_t const*>(p + t * row_bytes);
+            }
+            return v;
+        }
+    };
+    auto read_a = [&](char const* stage, int s, int i) {
+        if constexpr (AMODE == 0) {
+            return *reinterpret_cast<chunk_t const*>(stage + fa_base + i * MI * RB + f_off[s]);
+        } else {
+            return read_transposed(stage + f_km[i] + s * tr::KG * VL * RAM, RAM);
+        }
+    };
+    auto read_b = [&](char const* stage, int s, int j) {
+        if constexpr (BMODE == 0) {
+            return *reinterpret_cast<chunk_t const*>(stage + fb_base + j * MI * RB + f_off[s]);
+        } else {
+            return read_transposed(stage + A_BYTES + f_kn[j] + s * tr::KG * VL * RBN, RBN);
+        }
+    };
     // read order: what the first matrix instructions of a step need comes first
     auto read_frag = [&](char const* stage, int s, int q, chunk_t(&xa)[TM], chunk_t(&xb)[TN]) {
         if (q == 0) {
-            xa[0] = *reinterpret_cast<chunk_t const*>(stage + fa_base + f_off[s]);
+            xa[0] = read_a(stage, s, 0);
         } else if (q <= TN) {
-            if constexpr (BMODE == 0) {
-                xb[q - 1] = *reinterpret_cast<chunk_t const*>(stage + fb_base +
-                                                              (q - 1) * MI * RB + f_off[s]);
-            } else if constexpr (sizeof(T) == 2) {
-                // rows k..k+3 and k+4..k+7 share their low two bits, hence their swizzle
-                typedef short tr_t __attribute__((ext_vector_type(4)));
-                typedef short tr8_t __attribute__((ext_vector_type(8)));
-                char const* p = stage + A_BYTES + f_kn[q - 1] + s * tr::KG * VL * RBN;
-                tr_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (__attribute__((address_space(3))) tr_t*)(p));
-                tr_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (__attribute__((address_space(3))) tr_t*)(p + 4 * RBN));
-                tr8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-                xb[q - 1] = __builtin_bit_cast(chunk_t, both);
-            } else {
-                // rows k0..k0+3 of one lane share bit 2, hence their swizzle
-                char const* p = stage + A_BYTES + f_kn[q - 1] + s * tr::KG * VL * RBN;
-                chunk_t     v;
-#pragma unroll
-                for (int t = 0; t != VL; ++t) {
-                    v[t] = *reinterpret_cast<uint32_t const*>(p + t * RBN);
-                }
-                xb[q - 1] = v;
-            }
+            xb[q - 1] = read_b(stage, s, q - 1);
         } else {
-            xa[q - TN] = *reinterpret_cast<chunk_t const*>(stage + fa_base + (q - TN) * MI * RB +
-                                                           f_off[s]);
+            xa[q - TN] = read_a(stage, s, q - TN);
         }
     };
     constexpr int READS = TM + TN;
@@ -399,33 +446,44 @@ template <typename T>
 bool gemm_dma_eligible(gemm_args_t const& a)
 {
     constexpr uint32_t BK = DMA_ROW / sizeof(T);
+    // an operand contiguous along m / n needs a single k mode (its k rows are addressed by
+    // one stride)
+    bool const a_ok = a.a_mode == 0 || (a.a_mode == 1 && a.gk.n == 1);
     bool const b_ok = a.b_mode == 0 || (a.b_mode == 1 && a.gk.n == 1);
-    return a.a_mode == 0 && b_ok && a.c_mode == 3 && a.K % BK == 0 && a.K / BK >= 4 &&
+    return a_ok && b_ok && a.c_mode == 3 && a.K % BK == 0 && a.K / BK >= 4 &&
            a.offsets_fit_32 != 0;
 }
 
-template <typename T, int BM, int BN, int NS, int BMODE>
+template <typename T, int BM, int BN, int NS, int AMODE, int BMODE>
 void launch_gemm_dma_kernel_mode(gemm_args_t const& a, hipStream_t stream)
 {
     static_assert(NS >= 2 && NS <= 4, "eligibility guarantees four slices");
     constexpr int lds = NS * (BM + BN) * DMA_ROW;
     static bool const raised = [] {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_dma_kernel<T, BM, BN, NS, BMODE>),
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_dma_kernel<T, BM, BN, NS, AMODE, BMODE>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         return true;
     }();
     (void)raised;
     dim3 grid(a.tiles_m * a.tiles_n, a.batch, 1);
-    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, NS, BMODE>), grid, dim3(256), lds, stream, a);
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, NS, AMODE, BMODE>), grid, dim3(256), lds, stream, a);
 }
 
 template <typename T, int BM, int BN, int NS>
 void launch_gemm_dma_kernel(gemm_args_t const& a, hipStream_t stream)
 {
-    if (a.b_mode == 0) {
-        launch_gemm_dma_kernel_mode<T, BM, BN, NS, 0>(a, stream);
+    if (a.a_mode == 0) {
+        if (a.b_mode == 0) {
+            launch_gemm_dma_kernel_mode<T, BM, BN, NS, 0, 0>(a, stream);
+        } else {
+            launch_gemm_dma_kernel_mode<T, BM, BN, NS, 0, 1>(a, stream);
+        }
     } else {
-        launch_gemm_dma_kernel_mode<T, BM, BN, NS, 1>(a, stream);
+        if (a.b_mode == 0) {
+            launch_gemm_dma_kernel_mode<T, BM, BN, NS, 1, 0>(a, stream);
+        } else {
+            launch_gemm_dma_kernel_mode<T, BM, BN, NS, 1, 1>(a, stream);
+        }
     }
 }
 

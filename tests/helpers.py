@@ -103,7 +103,8 @@ def assert_close(got, want, es_dtype, scale=None, what=""):
         mag = np.abs(want[finite])
         scale = float(np.sqrt(np.mean(mag * mag))) if mag.size else 1.0
         scale = max(scale, 1e-30)
-    err = np.abs(got - want)
+    with np.errstate(invalid="ignore"):   # inf - inf where both sides overflowed alike
+        err = np.abs(got - want)
     bound = RTOL[es_dtype] * np.maximum(np.abs(want), scale)
     bad = ~fine & ~(err <= bound)
     if bad.any():

@@ -149,6 +149,14 @@ BIG_TILE_CASES = [
     ("ij,jk->ik", dict(i=264, j=80, k=264), "f32", True),
     ("ij,jk->ik", dict(i=130, j=64, k=520), "f32", True),
     ("bij,bjk->bik", dict(b=2, i=40, j=112, k=72), "f32", True),
+    # A contiguous along m (a transposed lhs), with B along n or along k
+    ("ji,jk->ik", dict(i=264, j=160, k=264), "f16", True),
+    ("ji,kj->ik", dict(i=520, j=128, k=264), "f16", True),
+    ("ji,jk->ik", dict(i=24, j=256, k=40), "f16", True),
+    ("bji,bjk->bik", dict(b=3, i=136, j=192, k=264), "f16", True),
+    ("jk,ji->ik", dict(i=264, j=160, k=136), "f16", True),      # operands swapped by the planner
+    ("ji,jk->ik", dict(i=264, j=80, k=264), "f32", True),
+    ("ji,kj->ik", dict(i=132, j=64, k=520), "f32", True),
     # K not a whole number of slices, or too short: the register-staged kernels
     ("ij,kj->ik", dict(i=264, j=72, k=264), "f16", False),
     ("ij,kj->ik", dict(i=264, j=296, k=264), "f16", False),
