@@ -491,10 +491,10 @@ def run_mfma_peak(km):
 
 
 def run_read_ceiling(km, steps, warmup):
-    """What a kernel that only reads reaches on this device: the generated row max over
-    1 GiB of f16 next to the vendor library's reduction (torch.amax) over the same tensor.
-    Both stop near 4.8 TB/s, well below the 8 TB/s that mixed read + write traffic is
-    priced against."""
+    """A kernel that only reads, on memory nobody has just written: the generated row max
+    over 1 GiB of f16 next to the vendor library's reduction (torch.amax) over the same
+    tensor.  Inside the attention chain the same kernel on the same shape is slower, because
+    there its input has just been written by the preceding node."""
     import torch
 
     import einsummable_amd as ea
