@@ -135,6 +135,23 @@ void kernel_manager_t::operator()(touch_t const& touch_, hipStream_t stream, voi
                 (reinterpret_cast<uintptr_t>(out) % 16 == 0) &&
                 (reinterpret_cast<uintptr_t>(inn) % 16 == 0);
     if (r > 1) wide = wide && (last.d_inn % vmax == 0) && (last.d_out % vmax == 0);
+    if (!wide && vmax > 1) {
+        // A window that is not vector aligned, in an output whose rows are: the kernel of
+        // the grouped path walks the output in 16-byte vectors and handles the window's
+        // ragged edges and the unaligned input element by element.
+        bool out_rows_wide = reinterpret_cast<uintptr_t>(out) % 16 == 0 &&
+                             (r == 1 || last.d_out % uint64_t(vmax) == 0);
+        uint64_t volume = 1;
+        for (auto const& d : t.selection) {
+            out_rows_wide = out_rows_wide && d.d_out < (1ull << 32);
+            volume *= d.size;
+        }
+        // (small windows are bound by the launch, and this path costs more on the host)
+        if (out_rows_wide && volume >= (1ull << 21)) {
+            touch_batch({t}, stream, out, {inn});
+            return;
+        }
+    }
 
     touch_launch_t a;
     a.vec = wide ? vmax : 1;

@@ -224,3 +224,19 @@ def test_touch_batch_errors(km):
         km.touch_batch([a, b], 0, d.data_ptr(), [d.data_ptr(), d.data_ptr()])
     assert ei.value.code == -1
     km.touch_batch([], 0, d.data_ptr(), [])
+
+
+@pytest.mark.parametrize("dt,castable", [(ea.F16, "+"), (ea.F16, None), (ea.F32, "^"), (ea.C64, "+")])
+def test_large_touch_whose_window_is_not_vector_aligned(km, dt, castable):
+    """Windows of a few million elements at odd offsets (input and output phases differ):
+    they run on 16-byte output vectors with element-wise edges; bit-identical to the oracle."""
+    r = rng(90 + dt)
+    rows, cols = 1500, 2048
+    t = ea.Touch([(rows + 3, rows + 8, 2, 5, rows), (cols + 24, cols + 32, 7, 13, cols - 11)],
+                 castable, dt)
+    blk = normal(r, (rows + 3) * (cols + 24), NP[dt], 0.5)
+    out0 = normal(r, (rows + 8) * (cols + 32), NP[dt], 0.5)
+    want = _apply_sequentially([t], [blk], out0)
+    d_out, d_blk = to_device(out0), to_device(blk)
+    km.touch(t, stream_handle(), d_out.data_ptr(), d_blk.data_ptr())
+    assert_bits_equal(to_host(d_out, NP[dt]), want, "large unaligned touch")
