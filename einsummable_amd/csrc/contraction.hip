@@ -134,9 +134,11 @@ struct contraction_plan_t : plan_t {
     bool        planned_dma = false;
     int         bm, bn;
 
-    void run(hipStream_t stream, void* out, void const* const* inns, void*, uint64_t) const override
+    void run(hipStream_t stream, void* out, void const* const* inns, void* workspace,
+             uint64_t) const override
     {
         gemm_args_t a = args;
+        a.ws = static_cast<float*>(workspace);
         a.A = swapped ? inns[1] : inns[0];
         a.B = swapped ? inns[0] : inns[1];
         a.C = out;
@@ -152,6 +154,7 @@ struct contraction_plan_t : plan_t {
                          (dtype == dtype_t::f32 && gemm_dma_eligible<float>(a));
         if (a.c_mode == 3 && !dma && !(a.a_mode == 0 && a.b_mode != 2)) a.c_mode = 0;
         // what build() described is what runs, unless a buffer's alignment forbids it
+        if (!dma) a.splits = 1;  // only the direct-to-LDS kernel splits k
         if (planned_dma && !dma && !misaligned) {
             throw km_error(km_status::device,
                            "contraction: the planned direct-to-LDS kernel cannot be launched");
@@ -298,7 +301,23 @@ std::shared_ptr<plan_t> plan_contraction(einsummable_t const& e, int)
     bool const dma = dma_ok;  // every tile has a direct-to-LDS kernel
     p->planned_dma = dma && (dt == dtype_t::f16 ? gemm_dma_eligible<_Float16>(a)
                                                 : gemm_dma_eligible<float>(a));
+    // Too few tiles for the device and a long reduction (skinny products, e.g. one token
+    // against a weight matrix): several workgroups share a tile's k range and a second
+    // kernel sums their fp32 partial tiles, which live in the workspace.
+    a.splits = 1;
     p->workspace_bytes = 0;
+    uint64_t const tiles = uint64_t(a.tiles_m) * a.tiles_n * Bt;
+    uint64_t const nk = K * dtype_size(dt) / 64;
+    if (p->planned_dma && tiles <= 128 && nk >= 16) {
+        uint64_t S = std::min<uint64_t>({256 / tiles, nk / 8, 64});
+        if (const char* env = std::getenv("ES_KM_GEMM_SPLITS")) {  // tuning and tests
+            S = std::min<uint64_t>(uint64_t(std::max(1, std::atoi(env))), nk / 4);
+        }
+        if (S > 1) {
+            a.splits = uint32_t(S);
+            p->workspace_bytes = S * Bt * M * N * 4;
+        }
+    }
     static const char* mode_name[] = {"k", "mn", "elem"};
     p->description = std::string("contraction_mfma_") + dtype_name(dt) + " tile=" +
                      std::to_string(p->bm) + "x" + std::to_string(p->bn) + " A=" +
@@ -306,7 +325,8 @@ std::shared_ptr<plan_t> plan_contraction(einsummable_t const& e, int)
                      (a.c_mode == 3 ? "wide" : (a.c_mode == 0 ? "vec" : "elem")) +
                      (swapped ? " swapped" : "") + (dma ? " load=direct_to_lds" : "") +
                      " M=" + std::to_string(M) + " N=" + std::to_string(N) + " K=" +
-                     std::to_string(K) + " batch=" + std::to_string(Bt);
+                     std::to_string(K) + " batch=" + std::to_string(Bt) +
+                     (a.splits > 1 ? " split_k=" + std::to_string(a.splits) : "");
     return p;
 }
 

@@ -316,13 +316,21 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
     constexpr int R1 = (READS + MMAS - 2) / (MMAS - 1);
     constexpr int L1 = (LOADS + MMAS - 2) / (MMAS - 1);
 
-    uint32_t const nk = a.K / BK;  // >= NS, no remainder (checked by the launcher)
+    // k slices of this workgroup: all of them, or this split's share (the first K/BK mod
+    // splits shares are one slice longer); every share has at least NS slices
+    uint32_t k_begin = 0;
+    uint32_t nk = a.K / BK;  // >= NS, no remainder (checked by the launcher)
+    if (a.splits > 1) {
+        uint32_t const q = nk / a.splits, r = nk % a.splits, z = blockIdx.z;
+        k_begin = z * q + (z < r ? z : r);
+        nk = q + (z < r ? 1 : 0);
+    }
 
     // prologue: four slices in flight, the first one landed
 #pragma unroll
     for (int s = 0; s != NS; ++s) {
         uint32_t ka, kb;
-        k_offsets(uint32_t(s), ka, kb);
+        k_offsets(k_begin + uint32_t(s), ka, kb);
 #pragma unroll
         for (int q = 0; q != LOADS; ++q) issue(uint32_t(s), q, ka, kb);
     }
@@ -339,7 +347,7 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
         char const*    cur = lds + (kt % NS) * STAGE;
         char const*    nxt = lds + ((kt + 1) % NS) * STAGE;
         uint32_t       ka = 0, kb = 0;
-        if (ISSUE) k_offsets(kt + NS, ka, kb);
+        if (ISSUE) k_offsets(k_begin + kt + NS, ka, kb);
 #pragma unroll
         for (int q = 0; q != MMAS; ++q) {
             int const p = q % PAIRS;
@@ -391,6 +399,27 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
 
     // Epilogue: each wave turns MI rows of its tile through a private LDS strip so that the
     // global stores are 16 bytes per lane and whole row segments per wavefront.
+    if (a.splits > 1) {
+        // partial tile, fp32: every lane holds four consecutive n of one m per register quad
+        float* const part = a.ws + (size_t(blockIdx.z) * a.batch + bz) * a.M * size_t(a.N);
+#pragma unroll
+        for (int i = 0; i != TM; ++i) {
+            uint32_t const m = tm * BM + wm * WM + i * MI + uint32_t(lane % MI);
+#pragma unroll
+            for (int j = 0; j != TN; ++j) {
+#pragma unroll
+                for (int e0 = 0; e0 < tr::NACC; e0 += 4) {
+                    uint32_t const n = tn * BN + wn * WN + j * MI + uint32_t(tr::acc_row(e0, lane));
+                    if (m < a.M && n < a.N) {  // N is a multiple of 4 on this path
+                        float4_t q = {float(acc[i][j][e0]), float(acc[i][j][e0 + 1]),
+                                      float(acc[i][j][e0 + 2]), float(acc[i][j][e0 + 3])};
+                        *reinterpret_cast<float4_t*>(part + size_t(m) * a.N + n) = q;
+                    }
+                }
+            }
+        }
+        return;
+    }
     T* const C = static_cast<T*>(a.C) + boc;
     constexpr int STRIP_PITCH = WN * int(sizeof(T)) + 16;
     constexpr int CPR = WN * int(sizeof(T)) / 16;
@@ -465,8 +494,53 @@ void launch_gemm_dma_kernel_mode(gemm_args_t const& a, hipStream_t stream)
         return true;
     }();
     (void)raised;
-    dim3 grid(a.tiles_m * a.tiles_n, a.batch, 1);
+    dim3 grid(a.tiles_m * a.tiles_n, a.batch, a.splits > 1 ? a.splits : 1);
     hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, NS, AMODE, BMODE>), grid, dim3(256), lds, stream, a);
+}
+
+// Second pass of a split-K contraction: C = sum over the splits' partial tiles, in split
+// order (deterministic), converted to T.  One thread per four consecutive n.
+template <typename T>
+__global__ __launch_bounds__(256) void gemm_fold_kernel(gemm_args_t a)
+{
+    uint64_t const quads_per_row = a.N / 4;
+    uint64_t const total = uint64_t(a.batch) * a.M * quads_per_row;
+    uint64_t const id = uint64_t(blockIdx.x) * 256 + threadIdx.x;
+    if (id >= total) return;
+    uint32_t const n = uint32_t(id % quads_per_row) * 4;
+    uint64_t const rest = id / quads_per_row;
+    uint32_t const m = uint32_t(rest % a.M);
+    uint32_t const bz = uint32_t(rest / a.M);
+    size_t const   plane = size_t(a.batch) * a.M * size_t(a.N);
+    float const*   p = a.ws + (size_t(bz) * a.M + m) * a.N + n;
+    float4_t       sum = {0, 0, 0, 0};
+    for (uint32_t z = 0; z != a.splits; ++z) {
+        sum += *reinterpret_cast<float4_t const*>(p + size_t(z) * plane);
+    }
+    int64_t boc = 0;
+    {
+        uint32_t i = bz;
+#pragma unroll
+        for (int d = 0; d != MAXG; ++d) {
+            uint32_t q = i / a.gb.size[d];
+            boc += int64_t(i - q * a.gb.size[d]) * a.gb.sz[d];
+            i = q;
+        }
+    }
+    int64_t mo_a, mo_c, no_b, no_c;
+    group_offsets(a.gm, m, mo_a, mo_c);
+    group_offsets(a.gn, n, no_b, no_c);
+    typedef T quad_t __attribute__((ext_vector_type(4)));
+    quad_t out = {T(sum[0]), T(sum[1]), T(sum[2]), T(sum[3])};
+    *reinterpret_cast<quad_t*>(static_cast<T*>(a.C) + boc + mo_c + no_c) = out;
+}
+
+template <typename T>
+void launch_gemm_fold(gemm_args_t const& a, hipStream_t stream)
+{
+    uint64_t const total = uint64_t(a.batch) * a.M * (a.N / 4);
+    hipLaunchKernelGGL((gemm_fold_kernel<T>), dim3(unsigned((total + 255) / 256)), dim3(256), 0,
+                       stream, a);
 }
 
 template <typename T, int BM, int BN, int NS>
@@ -485,6 +559,7 @@ void launch_gemm_dma_kernel(gemm_args_t const& a, hipStream_t stream)
             launch_gemm_dma_kernel_mode<T, BM, BN, NS, 1, 1>(a, stream);
         }
     }
+    if (a.splits > 1) launch_gemm_fold<T>(a, stream);
 }
 
 }  // namespace gemm

@@ -38,6 +38,11 @@ struct gemm_args_t {
                                  // 3: 16-byte row segments through LDS (tuned kernel)
     int         offsets_fit_32;  // every byte offset into A and B (per batch entry) < 2^32
     int         c_stream;        // C exceeds the caches: store it non-temporally
+    // Split-K (direct-to-LDS kernel): `splits` workgroups per tile, one per grid z, each
+    // over its own range of k slices, leave fp32 partial tiles in `ws`
+    // ([split][batch][M][N]); gemm_fold_kernel sums them into C.
+    uint32_t    splits;
+    float*      ws;
 };
 
 __device__ __forceinline__ void group_offsets(group_t const& g, uint32_t i, int64_t& ox,

@@ -203,11 +203,15 @@ class DeviceRunner:
         self.km, self.g, self.torch = km, graph, torch
         self.mem = {name: torch.empty(nbytes, dtype=torch.uint8, device="cuda")
                     for name, nbytes in graph.buffers.items()}
+        need = 0
         for n in graph.nodes:
             if n["kind"] == "einsummable":
                 ws = km.build(n["e"])
                 assert ws is not None, "no kernel for node " + n["label"]
-                assert ws == 0
+                n["ws"] = ws
+                need = max(need, ws)
+        # one scratch buffer serves every node: they run one after the other on one stream
+        self.workspace = torch.empty(max(need, 1), dtype=torch.uint8, device="cuda")
 
     def set_input(self, name, array):
         import numpy as np
@@ -228,7 +232,8 @@ class DeviceRunner:
             def launch(n=n):
                 if n["kind"] == "einsummable":
                     km(n["e"], stream, self.mem[n["out"]].data_ptr(),
-                       [self.mem[b].data_ptr() for b in n["inns"]])
+                       [self.mem[b].data_ptr() for b in n["inns"]],
+                       (self.workspace.data_ptr(), n["ws"]) if n["ws"] else None)
                 elif n["kind"] == "touch":
                     km.touch(n["t"], stream, self.mem[n["out"]].data_ptr(),
                              self.mem[n["inn"]].data_ptr())

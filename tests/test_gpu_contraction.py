@@ -198,3 +198,43 @@ def test_big_tile_matches_small_tile_bitwise_on_exact_data(km, monkeypatch):
             xs[1].astype(np.float64).reshape(392, 256).T).astype(np.float16)
     np.testing.assert_array_equal(a.view(np.uint16), b.view(np.uint16))
     np.testing.assert_array_equal(a.reshape(520, 392), want)
+
+
+SPLIT_K_CASES = [
+    # few tiles and a long reduction: several workgroups per tile, fp32 partial tiles in the
+    # workspace, a fold kernel; all four operand layouts, batch, ragged m / n, a one-row lhs
+    ("ij,kj->ik", dict(i=8, j=2048, k=264), "f16"),
+    ("ij,jk->ik", dict(i=1, j=1024, k=256), "f16"),
+    ("ji,jk->ik", dict(i=136, j=1536, k=72), "f16"),
+    ("ji,kj->ik", dict(i=40, j=1024, k=136), "f16"),
+    ("bij,bkj->bik", dict(b=3, i=24, j=1024, k=40), "f16"),
+    ("ij,kj->ik", dict(i=130, j=1008, k=136), "f32"),
+    ("ij,jk->ik", dict(i=8, j=4096, k=64), "f32"),
+]
+
+
+@pytest.mark.parametrize("case", range(len(SPLIT_K_CASES)))
+def test_split_k_contractions(km, case):
+    spec, sizes, dt = SPLIT_K_CASES[case]
+    e = contraction(spec, sizes, dt)
+    ws = km.build(e)
+    assert ws and "split_k=" in km.describe(e), km.describe(e)
+    check(km, spec, sizes, dt, seed=40 + case)
+
+
+def test_split_k_is_deterministic_and_checks_its_workspace(km):
+    import torch
+    from helpers import stream_handle
+
+    e = contraction("ij,kj->ik", dict(i=8, j=2048, k=264), "f16")
+    ws = km.build(e)
+    assert ws > 0
+    r = rng(50)
+    xs = [uniform(r, 8 * 2048, np.float16), uniform(r, 264 * 2048, np.float16)]
+    a = run_einsummable(km, e, xs)
+    b = run_einsummable(km, e, xs)
+    np.testing.assert_array_equal(a.view(np.uint16), b.view(np.uint16))
+    d = torch.zeros(264 * 2048, dtype=torch.float16, device="cuda")
+    with pytest.raises(ea.KmError) as ei:
+        km(e, stream_handle(), d.data_ptr(), [d.data_ptr(), d.data_ptr()])
+    assert ei.value.code == -3
