@@ -21,6 +21,7 @@ from .km import (  # noqa: F401
     codegen_source,
     lib_path,
     load_library,
+    memgraph_describe,
     merge_adjacent_dims,
     scalarop_roundtrip,
 )

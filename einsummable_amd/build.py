@@ -19,7 +19,7 @@ SOURCES = [
     "ir.cc",
     "kernel_manager.cc",
     "c_api.cc",
-    "exec_graph.cc",
+    "exec_graph.cc", "memgraph_wire.cc",
     "codegen.cc",
     "touch.hip",
     "transpose.hip",

@@ -5,6 +5,7 @@
 
 #include "codegen.h"
 #include "exec_graph.h"
+#include "memgraph_wire.h"
 #include "gemm_kernel.h"
 #include "kernel_manager.h"
 
@@ -91,6 +92,60 @@ int guarded(es_km_t* h, F&& f)
         err_slot(h) = e.what();
         return ES_KM_ERR_DEVICE;
     }
+}
+
+// One line per node, every decoded field in a fixed order.
+std::string describe_memgraph(es::memgraph_t const& mg)
+{
+    auto u = [](uint64_t v) { return std::to_string(v); };
+    auto list = [&](auto const& xs) {
+        std::string s = "[";
+        for (size_t i = 0; i != xs.size(); ++i) s += (i ? "," : "") + std::to_string(xs[i]);
+        return s + "]";
+    };
+    std::string out = "memgraph compute_locs=" + std::to_string(mg.num_compute_locs) +
+                      " storage_locs=" + std::to_string(mg.num_storage_locs) + " map=" +
+                      list(mg.storage_locs) + " nodes=" + std::to_string(mg.nodes.size()) + "\n";
+    for (size_t id = 0; id != mg.nodes.size(); ++id) {
+        es::mg_node_t const& n = mg.nodes[id];
+        out += std::to_string(id) + " kind=" + std::to_string(int(n.kind)) +
+               " loc=" + std::to_string(n.loc) + " src_loc=" + std::to_string(n.src_loc) +
+               " offset=" + u(n.offset) + " size=" + u(n.size) + " src_offset=" + u(n.src_offset) +
+               " storage=" + std::to_string(n.storage_loc) + ":" + std::to_string(n.storage_id) +
+               " group=" + std::to_string(n.group) + " inns=" + list(n.inns) + " mems=[";
+        for (size_t i = 0; i != n.mems.size(); ++i) {
+            out += (i ? "," : "") + u(n.mems[i].offset) + ":" + u(n.mems[i].size);
+        }
+        out += "]";
+        if (n.einsummable) {
+            es::mg_einsummable_t const& e = *n.einsummable;
+            out += " einsummable{" + list(e.join_shape) + ";";
+            for (auto const& inn : e.inns) out += list(inn);
+            out += ";" + std::to_string(e.out_rank) + ";" + e.join + ";" + e.castable + "}";
+        }
+        if (n.touch) {
+            es::touch_t const& t = *n.touch;
+            out += std::string(" touch{") + es::dtype_name(t.dtype) + ";";
+            if (t.castable) out += es::castable_to_char(t.castable);
+            out += ";";
+            for (auto const& d : t.selection) {
+                out += list(std::vector<uint64_t>{d.d_inn, d.d_out, d.offset_inn, d.offset_out,
+                                                  d.size});
+            }
+            out += "}";
+        }
+        if (n.kind == es::mg_kind::constant) {
+            es::mg_fill_t const& f = n.fill;
+            if (f.is_lowertri) {
+                out += " lowertri{" + f.lower + ";" + f.upper + ";" + u(f.nrow) + ";" + u(f.ncol) +
+                       ";" + std::to_string(f.start) + "}";
+            } else {
+                out += " constant{" + f.value + ";" + list(f.shape) + "}";
+            }
+        }
+        out += "\n";
+    }
+    return out;
 }
 
 }  // namespace
@@ -510,6 +565,116 @@ int es_km_graph_node_info(es_km_graph_t* g, int id, int* position, int* stream, 
 int es_km_graph_cross_stream_waits(es_km_graph_t* g)
 {
     return g ? g->graph->n_cross_stream_waits() : ES_KM_ERR_INVALID;
+}
+
+int es_km_graph_add_dummy(es_km_graph_t* g, uint64_t offset, uint64_t size, const int* deps,
+                          int n_deps)
+{
+    return guarded(g ? g->owner : nullptr, [&]() -> int {
+        if (!g) throw es::ir_error("null graph");
+        return g->graph->add_dummy(es::mem_t{offset, size}, make_deps(deps, n_deps));
+    });
+}
+
+int es_km_graph_add_evict(es_km_graph_t* g, uint64_t offset, uint64_t size, int storage_id,
+                          const int* deps, int n_deps)
+{
+    return guarded(g ? g->owner : nullptr, [&]() -> int {
+        if (!g) throw es::ir_error("null graph");
+        return g->graph->add_evict(es::mem_t{offset, size}, storage_id, make_deps(deps, n_deps));
+    });
+}
+
+int es_km_graph_add_load(es_km_graph_t* g, int storage_id, uint64_t offset, uint64_t size,
+                         const int* deps, int n_deps)
+{
+    return guarded(g ? g->owner : nullptr, [&]() -> int {
+        if (!g) throw es::ir_error("null graph");
+        return g->graph->add_load(storage_id, es::mem_t{offset, size}, make_deps(deps, n_deps));
+    });
+}
+
+int es_km_graph_declare_storage(es_km_graph_t* g, int storage_id, uint64_t size)
+{
+    return guarded(g ? g->owner : nullptr, [&]() -> int {
+        if (!g) throw es::ir_error("null graph");
+        g->graph->declare_storage(storage_id, size);
+        return ES_KM_OK;
+    });
+}
+
+int es_km_graph_storage_write(es_km_graph_t* g, int storage_id, const void* src, uint64_t size)
+{
+    return guarded(g ? g->owner : nullptr, [&]() -> int {
+        if (!g) throw es::ir_error("null graph");
+        if (!src && size) throw es::ir_error("storage write: null source");
+        g->graph->storage_write(storage_id, src, size);
+        return ES_KM_OK;
+    });
+}
+
+int es_km_graph_storage_read(es_km_graph_t* g, int storage_id, void* dst, uint64_t size)
+{
+    return guarded(g ? g->owner : nullptr, [&]() -> int {
+        if (!g) throw es::ir_error("null graph");
+        if (!dst && size) throw es::ir_error("storage read: null destination");
+        g->graph->storage_read(storage_id, dst, size);
+        return ES_KM_OK;
+    });
+}
+
+int es_km_graph_load_memgraph(es_km_graph_t* g, const void* bytes, uint64_t size, int loc,
+                              const char* const* var_names, const double* var_values, int n_vars)
+{
+    return guarded(g ? g->owner : nullptr, [&]() -> int {
+        if (!g) throw es::ir_error("null graph");
+        if (n_vars < 0 || (n_vars > 0 && (!var_names || !var_values))) {
+            throw es::ir_error("memgraph: bad scalar variables");
+        }
+        std::vector<std::pair<std::string, double>> vars;
+        for (int i = 0; i != n_vars; ++i) vars.push_back({var_names[i], var_values[i]});
+        es::memgraph_t mg = es::decode_memgraph(bytes, size);
+        mg.populate(*g->graph, loc, vars);
+        return g->graph->n_nodes();
+    });
+}
+
+int es_km_graph_num_nodes(es_km_graph_t* g) { return g ? g->graph->n_nodes() : ES_KM_ERR_INVALID; }
+
+uint64_t es_km_graph_arena_bytes(es_km_graph_t* g) { return g ? g->graph->arena_bytes() : 0; }
+
+int es_km_graph_node_mems(es_km_graph_t* g, int id, int* kind, uint64_t* offsets, uint64_t* sizes,
+                          int cap, int* n_mems)
+{
+    return guarded(g ? g->owner : nullptr, [&]() -> int {
+        if (!g) throw es::ir_error("null graph");
+        if (id < 0 || id >= g->graph->n_nodes()) throw es::ir_error("graph: no such node");
+        if (kind) *kind = g->graph->kind_of(id);
+        std::vector<es::mem_t> const& m = g->graph->mems_of(id);
+        if (n_mems) *n_mems = int(m.size());
+        for (int i = 0; i < cap && i < int(m.size()); ++i) {
+            if (offsets) offsets[i] = m[size_t(i)].offset;
+            if (sizes) sizes[i] = m[size_t(i)].size;
+        }
+        return ES_KM_OK;
+    });
+}
+
+int64_t es_km_memgraph_describe(const void* bytes, uint64_t size, char* out, uint64_t cap)
+{
+    try {
+        es::memgraph_t mg = es::decode_memgraph(bytes, size);
+        std::string    s = describe_memgraph(mg);
+        if (out && cap) {
+            uint64_t const n = std::min<uint64_t>(cap - 1, s.size());
+            std::memcpy(out, s.data(), n);
+            out[n] = 0;
+        }
+        return int64_t(s.size());
+    } catch (std::exception const& e) {
+        g_null_error = e.what();
+        return ES_KM_ERR_INVALID;
+    }
 }
 
 }

@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <cstring>
 
 namespace es
 {
@@ -31,6 +32,9 @@ apply_graph_t::~apply_graph_t()
     for (size_t s = 1; s < streams_.size(); ++s) (void)hipStreamDestroy(streams_[s]);
     for (void* w : workspace_) {
         if (w) (void)hipFree(w);
+    }
+    for (auto& s : slots_) {
+        if (s.second.host) (void)hipHostFree(s.second.host);
     }
     for (hipEvent_t e : events_) (void)hipEventDestroy(e);
     for (hipEvent_t e : joins_) (void)hipEventDestroy(e);
@@ -139,17 +143,109 @@ int apply_graph_t::add_copy(mem_t dst, mem_t src, std::vector<int> const& deps)
     return insert(std::move(n), deps);
 }
 
+int apply_graph_t::add_dummy(mem_t range, std::vector<int> const& deps)
+{
+    node_t n;
+    n.kind = kind_t::dummy;
+    n.mems = {range};
+    return insert(std::move(n), deps);
+}
+
+apply_graph_t::slot_t* apply_graph_t::slot(int storage_id)
+{
+    for (auto& s : slots_) {
+        if (s.first == storage_id) return &s.second;
+    }
+    return nullptr;
+}
+
+apply_graph_t::slot_t const* apply_graph_t::slot(int storage_id) const
+{
+    return const_cast<apply_graph_t*>(this)->slot(storage_id);
+}
+
+void apply_graph_t::declare_storage(int storage_id, uint64_t size)
+{
+    if (finalized_) throw km_error(km_status::invalid, "apply graph: already finalized");
+    if (storage_id < 0) throw km_error(km_status::invalid, "apply graph: negative storage id");
+    slot_t* s = slot(storage_id);
+    if (!s) {
+        slots_.push_back({storage_id, slot_t{}});
+        s = &slots_.back().second;
+    }
+    s->size = std::max(s->size, size);
+}
+
+int apply_graph_t::add_evict(mem_t src, int storage_id, std::vector<int> const& deps)
+{
+    declare_storage(storage_id, src.size);
+    node_t n;
+    n.kind = kind_t::evict;
+    n.storage_id = storage_id;
+    n.mems = {mem_t{0, 0}, src};  // reads the arena, writes none of it
+    return insert(std::move(n), deps);
+}
+
+int apply_graph_t::add_load(int storage_id, mem_t dst, std::vector<int> const& deps)
+{
+    declare_storage(storage_id, dst.size);
+    node_t n;
+    n.kind = kind_t::load;
+    n.storage_id = storage_id;
+    n.mems = {dst};
+    return insert(std::move(n), deps);
+}
+
+void apply_graph_t::storage_write(int storage_id, void const* src, uint64_t size)
+{
+    slot_t* s = slot(storage_id);
+    if (!finalized_ || !s || !s->host) {
+        throw km_error(km_status::invalid, "apply graph: no storage slot " +
+                                               std::to_string(storage_id) +
+                                               " (declared slots exist after finalize)");
+    }
+    if (size > s->size) throw km_error(km_status::invalid, "apply graph: storage slot too small");
+    std::memcpy(s->host, src, size);
+}
+
+void apply_graph_t::storage_read(int storage_id, void* dst, uint64_t size) const
+{
+    slot_t const* s = slot(storage_id);
+    if (!finalized_ || !s || !s->host) {
+        throw km_error(km_status::invalid, "apply graph: no storage slot " +
+                                               std::to_string(storage_id) +
+                                               " (declared slots exist after finalize)");
+    }
+    if (size > s->size) throw km_error(km_status::invalid, "apply graph: storage slot too small");
+    std::memcpy(dst, s->host, size);
+}
+
+uint64_t apply_graph_t::arena_bytes() const
+{
+    uint64_t need = 0;
+    for (node_t const& n : nodes_) {
+        for (mem_t const& m : n.mems) {
+            if (m.size) need = std::max(need, m.offset + m.size);
+        }
+    }
+    return need;
+}
+
 void apply_graph_t::add_memory_dependencies()
 {
     if (finalized_) throw km_error(km_status::invalid, "apply graph: already finalized");
     for (size_t v = 0; v != nodes_.size(); ++v) {
         node_t& nv = nodes_[v];
+        if (nv.kind == kind_t::dummy) continue;
         for (size_t u = 0; u != v; ++u) {
             node_t const& nu = nodes_[u];
+            if (nu.kind == kind_t::dummy) continue;
             bool dep = false;
             // v reads or rewrites what u wrote; v overwrites what u read
             for (mem_t const& m : nv.mems) dep = dep || overlaps(nu.mems[0], m);
             for (size_t k = 1; k < nu.mems.size(); ++k) dep = dep || overlaps(nv.mems[0], nu.mems[k]);
+            // the storage slot is memory too: evict writes it, load reads it
+            if (nu.storage_id >= 0 && nu.storage_id == nv.storage_id) dep = true;
             if (dep) nv.deps.push_back(int(u));
         }
         std::sort(nv.deps.begin(), nv.deps.end());
@@ -241,6 +337,11 @@ void apply_graph_t::finalize(int n_streams)
             if (workspace_bytes_[size_t(s)] == 0) continue;
             check(hipMalloc(&workspace_[size_t(s)], workspace_bytes_[size_t(s)]), "hipMalloc");
         }
+        for (auto& s : slots_) {
+            if (s.second.size == 0) continue;
+            check(hipHostMalloc(&s.second.host, s.second.size, hipHostMallocDefault),
+                  "hipHostMalloc");
+        }
         check(hipEventCreateWithFlags(&fork_, hipEventDisableTiming), "hipEventCreateWithFlags");
         for (int s = 1; s != n_streams; ++s) {
             hipEvent_t e;
@@ -253,6 +354,7 @@ void apply_graph_t::finalize(int n_streams)
 
 void apply_graph_t::launch(node_t const& n, hipStream_t stream, char* arena) const
 {
+    if (n.kind == kind_t::dummy) return;
     void* const out = arena + n.mems[0].offset;
     switch (n.kind) {
         case kind_t::einsummable: {
@@ -284,6 +386,20 @@ void apply_graph_t::launch(node_t const& n, hipStream_t stream, char* arena) con
             check(hipMemcpyAsync(out, arena + n.mems[1].offset, n.mems[0].size,
                                  hipMemcpyDeviceToDevice, stream),
                   "hipMemcpyAsync");
+            break;
+        case kind_t::evict:
+            if (n.mems[1].size == 0) break;
+            check(hipMemcpyAsync(slot(n.storage_id)->host, arena + n.mems[1].offset,
+                                 n.mems[1].size, hipMemcpyDeviceToHost, stream),
+                  "hipMemcpyAsync");
+            break;
+        case kind_t::load:
+            if (n.mems[0].size == 0) break;
+            check(hipMemcpyAsync(out, slot(n.storage_id)->host, n.mems[0].size,
+                                 hipMemcpyHostToDevice, stream),
+                  "hipMemcpyAsync");
+            break;
+        case kind_t::dummy:
             break;
     }
 }

@@ -1,9 +1,10 @@
 // The exec-node layer over the kernel manager: a dependency graph of apply (einsummable /
-// touch) and fill nodes addressed by offsets into one device arena, run on one GPU.
+// touch), fill, copy, evict / load and dummy nodes addressed by offsets into one device
+// arena, run on one GPU.
 //
 // It plays the part of the reference's GPU exec graph for these node kinds
 // (src/engine/exec_graph.h:17-80; gpu_einsummable_t, gpu_touch_t, gpu_constant_t,
-// gpu_lowerTri_t, gpu_copy_t in src/engine/gpu/exec_nodes.h and
+// gpu_lowerTri_t, gpu_copy_t, gpu_evict_t, gpu_load_t, dummy_t in src/engine/gpu/exec_nodes.h and
 // src/engine/gpu/exec_graph.cc:258-404, 600-690).  The reference drives its graph from a host
 // event loop: every node takes a stream from a pool, launches, and reports back through
 // cudaStreamAddCallback, after which the loop releases the node's dependents
@@ -24,6 +25,7 @@
 
 #include <cstdint>
 #include <string>
+#include <utility>
 #include <vector>
 
 namespace es
@@ -54,6 +56,23 @@ public:
     int add_lowertri_fill(dtype_t dtype, uint64_t lower_bits, uint64_t upper_bits, uint64_t nrow,
                           uint64_t ncol, int64_t start, mem_t out, std::vector<int> const& deps);
     int add_copy(mem_t dst, mem_t src, std::vector<int> const& deps);
+    // A node that launches nothing and only carries dependencies: what the reference makes
+    // of inputmem / inputsto / partialize / alloc / del nodes and of nodes that live on
+    // another device (gpu/exec_graph.cc:94-97).  `range` is kept for inspection only and
+    // takes no part in add_memory_dependencies.
+    int add_dummy(mem_t range, std::vector<int> const& deps);
+    // Host storage (gpu_evict_t / gpu_load_t, gpu/exec_graph.cc:466-577; the reference's
+    // storage is host memory too, src/engine/gpu/storage_manager.h).  evict copies an arena
+    // range into the storage slot `storage_id`, load copies the slot back.  Slots are pinned
+    // host buffers allocated at finalize, one per id, sized for the largest user; the
+    // copies are asynchronous on the node's stream like every other node.
+    int add_evict(mem_t src, int storage_id, std::vector<int> const& deps);
+    int add_load(int storage_id, mem_t dst, std::vector<int> const& deps);
+    // declares a slot that the caller fills before run (an inputsto node)
+    void declare_storage(int storage_id, uint64_t size);
+    // after finalize: host-side access to a slot (the caller orders these against run)
+    void storage_write(int storage_id, void const* src, uint64_t size);
+    void storage_read(int storage_id, void* dst, uint64_t size) const;
 
     // Adds, between every pair of nodes in insertion order, the dependency their memory
     // ranges imply (read after write, write after write, write after read).
@@ -68,6 +87,12 @@ public:
     void run(hipStream_t main, void* arena) const;
 
     int n_nodes() const { return int(nodes_.size()); }
+    // smallest arena that holds every range a node touches
+    uint64_t arena_bytes() const;
+    // 0 einsummable, 1 touch, 2 constant fill, 3 lowertri fill, 4 copy, 5 dummy, 6 evict,
+    // 7 load
+    int                       kind_of(int id) const { return int(nodes_[id].kind); }
+    std::vector<mem_t> const& mems_of(int id) const { return nodes_[id].mems; }
     // after finalize: launch position, stream and dependencies (own + implied) of a node
     int                     position_of(int id) const { return nodes_[id].position; }
     int                     stream_of(int id) const { return nodes_[id].stream; }
@@ -76,7 +101,7 @@ public:
     int n_cross_stream_waits() const { return n_waits_; }
 
 private:
-    enum class kind_t { einsummable, touch, constant, lowertri, copy };
+    enum class kind_t { einsummable, touch, constant, lowertri, copy, dummy, evict, load };
     struct node_t {
         kind_t             kind;
         einsummable_t      e;
@@ -85,6 +110,7 @@ private:
         dtype_t            dtype = dtype_t::f32;
         uint64_t           bits0 = 0, bits1 = 0, n0 = 0, n1 = 0;
         int64_t            start = 0;
+        int                storage_id = -1;
         std::vector<mem_t> mems;
         std::vector<int>   deps;
         std::vector<int>   waits;  // dependencies on other streams, reduced
@@ -107,6 +133,13 @@ private:
     // from a pool per launch (src/engine/gpu/workspace.cc:48-91)
     std::vector<void*>       workspace_;
     std::vector<uint64_t>    workspace_bytes_;
+    struct slot_t {
+        uint64_t size = 0;
+        void*    host = nullptr;  // pinned
+    };
+    std::vector<std::pair<int, slot_t>> slots_;  // by storage id
+    slot_t*       slot(int storage_id);
+    slot_t const* slot(int storage_id) const;
     hipEvent_t               fork_ = nullptr;
     std::vector<hipEvent_t>  joins_;
     int                      n_waits_ = 0;

@@ -417,6 +417,73 @@ std::string scalarop_t::str() const
 
 bool scalarop_t::has_variables() const { return node_has_variable(root); }
 
+namespace
+{
+void replace_in(node_t& n, std::vector<std::pair<std::string, double>> const& values)
+{
+    if (n.kind == op_kind::variable) {
+        for (auto const& nv : values) {
+            if (nv.first != n.name) continue;
+            if (n.dtype == dtype_t::c64) throw ir_error("replace_variables: complex variable");
+            n.kind = op_kind::constant;
+            n.re = round_to_dtype(n.dtype, nv.second);
+            n.im = 0.0;
+            n.name.clear();
+            break;
+        }
+    }
+    for (node_t& c : n.children) replace_in(c, values);
+}
+}  // namespace
+
+scalarop_t scalarop_t::replace_variables(
+    std::vector<std::pair<std::string, double>> const& values) const
+{
+    scalarop_t ret = *this;
+    replace_in(ret.root, values);
+    return ret;
+}
+
+scalar_bits_t parse_scalar(std::string const& text)
+{
+    scalarop_t op = scalarop_t::parse("constant{" + text + "}");
+    node_t const& n = op.root;
+    scalar_bits_t ret{n.dtype, 0};
+    switch (n.dtype) {
+        case dtype_t::f16: {
+            _Float16 v = _Float16(n.re);
+            uint16_t b;
+            std::memcpy(&b, &v, 2);
+            ret.bits = b;
+            break;
+        }
+        case dtype_t::f32: {
+            float    v = float(n.re);
+            uint32_t b;
+            std::memcpy(&b, &v, 4);
+            ret.bits = b;
+            break;
+        }
+        case dtype_t::f64:
+            std::memcpy(&ret.bits, &n.re, 8);
+            break;
+        case dtype_t::c64: {
+            float    v[2] = {float(n.re), float(n.im)};
+            std::memcpy(&ret.bits, v, 8);
+            break;
+        }
+    }
+    return ret;
+}
+
+std::optional<dtype_t> dtype_from_name(std::string const& name)
+{
+    for (dtype_t d : {dtype_t::f16, dtype_t::f32, dtype_t::f64, dtype_t::c64}) {
+        if (name == dtype_name(d)) return d;
+    }
+    return std::nullopt;
+}
+
 bool scalarop_t::is_identity() const { return is_hole(root, 0); }
 
 bool scalarop_t::is_mul() const

@@ -9,6 +9,7 @@
 #include <optional>
 #include <stdexcept>
 #include <string>
+#include <utility>
 #include <vector>
 
 namespace es
@@ -23,6 +24,15 @@ const char* dtype_name(dtype_t);
 // '+' 'x' 'v' '^' (scalarop.cc:3078-3093); 0 means "no castable"
 std::optional<castable_t> castable_from_char(char c);
 char                      castable_to_char(std::optional<castable_t> const&);
+
+// A scalar in the reference's text form, "f32|1.5", "f16|NINF", "c64|(1,2)"
+// (scalarop.cc:2720-2830): its dtype and its bytes in the low bytes of a uint64.
+struct scalar_bits_t {
+    dtype_t  dtype;
+    uint64_t bits;
+};
+scalar_bits_t parse_scalar(std::string const& text);
+std::optional<dtype_t> dtype_from_name(std::string const& name);
 
 struct ir_error : std::runtime_error {
     using std::runtime_error::runtime_error;
@@ -67,6 +77,11 @@ struct scalarop_t {
     //   *[hole|f16@0,power{-1}[+[constant{f16|1},exp[*[constant{f16|-1},hole|f16@0]]]]]
     // (grammar: scalarop.cc:2881-3011).  Throws ir_error on malformed or ill-typed text.
     static scalarop_t parse(std::string const& text);
+
+    // Every variable named in `values` becomes a constant of the variable's dtype
+    // (scalarop_t::replace_variables, scalarop.cc; einsummable_t::replace_scalar_variables,
+    // einsummable.cc:221-233).  Variables not named stay.
+    scalarop_t replace_variables(std::vector<std::pair<std::string, double>> const& values) const;
 
     std::string str() const;
     dtype_t     out_dtype() const { return root.dtype; }

@@ -37,6 +37,17 @@ EXPORTS = [
     "es_km_graph_run",
     "es_km_graph_node_info",
     "es_km_graph_cross_stream_waits",
+    "es_km_graph_add_dummy",
+    "es_km_graph_add_evict",
+    "es_km_graph_add_load",
+    "es_km_graph_declare_storage",
+    "es_km_graph_storage_write",
+    "es_km_graph_storage_read",
+    "es_km_graph_load_memgraph",
+    "es_km_graph_num_nodes",
+    "es_km_graph_arena_bytes",
+    "es_km_graph_node_mems",
+    "es_km_memgraph_describe",
 ]
 
 
@@ -154,6 +165,19 @@ def load_library():
     lib.es_km_graph_run.argtypes = [V, V, V]
     lib.es_km_graph_node_info.argtypes = [V, I, V, V, V, I, V]
     lib.es_km_graph_cross_stream_waits.argtypes = [V]
+    lib.es_km_graph_add_dummy.argtypes = [V, U64, U64, V, I]
+    lib.es_km_graph_add_evict.argtypes = [V, U64, U64, I, V, I]
+    lib.es_km_graph_add_load.argtypes = [V, I, U64, U64, V, I]
+    lib.es_km_graph_declare_storage.argtypes = [V, I, U64]
+    lib.es_km_graph_storage_write.argtypes = [V, I, V, U64]
+    lib.es_km_graph_storage_read.argtypes = [V, I, V, U64]
+    lib.es_km_graph_load_memgraph.argtypes = [V, V, U64, I, V, V, I]
+    lib.es_km_graph_num_nodes.argtypes = [V]
+    lib.es_km_graph_arena_bytes.argtypes = [V]
+    lib.es_km_graph_arena_bytes.restype = U64
+    lib.es_km_graph_node_mems.argtypes = [V, I, V, V, V, I, V]
+    lib.es_km_memgraph_describe.argtypes = [V, U64, V, U64]
+    lib.es_km_memgraph_describe.restype = ctypes.c_int64
     _lib = lib
     return lib
 
@@ -462,3 +486,72 @@ class ApplyGraph:
 
     def cross_stream_waits(self):
         return self._check(self._lib.es_km_graph_cross_stream_waits(self._g))
+
+    def add_dummy(self, mem=(0, 0), deps=None):
+        d, nd = self._deps(deps)
+        return self._check(self._lib.es_km_graph_add_dummy(self._g, int(mem[0]), int(mem[1]),
+                                                           d, nd))
+
+    def add_evict(self, mem, storage_id, deps=None):
+        d, nd = self._deps(deps)
+        return self._check(self._lib.es_km_graph_add_evict(self._g, int(mem[0]), int(mem[1]),
+                                                           int(storage_id), d, nd))
+
+    def add_load(self, storage_id, mem, deps=None):
+        d, nd = self._deps(deps)
+        return self._check(self._lib.es_km_graph_add_load(self._g, int(storage_id), int(mem[0]),
+                                                          int(mem[1]), d, nd))
+
+    def declare_storage(self, storage_id, size):
+        self._check(self._lib.es_km_graph_declare_storage(self._g, int(storage_id), int(size)))
+
+    def storage_write(self, storage_id, data):
+        """data: bytes-like, copied into the slot (after finalize)."""
+        data = bytes(data)
+        self._check(self._lib.es_km_graph_storage_write(self._g, int(storage_id), data,
+                                                        len(data)))
+
+    def storage_read(self, storage_id, size):
+        buf = ctypes.create_string_buffer(int(size))
+        self._check(self._lib.es_km_graph_storage_read(self._g, int(storage_id), buf, int(size)))
+        return buf.raw
+
+    def load_memgraph(self, wire, loc=0, scalar_vars=None):
+        """Append every node of a serialized MemGraph (the reference's memgraph_t::to_wire
+        bytes) for compute location `loc`; node ids equal the memgraph's."""
+        wire = bytes(wire)
+        items = sorted((scalar_vars or {}).items())
+        names = (ctypes.c_char_p * max(len(items), 1))(*[k.encode() for k, _ in items])
+        vals = (ctypes.c_double * max(len(items), 1))(*[float(v) for _, v in items])
+        return self._check(self._lib.es_km_graph_load_memgraph(
+            self._g, wire, len(wire), int(loc), names, vals, len(items)))
+
+    def num_nodes(self):
+        return self._check(self._lib.es_km_graph_num_nodes(self._g))
+
+    def arena_bytes(self):
+        return int(self._lib.es_km_graph_arena_bytes(self._g))
+
+    NODE_KINDS = ("einsummable", "touch", "constant", "lowertri", "copy", "dummy", "evict",
+                  "load")
+
+    def node_mems(self, node):
+        """(kind name, [(offset, size)]) of a node."""
+        kind, n = ctypes.c_int(-1), ctypes.c_int(0)
+        offs, sizes = (ctypes.c_uint64 * 64)(), (ctypes.c_uint64 * 64)()
+        self._check(self._lib.es_km_graph_node_mems(self._g, node, ctypes.byref(kind), offs,
+                                                    sizes, 64, ctypes.byref(n)))
+        k = min(n.value, 64)
+        return self.NODE_KINDS[kind.value], [(offs[i], sizes[i]) for i in range(k)]
+
+
+def memgraph_describe(wire):
+    """One line per node of a serialized MemGraph, every decoded field in a fixed order."""
+    lib = load_library()
+    wire = bytes(wire)
+    n = lib.es_km_memgraph_describe(wire, len(wire), None, 0)
+    if n < 0:
+        raise KmError(int(n), lib.es_km_last_error(None).decode())
+    buf = ctypes.create_string_buffer(int(n) + 1)
+    lib.es_km_memgraph_describe(wire, len(wire), buf, int(n) + 1)
+    return buf.value.decode()

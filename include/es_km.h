@@ -212,6 +212,58 @@ int es_km_graph_node_info(es_km_graph_t* g, int id, int* position, int* stream, 
                           int* n_deps);
 int es_km_graph_cross_stream_waits(es_km_graph_t* g);
 
+/* Nodes that launch nothing and only carry dependencies (dummy_t, which the reference makes
+ * of inputmem / inputsto / partialize / alloc / del nodes, src/engine/gpu/exec_graph.cc:94-97).
+ * The range is kept for inspection and takes no part in add_memory_dependencies. */
+int es_km_graph_add_dummy(es_km_graph_t* g, uint64_t offset, uint64_t size, const int* deps,
+                          int n_deps);
+
+/* Host storage: gpu_evict_t::launch / gpu_load_t::launch, src/engine/gpu/exec_graph.cc:482-577
+ * (memgraph_t::evict_t / load_t, src/einsummable/memgraph.h:306-325).  evict copies an arena
+ * range to the storage slot `storage_id`, load copies the slot to an arena range; both are
+ * asynchronous copies on the node's stream.  A slot is a pinned host buffer the graph
+ * allocates at finalize, sized for its largest user (the reference allocates one per evict
+ * and frees it after the load, storage_manager.h).  declare_storage announces a slot the
+ * caller fills itself (an inputsto node, memgraph.h:222-228); storage_write / storage_read
+ * are host copies, valid after finalize, which the caller orders against run. */
+int es_km_graph_add_evict(es_km_graph_t* g, uint64_t offset, uint64_t size, int storage_id,
+                          const int* deps, int n_deps);
+int es_km_graph_add_load(es_km_graph_t* g, int storage_id, uint64_t offset, uint64_t size,
+                         const int* deps, int n_deps);
+int es_km_graph_declare_storage(es_km_graph_t* g, int storage_id, uint64_t size);
+int es_km_graph_storage_write(es_km_graph_t* g, int storage_id, const void* src, uint64_t size);
+int es_km_graph_storage_read(es_km_graph_t* g, int storage_id, void* dst, uint64_t size);
+
+/* memgraph_t::from_wire (src/einsummable/memgraph.cc:381-480) followed by what
+ * exec_graph_t::make_gpu_exec_graph does with the result (src/engine/gpu/exec_graph.cc:26-245):
+ * `bytes` is a serialized MemGraph message (src/proto/einsummable.proto:233-238, as written by
+ * memgraph_t::to_wire, memgraph.cc:258-379); every node of it becomes one node of the empty
+ * graph `g`, with the same id, for compute location `loc`:
+ *   inputmem, inputsto, partialize, alloc, del, nodes of other locations -> dummy
+ *   apply -> einsummable (scalar variables named in var_names replaced by var_values first,
+ *            exec_graph.cc:108-110) or touch with its group
+ *   constant -> constant / lowertri fill;  copy, move within `loc` -> copy
+ *   evict, load -> host storage;  inputsto read here -> declared storage slot
+ * A move between two locations is an error (one process drives one device).  A lowertri
+ * fill has nrow and ncol exchanged, as the reference's reader leaves them
+ * (src/einsummable/fill.cc:137-143).  Returns the number of nodes or a negative error;
+ * finalize and run the graph as usual. */
+int es_km_graph_load_memgraph(es_km_graph_t* g, const void* bytes, uint64_t size, int loc,
+                              const char* const* var_names, const double* var_values, int n_vars);
+
+/* Inspection: node count, the smallest arena holding every range, and a node's kind
+ * (0 einsummable, 1 touch, 2 constant fill, 3 lowertri fill, 4 copy, 5 dummy, 6 evict,
+ * 7 load) and ranges (for a dummy made of an inputmem: where the caller puts that input). */
+int      es_km_graph_num_nodes(es_km_graph_t* g);
+uint64_t es_km_graph_arena_bytes(es_km_graph_t* g);
+int es_km_graph_node_mems(es_km_graph_t* g, int id, int* kind, uint64_t* offsets, uint64_t* sizes,
+                          int cap, int* n_mems);
+
+/* Diagnostics without a device: decodes a serialized MemGraph and writes one line per node
+ * with every decoded field into `out` (at most cap bytes, NUL-terminated).  Returns the
+ * full length of the text or a negative error (message via es_km_last_error(NULL)). */
+int64_t es_km_memgraph_describe(const void* bytes, uint64_t size, char* out, uint64_t cap);
+
 #ifdef __cplusplus
 }
 #endif

@@ -20,6 +20,7 @@
 
 #include <complex>
 #include <cstring>
+#include <map>
 #include <optional>
 #include <stdexcept>
 #include <string>
@@ -280,6 +281,46 @@ public:
         return id(es_km_graph_add_copy(g_, dst.offset, src.offset, dst.size, inns.data(),
                                        int(inns.size())));
     }
+    // dummy_t: launches nothing, only orders (inputmem / partialize / alloc / del nodes)
+    int insert_dummy(mem_t range = {0, 0}, std::vector<int> const& inns = {})
+    {
+        return id(es_km_graph_add_dummy(g_, range.offset, range.size, inns.data(),
+                                        int(inns.size())));
+    }
+    // gpu_evict_t / gpu_load_t: arena range <-> host storage slot
+    int insert_evict(mem_t src, int storage_id, std::vector<int> const& inns = {})
+    {
+        return id(es_km_graph_add_evict(g_, src.offset, src.size, storage_id, inns.data(),
+                                        int(inns.size())));
+    }
+    int insert_load(int storage_id, mem_t dst, std::vector<int> const& inns = {})
+    {
+        return id(es_km_graph_add_load(g_, storage_id, dst.offset, dst.size, inns.data(),
+                                       int(inns.size())));
+    }
+    void storage_write(int storage_id, void const* src, uint64_t size)
+    {
+        check(es_km_graph_storage_write(g_, storage_id, src, size));
+    }
+    void storage_read(int storage_id, void* dst, uint64_t size) const
+    {
+        check(es_km_graph_storage_read(g_, storage_id, dst, size));
+    }
+    // memgraph_t::from_wire + make_gpu_exec_graph for compute location `loc`: every node of
+    // the serialized memgraph becomes the node of the same id (the graph must be empty)
+    int load_memgraph(std::string const& wire, int loc = 0,
+                      std::map<std::string, double> const& scalar_vars = {})
+    {
+        std::vector<char const*> names;
+        std::vector<double>      values;
+        for (auto const& kv : scalar_vars) {
+            names.push_back(kv.first.c_str());
+            values.push_back(kv.second);
+        }
+        return id(es_km_graph_load_memgraph(g_, wire.data(), wire.size(), loc, names.data(),
+                                            values.data(), int(names.size())));
+    }
+    uint64_t arena_bytes() const { return es_km_graph_arena_bytes(g_); }
     void add_memory_dependencies() { check(es_km_graph_add_memory_dependencies(g_)); }
     void finalize(int n_streams) { check(es_km_graph_finalize(g_, n_streams)); }
     // the whole graph, ordered after and before `stream`; no host synchronisation

@@ -219,6 +219,54 @@ int main()
         expect(ok, "exec graph: dependent nodes and a touch group on two streams");
     }
 
+    {  // host storage (gpu_evict_t / gpu_load_t) and a serialized memgraph
+       // (memgraph_t::from_wire): inputmem, alloc, relu as an apply node, evict, load
+        uint64_t const n = 1024, B = n * 4;
+        auto x = random_f32(gen, n, -1, 1);
+        device_buffer_t arena(3 * B);
+        std::vector<float> host(3 * n, 5.0f), got(3 * n), slot(n);
+        std::copy(x.begin(), x.end(), host.begin());
+        arena.upload(host.data());
+        auto varint = [](uint64_t v) {
+            std::string o;
+            do {
+                o.push_back(char((v & 0x7f) | (v > 0x7f ? 0x80 : 0)));
+                v >>= 7;
+            } while (v);
+            return o;
+        };
+        auto scalar = [&](int f, uint64_t v) { return varint(uint64_t(f) << 3) + varint(v); };
+        auto bytes = [&](int f, std::string const& b) {
+            return varint(uint64_t(f) << 3 | 2) + varint(b.size()) + b;
+        };
+        auto los = [&](uint64_t off) { return scalar(1, 0) + scalar(2, off) + scalar(3, B); };
+        std::string const relu = "ite_>=[constant{f32|0},hole|f32@0,constant{f32|0},hole|f32@0]";
+        std::string es = scalar(1, n) + bytes(2, scalar(1, 0)) + scalar(3, 1) + bytes(4, relu);
+        std::string apply = scalar(1, 0) + scalar(2, B) + scalar(2, 0) + scalar(3, B) +
+                            scalar(3, B) + bytes(4, es) + scalar(6, uint64_t(-1));
+        std::string sto = scalar(1, 0) + scalar(2, 9) + scalar(3, 0);
+        std::string wire = scalar(1, 1) + scalar(2, 1) +
+                           bytes(4, bytes(1, los(0))) +                                   // 0
+                           bytes(4, bytes(9, los(B))) +                                   // 1
+                           bytes(4, bytes(4, apply) + scalar(11, 0) + scalar(11, 1)) +    // 2
+                           bytes(4, bytes(6, sto + scalar(4, B) + scalar(5, B)) + scalar(11, 2)) +
+                           bytes(4, bytes(7, sto + scalar(4, 2 * B) + scalar(5, B)) + scalar(11, 3));
+        exec_graph_t g(km);
+        expect(g.load_memgraph(wire) == 5, "memgraph: five nodes");
+        expect(g.arena_bytes() == 3 * B, "memgraph: arena size");
+        g.finalize(2);
+        g.run(stream, arena.ptr);
+        HIP_OK(hipStreamSynchronize(stream));
+        arena.download(got.data());
+        g.storage_read(9, slot.data(), B);
+        bool ok = true;
+        for (uint64_t i = 0; i != n; ++i) {
+            float r = std::max(x[i], 0.0f);
+            ok = ok && got[n + i] == r && got[2 * n + i] == r && slot[i] == r;
+        }
+        expect(ok, "memgraph from wire: apply, evict to host storage, load back");
+    }
+
     HIP_OK(hipStreamDestroy(stream));
     std::printf("PASS\n");
     return 0;
