@@ -306,10 +306,18 @@ std::shared_ptr<plan_t> plan_contraction(einsummable_t const& e, int)
     // kernel sums their fp32 partial tiles, which live in the workspace.
     a.splits = 1;
     p->workspace_bytes = 0;
+    a.lin = a.gm.n == 1 && a.gn.n == 1 && a.gk.n == 1 && a.gn.sy[0] == 1 && a.gm.sy[0] > 0 &&
+            uint64_t(a.gm.sy[0]) * 256 * dtype_size(dt) < (1ull << 31);
+    {
+        uint64_t const in_group = 4ull * a.tiles_n;
+        uint64_t const n_tiles = uint64_t(a.tiles_m) * a.tiles_n;
+        a.group_magic = n_tiles * in_group < (1ull << 32) ? uint32_t((1ull << 32) / in_group) + 1
+                                                          : 0;
+    }
     uint64_t const tiles = uint64_t(a.tiles_m) * a.tiles_n * Bt;
     uint64_t const nk = K * dtype_size(dt) / 64;
-    if (p->planned_dma && tiles <= 128 && nk >= 16) {
-        uint64_t S = std::min<uint64_t>({256 / tiles, nk / 8, 64});
+    if (p->planned_dma && nk >= 16) {
+        uint64_t S = tiles <= 128 ? std::min<uint64_t>({256 / tiles, nk / 8, 64}) : 1;
         if (const char* env = std::getenv("ES_KM_GEMM_SPLITS")) {  // tuning and tests
             S = std::min<uint64_t>(uint64_t(std::max(1, std::atoi(env))), nk / 4);
         }
@@ -317,6 +325,12 @@ std::shared_ptr<plan_t> plan_contraction(einsummable_t const& e, int)
             a.splits = uint32_t(S);
             p->workspace_bytes = S * Bt * M * N * 4;
         }
+    }
+    a.shortk = 0;
+    if (dt == dtype_t::f16 && p->planned_dma && p->bm == 128 && p->bn == 128 &&
+        gemm::gemm_shortk_eligible(a)) {
+        const char* env = std::getenv("ES_KM_GEMM_RESIDENT_A");  // tuning and tests
+        a.shortk = !(env && env[0] == '0');
     }
     static const char* mode_name[] = {"k", "mn", "elem"};
     p->description = std::string("contraction_mfma_") + dtype_name(dt) + " tile=" +
@@ -326,7 +340,8 @@ std::shared_ptr<plan_t> plan_contraction(einsummable_t const& e, int)
                      (swapped ? " swapped" : "") + (dma ? " load=direct_to_lds" : "") +
                      " M=" + std::to_string(M) + " N=" + std::to_string(N) + " K=" +
                      std::to_string(K) + " batch=" + std::to_string(Bt) +
-                     (a.splits > 1 ? " split_k=" + std::to_string(a.splits) : "");
+                     (a.splits > 1 ? " split_k=" + std::to_string(a.splits) : "") +
+                     (a.shortk ? " resident_a" : "");
     return p;
 }
 

@@ -93,22 +93,36 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
     }
     constexpr uint32_t GROUP_M = 4;
     uint32_t const     in_group = GROUP_M * a.tiles_n;
-    uint32_t const     first_m = (tile / in_group) * GROUP_M;
-    uint32_t const     rows = (a.tiles_m - first_m) < GROUP_M ? (a.tiles_m - first_m) : GROUP_M;
-    uint32_t const     tm = first_m + (tile % in_group) % rows;
-    uint32_t const     tn = (tile % in_group) / rows;
-    uint32_t const     bz = blockIdx.y;
+    // all of this is uniform: a multiply-high and shifts stay on the scalar unit, while a
+    // division is a long vector sequence that every workgroup would pay before its first load
+    uint32_t const group = a.group_magic ? __umulhi(tile, a.group_magic) : tile / in_group;
+    uint32_t const in_g = tile - group * in_group;
+    uint32_t const first_m = group * GROUP_M;
+    uint32_t const rows = (a.tiles_m - first_m) < GROUP_M ? (a.tiles_m - first_m) : GROUP_M;
+    uint32_t       tm, tn;
+    if (rows == GROUP_M) {
+        tm = first_m + in_g % GROUP_M;
+        tn = in_g / GROUP_M;
+    } else {
+        tm = first_m + in_g % rows;
+        tn = in_g / rows;
+    }
+    uint32_t const bz = blockIdx.y;
 
     int64_t boa, bob, boc;
     {
         group_offsets(a.gb, bz, boa, bob);
-        boc = 0;
-        uint32_t i = bz;
+        if (a.gb.n == 1) {
+            boc = int64_t(bz) * a.gb.sz[0];
+        } else {
+            boc = 0;
+            uint32_t i = bz;
 #pragma unroll
-        for (int d = 0; d != MAXG; ++d) {
-            uint32_t q = i / a.gb.size[d];
-            boc += int64_t(i - q * a.gb.size[d]) * a.gb.sz[d];
-            i = q;
+            for (int d = 0; d != MAXG; ++d) {
+                uint32_t q = i / a.gb.size[d];
+                boc += int64_t(i - q * a.gb.size[d]) * a.gb.sz[d];
+                i = q;
+            }
         }
     }
     // the bases go into scalar registers of the load instructions
@@ -457,7 +471,7 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
                 group_offsets(a.gn, n, no_b, no_c);
                 chunk_t* const dst = reinterpret_cast<chunk_t*>(C + mo_c + no_c);
                 if (a.c_stream) {
-                    __builtin_nontemporal_store(v, dst);
+                    store_16_streaming(dst, v);
                 } else {
                     *dst = v;
                 }

@@ -1,6 +1,7 @@
 // fp16-in / fp32-accumulate instantiations of the MFMA GEMM kernel.
 #include "gemm_dma_kernel.h"
 #include "gemm_kernel.h"
+#include "gemm_shortk_kernel.h"
 
 namespace es
 {
@@ -14,6 +15,7 @@ void launch_gemm_f16(int bm, int bn, gemm_args_t const& a, hipStream_t stream)
     using T = _Float16;
     if (a.tiles_m == 0) return;
     if (gemm_dma_eligible<T>(a)) {
+        if (a.shortk && gemm_shortk_eligible(a)) return launch_gemm_shortk(a, stream);
         if (bm == 256 && bn == 256) return launch_gemm_dma_kernel<T, 256, 256, 4>(a, stream);
         if (bm == 256 && bn == 128) return launch_gemm_dma_kernel<T, 256, 128, 4>(a, stream);
         if (bm == 128 && bn == 256) return launch_gemm_dma_kernel<T, 128, 256, 4>(a, stream);

@@ -43,6 +43,14 @@ struct gemm_args_t {
     // ([split][batch][M][N]); gemm_fold_kernel sums them into C.
     uint32_t    splits;
     float*      ws;
+    // m, n and k are single modes, C is contiguous along n and 256 rows of C span less than
+    // 2^31 bytes: every in-tile offset is a 32-bit multiple of a stride
+    int         lin;
+    // planned for the kernel that keeps A in registers and walks along n (K = 128, fp16)
+    int         shortk;
+    // floor(2^32 / (4 * tiles_n)) + 1 when tile index * 4 * tiles_n < 2^32 (then the high
+    // half of tile * magic is the exact quotient), else 0
+    uint32_t    group_magic;
 };
 
 __device__ __forceinline__ void group_offsets(group_t const& g, uint32_t i, int64_t& ox,
@@ -73,6 +81,16 @@ typedef double   double2_t __attribute__((ext_vector_type(2)));
 
 // 16 bytes of an operand row; a native vector so that it lives in registers
 typedef uint32_t chunk_t __attribute__((ext_vector_type(4)));
+
+// A 16-byte store that does not allocate in the caches (a C larger than the caches would
+// otherwise evict the operand tiles the other workgroups are re-reading).  Written as an
+// instruction: with __builtin_nontemporal_store in one arm of a branch and a plain store of
+// the same value to the same address in the other, the optimiser merges the two into one
+// plain store and the hint is silently lost.
+__device__ __forceinline__ void store_16_streaming(void* dst, chunk_t const& v)
+{
+    asm volatile("global_store_dwordx4 %0, %1, off nt\n\ts_nop 1" : : "v"(dst), "v"(v) : "memory");
+}
 
 template <typename T>
 struct elems_of;
@@ -855,11 +873,16 @@ void launch_gemm_f64(int bm, int bn, gemm_args_t const& a, hipStream_t stream);
 double probe_mfma_f16(void const* operands, void* scratch, int blocks, int iters,
                       hipStream_t stream);
 
+// The fp16 kernel for reductions of exactly 128 elements (gemm_shortk_kernel.h)
+bool gemm_shortk_eligible(gemm_args_t const& a);
+void launch_gemm_shortk(gemm_args_t const& a, hipStream_t stream);
+
 // the same problem cut into bm x bn tiles
 inline gemm_args_t with_tile(gemm_args_t a, int bm, int bn)
 {
     a.tiles_m = (a.M + uint32_t(bm) - 1) / uint32_t(bm);
     a.tiles_n = (a.N + uint32_t(bn) - 1) / uint32_t(bn);
+    a.group_magic = 0;  // belongs to the tile counts it was computed for
     return a;
 }
 

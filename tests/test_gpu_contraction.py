@@ -238,3 +238,48 @@ def test_split_k_is_deterministic_and_checks_its_workspace(km):
     with pytest.raises(ea.KmError) as ei:
         km(e, stream_handle(), d.data_ptr(), [d.data_ptr(), d.data_ptr()])
     assert ei.value.code == -3
+
+
+RESIDENT_A_CASES = [
+    # reductions of exactly 128 fp16 elements over at least 2048 tiles: the lhs rows stay in
+    # registers and a workgroup walks along n.  Full tiles, ragged m and n, a batch of two
+    # modes with strides (heads stored between sequence and head dimension), more than 16
+    # tiles along n (two walks per row of tiles)
+    ("bid,bjd->bij", dict(b=32, i=1024, j=1024, d=128)),
+    ("bid,bjd->bij", dict(b=37, i=1000, j=1016, d=128)),
+    ("bihd,bjhd->bhij", dict(b=2, h=16, i=1024, j=1024, d=128)),
+    ("bid,bjd->bij", dict(b=7, i=1024, j=5000, d=128)),
+]
+
+
+@pytest.mark.parametrize("case", range(len(RESIDENT_A_CASES)))
+def test_resident_lhs_kernel_for_head_dimension_reductions(km, monkeypatch, case):
+    spec, sizes = RESIDENT_A_CASES[case]
+    e = contraction(spec, sizes, "f16")
+    km.build(e)
+    assert "resident_a" in km.describe(e), km.describe(e)
+    monkeypatch.setenv("ES_KM_GEMM_RESIDENT_A", "0")
+    per_tile = ea.KernelManager(0)
+    per_tile.build(e)
+    assert "resident_a" not in per_tile.describe(e)
+    r = rng(60 + case)
+    xs = [normal(r, int(np.prod(e.inn_shape(k))), np.float16) for k in range(2)]
+    a = run_einsummable(km, e, xs)
+    b = run_einsummable(per_tile, e, xs)
+    # both kernels add the same eight 16-wide products per output in the same order
+    np.testing.assert_array_equal(a.view(np.uint16), b.view(np.uint16))
+    # and a slice of it against the oracle (the whole product is billions of flops)
+    lhs_shape, rhs_shape = e.inn_shape(0), e.inn_shape(1)
+    if spec.startswith("bid"):
+        L = xs[0].reshape(lhs_shape)[-1:, -136:, :]
+        R = xs[1].reshape(rhs_shape)[-1:, -264:, :]
+        sub = contraction(spec, dict(b=1, i=136, j=264, d=128), "f16")
+        got = a.reshape(sizes["b"], sizes["i"], sizes["j"])[-1:, -136:, -264:]
+    else:
+        L = xs[0].reshape(lhs_shape)[-1:, -136:, -1:, :]
+        R = xs[1].reshape(rhs_shape)[-1:, -264:, -1:, :]
+        sub = contraction(spec, dict(b=1, h=1, i=136, j=264, d=128), "f16")
+        got = a.reshape(sizes["b"], sizes["h"], sizes["i"], sizes["j"])[-1:, -1:, -136:, -264:]
+    want = oracle_einsummable(sub, [np.ascontiguousarray(L).reshape(-1),
+                                    np.ascontiguousarray(R).reshape(-1)], oracle.WIDE)
+    assert_close(np.ascontiguousarray(got).reshape(-1), want, DT["f16"], what=spec)
