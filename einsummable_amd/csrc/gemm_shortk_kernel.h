@@ -36,6 +36,7 @@ constexpr int SK_NBUF = 2;                        // ring of B buffers
 constexpr int SK_OUT_PITCH = SK_BN * 2 + 16;      // staging row: 128 outputs + pad
 constexpr int SK_OUT = SK_BM * SK_OUT_PITCH;      // one staging tile
 constexpr int SK_LDS = SK_NBUF * SK_BUF + 2 * SK_OUT;
+constexpr int SK_WALK = 16;                       // tiles along n per workgroup
 constexpr int SK_THREADS = 512;                   // 4 multiplying, 2 loading, 2 storing waves
 
 __global__ __launch_bounds__(SK_THREADS) void gemm_shortk_kernel(gemm_args_t a,
@@ -277,7 +278,7 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_shortk_kernel(gemm_args_t a,
 
 // Both operands contiguous along a single k mode of exactly 128 elements, single m and n
 // modes, C contiguous along n, strides small enough for 32-bit in-tile offsets, and enough
-// tiles for a workgroup per row of tiles to fill the device.
+// rows of tiles for several workgroups per compute unit.
 bool gemm_shortk_eligible(gemm_args_t const& a)
 {
     if (!a.lin || a.K != SK_K || a.a_mode != 0 || a.b_mode != 0 || a.c_mode != 3) return false;
@@ -287,14 +288,18 @@ bool gemm_shortk_eligible(gemm_args_t const& a)
     if (uint64_t(a.gm.sx[0]) * 256 * 2 >= (1ull << 31)) return false;
     if (uint64_t(a.gn.sx[0]) * 256 * 2 >= (1ull << 31)) return false;
     uint64_t const tiles_m = (a.M + SK_BM - 1) / SK_BM, tiles_n = (a.N + SK_BN - 1) / SK_BN;
-    return tiles_n >= 4 && tiles_m * tiles_n * a.batch >= 2048 &&
+    uint64_t const walks = (tiles_n + SK_WALK - 1) / SK_WALK;  // workgroups per row of tiles
+    // Measured against the kernel that takes a workgroup per tile: ahead from about four
+    // workgroups per compute unit on (1.3x at 16 per compute unit), behind below that,
+    // where its long set-up (the rows of A) is not hidden by other workgroups
+    return tiles_n >= 4 && tiles_m * walks * a.batch >= 1024 &&
            tiles_m * tiles_n * a.batch < (1ull << 31);
 }
 
 void launch_gemm_shortk(gemm_args_t const& a0, hipStream_t stream)
 {
     gemm_args_t a = with_tile(a0, SK_BM, SK_BN);
-    uint32_t const tpb = a.tiles_n < 16 ? a.tiles_n : 16;
+    uint32_t const tpb = a.tiles_n < SK_WALK ? a.tiles_n : SK_WALK;
     uint32_t const chunks = (a.tiles_n + tpb - 1) / tpb;
     static bool const raised = [] {
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_shortk_kernel),

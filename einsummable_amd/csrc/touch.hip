@@ -401,7 +401,12 @@ __global__ __launch_bounds__(256) void fill_constant_kernel(uint64_t n_vec, vec_
     static_assert(V == 4, "16-byte pattern");
     u32x4 const v = {pat.v[0], pat.v[1], pat.v[2], pat.v[3]};
     if (n_vec >= (4u << 20)) {
-        __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(out) + i);
+        // as an instruction: the optimiser merges a hinted and a plain store of the same
+        // value in the two arms of a branch into one plain store
+        asm volatile("global_store_dwordx4 %0, %1, off nt\n\ts_nop 1"
+                     :
+                     : "v"(reinterpret_cast<u32x4*>(out) + i), "v"(v)
+                     : "memory");
     } else {
         reinterpret_cast<u32x4*>(out)[i] = v;
     }
