@@ -326,6 +326,16 @@ std::shared_ptr<plan_t> plan_contraction(einsummable_t const& e, int)
             p->workspace_bytes = S * Bt * M * N * 4;
         }
     }
+    a.warm_a_bytes = a.warm_b_bytes = 0;
+    if (a.c_stream && dt == dtype_t::f16) {
+        uint64_t const lhs = e.inn_nelem(swapped ? 1 : 0) * dtype_size(dt);
+        uint64_t const rhs = e.inn_nelem(swapped ? 0 : 1) * dtype_size(dt);
+        const char*    env = std::getenv("ES_KM_GEMM_WARM");  // tuning and tests
+        if (lhs + rhs <= (160ull << 20) && !(env && env[0] == '0')) {
+            a.warm_a_bytes = lhs;
+            a.warm_b_bytes = rhs;
+        }
+    }
     a.shortk = 0;
     if (dt == dtype_t::f16 && p->planned_dma && p->bm == 128 && p->bn == 128 &&
         gemm::gemm_shortk_eligible(a)) {
@@ -341,7 +351,7 @@ std::shared_ptr<plan_t> plan_contraction(einsummable_t const& e, int)
                      " M=" + std::to_string(M) + " N=" + std::to_string(N) + " K=" +
                      std::to_string(K) + " batch=" + std::to_string(Bt) +
                      (a.splits > 1 ? " split_k=" + std::to_string(a.splits) : "") +
-                     (a.shortk ? " resident_a" : "");
+                     (a.shortk ? " resident_a" : "") + (a.warm_a_bytes ? " warm_operands" : "");
     return p;
 }
 

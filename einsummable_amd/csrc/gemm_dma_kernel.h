@@ -44,6 +44,18 @@ __device__ __forceinline__ void load_to_lds_16(void const* base, uint32_t voff, 
         : "memory");  // m0 is not kept live by the compiler across statements
 }
 
+// 64 lanes x 4 bytes from `base + voff` (per lane) to LDS at `lds_addr + 4 * lane`
+__device__ __forceinline__ void load_to_lds_4(void const* base, uint32_t voff, uint32_t lds_addr)
+{
+    asm volatile(
+        "s_mov_b32 m0, %0\n\t"
+        "s_nop 0\n\t"
+        "global_load_lds_dword %1, %2"
+        :
+        : "s"(lds_addr), "v"(voff), "s"(base)
+        : "memory");
+}
+
 template <int VM>
 __device__ __forceinline__ void wait_loads_and_lds()
 {

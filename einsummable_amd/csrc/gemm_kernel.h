@@ -45,6 +45,10 @@ struct gemm_args_t {
     float*      ws;
     // m, n and k are single modes, C is contiguous along n and 256 rows of C span less than
     // 2^31 bytes: every in-tile offset is a 32-bit multiple of a stride
+    // Bytes of the two operands when C is streamed past the caches and both operands together
+    // fit the memory-side cache with room to spare, else 0: they are then read once, by a
+    // kernel of their own, right before the product (gemm_warm_operands).
+    uint64_t    warm_a_bytes, warm_b_bytes;
     int         lin;
     // planned for the kernel that keeps A in registers and walks along n (K = 128, fp16)
     int         shortk;
@@ -872,6 +876,13 @@ void launch_gemm_f32(int bm, int bn, gemm_args_t const& a, hipStream_t stream);
 void launch_gemm_f64(int bm, int bn, gemm_args_t const& a, hipStream_t stream);
 double probe_mfma_f16(void const* operands, void* scratch, int blocks, int iters,
                       hipStream_t stream);
+
+// Reads `bytes` at `p` and keeps nothing: the lines end up in the L2 and in the memory-side
+// cache behind it.  Used ahead of a product whose output is written at HBM speed: operand
+// reads that have to go to HBM in the middle of that write stream cost far more than their
+// size suggests (attention scores, 128 MiB of operands against 1 GiB of output: 0.35 ms
+// with cold operands, 0.21 ms with warm ones plus 0.03 ms for warming them).
+void gemm_warm_operands(void const* p, uint64_t bytes, hipStream_t stream);
 
 // The fp16 kernel for reductions of exactly 128 elements (gemm_shortk_kernel.h)
 bool gemm_shortk_eligible(gemm_args_t const& a);

@@ -35,7 +35,9 @@ constexpr int SK_BUF = SK_BN * SK_RB;             // one B buffer
 constexpr int SK_NBUF = 2;                        // ring of B buffers
 constexpr int SK_OUT_PITCH = SK_BN * 2 + 16;      // staging row: 128 outputs + pad
 constexpr int SK_OUT = SK_BM * SK_OUT_PITCH;      // one staging tile
-constexpr int SK_LDS = SK_NBUF * SK_BUF + 2 * SK_OUT;
+constexpr int SK_LDS = SK_NBUF * SK_BUF + 2 * SK_OUT + 512;  // + scratch of the prefetches
+constexpr int SK_PF_DIST = 4;                     // tiles the L2 prefetch runs ahead
+constexpr int SK_PF_LOADS = 2;                    // 128-byte lines per row of B
 constexpr int SK_WALK = 16;                       // tiles along n per workgroup
 constexpr int SK_THREADS = 512;                   // 4 multiplying, 2 loading, 2 storing waves
 
@@ -95,6 +97,7 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_shortk_kernel(gemm_args_t a,
         constexpr int  PER_WAVE = SK_BN / 4 / 2;  // load instructions per tile per wave
         auto tile_loads = [&](uint32_t tn) {
             uint32_t const buf = (tn - t0) % SK_NBUF;
+            static_assert(SK_NBUF == 2, "the waits below assume one tile of lookahead");
             uint32_t const n0 = tn * SK_BN;
             uint32_t const last = a.N - 1 - n0;  // rows past the end re-read the last one
             // the base goes into a scalar register pair of the load instructions (the
@@ -112,32 +115,84 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_shortk_kernel(gemm_args_t a,
                 load_to_lds_16(base, voff, lds_base + buf * SK_BUF + q * 1024);
             }
         };
-        // wait until tile `t` has landed: tiles younger than it (at most two) stay in flight
-        auto wait_tile = [&](uint32_t t) {
-            uint32_t const newest = t + (SK_NBUF - 1) < t1 ? t + (SK_NBUF - 1) : t1;  // one past
-            uint32_t const younger = newest > t + 1 ? newest - (t + 1) : 0;
-            if (younger >= 2) {
-                wait_loads_and_lds<2 * PER_WAVE>();
-            } else if (younger == 1) {
-                wait_loads_and_lds<PER_WAVE>();
-            } else {
-                wait_loads_and_lds<0>();
+        // Brings tile `tn` into the L2 only (one dword per 128-byte line into a scratch
+        // corner of LDS that nobody reads).  The tile needed next must not wait for HBM: with
+        // C being written at full speed a read that misses the L2 takes microseconds, and
+        // the lookahead of the buffer ring alone is one tile.
+        auto prefetch = [&](T const* Bx, uint32_t tn) {
+            uint32_t const n0 = tn * SK_BN;
+            uint32_t const last = a.N - 1 - n0;
+            uint64_t const p = reinterpret_cast<uint64_t>(Bx + int64_t(n0) * ldb);
+            uint32_t const lo = uint32_t(__builtin_amdgcn_readfirstlane(uint32_t(p)));
+            uint32_t const hi = uint32_t(__builtin_amdgcn_readfirstlane(uint32_t(p >> 32)));
+            T const* const base = reinterpret_cast<T const*>((uint64_t(hi) << 32) | lo);
+            uint32_t const row = uint32_t(half) * 64 + uint32_t(lane);
+            uint32_t const src = row < last ? row : last;
+#pragma unroll
+            for (int u = 0; u != SK_PF_LOADS; ++u) {
+                load_to_lds_4(base, src * ldb * 2 + uint32_t(u) * 128,
+                              lds_base + SK_NBUF * SK_BUF + 2 * SK_OUT + uint32_t(half) * 256);
             }
         };
-        for (uint32_t t = t0; t != t1 && t != t0 + (SK_NBUF - 1); ++t) tile_loads(t);
-        wait_tile(t0);
+        tile_loads(t0);
+        uint32_t ahead = 0;  // prefetch instructions younger than the tile loads
+        for (uint32_t p = 1; p <= SK_PF_DIST && t0 + p < t1; ++p) {
+            prefetch(B, t0 + p);
+            ahead += SK_PF_LOADS;
+        }
+        // The workgroup that will follow this one on the compute unit (the XCD's 32 units take
+        // consecutive logical workgroups in turn): its rows of A and its first tile of B.
+        // Its own first loads then hit the L2 instead of waiting for HBM.
+        {
+            uint32_t const per_xcd = gridDim.x / 8;
+            uint32_t const next = id + 32;
+            if (blockIdx.x < per_xcd * 8 && blockIdx.x / 8 + 32 < per_xcd) {
+                uint32_t const nbz = next / per_batch;
+                uint32_t const nrem = next - nbz * per_batch;
+                uint32_t const nchunk = nrem / a.tiles_m;
+                uint32_t const ntm = nrem - nchunk * a.tiles_m;
+                int64_t        nboa, nbob;
+                group_offsets(a.gb, nbz, nboa, nbob);
+                // rows of A: 128 rows of 256 bytes, this wave's half
+                {
+                    T const* const An = static_cast<T const*>(a.A) + nboa;
+                    uint32_t const m_first = ntm * SK_BM;
+                    uint32_t const last = a.M - 1 - m_first;
+                    uint64_t const p = reinterpret_cast<uint64_t>(An + int64_t(m_first) * lda);
+                    uint32_t const lo = uint32_t(__builtin_amdgcn_readfirstlane(uint32_t(p)));
+                    uint32_t const hi = uint32_t(__builtin_amdgcn_readfirstlane(uint32_t(p >> 32)));
+                    T const* const base = reinterpret_cast<T const*>((uint64_t(hi) << 32) | lo);
+                    uint32_t const row = uint32_t(half) * 64 + uint32_t(lane);
+                    uint32_t const src = row < last ? row : last;
+#pragma unroll
+                    for (int u = 0; u != SK_PF_LOADS; ++u) {
+                        load_to_lds_4(base, src * lda * 2 + uint32_t(u) * 128,
+                                      lds_base + SK_NBUF * SK_BUF + 2 * SK_OUT + uint32_t(half) * 256);
+                    }
+                }
+                prefetch(static_cast<T const*>(a.B) + nbob, nchunk * tiles_per_block);
+                ahead += 2 * SK_PF_LOADS;
+            }
+        }
+        // the tile has landed; the prefetches behind it may still be in flight
+        switch (ahead / SK_PF_LOADS) {
+            case 0: wait_loads_and_lds<0>(); break;
+            case 1: wait_loads_and_lds<1 * SK_PF_LOADS>(); break;
+            case 2: wait_loads_and_lds<2 * SK_PF_LOADS>(); break;
+            case 3: wait_loads_and_lds<3 * SK_PF_LOADS>(); break;
+            case 4: wait_loads_and_lds<4 * SK_PF_LOADS>(); break;
+            case 5: wait_loads_and_lds<5 * SK_PF_LOADS>(); break;
+            default: wait_loads_and_lds<6 * SK_PF_LOADS>(); break;
+        }
         __builtin_amdgcn_s_barrier();
         for (uint32_t t = t0; t != t1; ++t) {
-            // the buffer of tile t + 3 is the one tile t - 1 was read from
-            if (t + (SK_NBUF - 1) < t1) tile_loads(t + (SK_NBUF - 1));
-            if (t + 1 != t1) {
-                // tiles issued so far: up to t + 3; younger than t + 1: up to two
-                uint32_t const issued = t + SK_NBUF < t1 ? t + SK_NBUF : t1;  // one past
-                uint32_t const younger = issued - (t + 2);
-                if (younger >= 2) {
-                    wait_loads_and_lds<2 * PER_WAVE>();
-                } else if (younger == 1) {
-                    wait_loads_and_lds<PER_WAVE>();
+            // the buffer of tile t + 1 is the one tile t - 1 was read from
+            if (t + 1 < t1) tile_loads(t + 1);
+            bool const pf = t + 1 + SK_PF_DIST < t1;
+            if (pf) prefetch(B, t + 1 + SK_PF_DIST);
+            if (t + 1 < t1) {
+                if (pf) {
+                    wait_loads_and_lds<SK_PF_LOADS>();
                 } else {
                     wait_loads_and_lds<0>();
                 }
