@@ -187,6 +187,7 @@ void kernel_manager_t::operator()(touch_t const& touch_, hipStream_t stream, voi
         small = small && a.size[s] < (1ull << 32);
     }
     a.small = small && a.n_vec < (1ull << 32);
+    a.outer = a.size[0] != 1 || a.size[1] != 1 ? 3 : (a.size[2] != 1 ? 1 : 0);
 
     int op = 0;
     if (t.castable) op = 1 + int(t.castable.value());

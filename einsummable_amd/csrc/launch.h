@@ -19,6 +19,8 @@ struct touch_launch_t {
     uint64_t n_vec;  // size[0]*size[1]*size[2]*vec_per_row
     int      vec;    // elements per vector: 16 / elem_size, or 1
     bool     small;  // n_vec and every extent fit 32 bits
+    int      outer;  // outer dimensions with more than one entry (0: the region is one row,
+                     // 1: rows of one outer dimension, slot 2; else the general decomposition)
 };
 
 // op: 0 copy, 1 add, 2 mul, 3 min, 4 max.  dtype_code: 0 f16, 1 f32, 2 f64, 3 c64.

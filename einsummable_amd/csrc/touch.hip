@@ -21,7 +21,7 @@ namespace
 {
 
 constexpr int TOUCH_BLOCK = 256;
-constexpr int TOUCH_UNROLL = 4;
+constexpr int TOUCH_UNROLL = 1;
 
 struct c64_t {
     float re, im;
@@ -93,7 +93,17 @@ __global__ __launch_bounds__(TOUCH_BLOCK) void touch_kernel(touch_launch_t a, T*
         live[u] = idx < a.n_vec;
         if (live[u]) {
             uint64_t oi, ii;
-            if (a.small) {
+            if (a.outer == 0) {
+                // one contiguous row on both sides (what a whole-tensor copy simplifies to):
+                // no index decomposition at all
+                ii = a.base_inn + idx * V;
+                oi = a.base_out + idx * V;
+            } else if (a.outer == 1 && a.small) {
+                uint32_t const r = uint32_t(idx) / uint32_t(a.vec_per_row);
+                uint32_t const c = uint32_t(idx) - r * uint32_t(a.vec_per_row);
+                ii = a.base_inn + r * a.str_inn[2] + uint64_t(c) * V;
+                oi = a.base_out + r * a.str_out[2] + uint64_t(c) * V;
+            } else if (a.small) {
                 uint32_t r = uint32_t(idx);
                 uint32_t c = r % uint32_t(a.vec_per_row);
                 r /= uint32_t(a.vec_per_row);
