@@ -23,6 +23,9 @@
 #pragma once
 #include "gemm_dma_kernel.h"
 
+#include <algorithm>
+#include <cstdlib>
+
 namespace es
 {
 namespace gemm
@@ -38,7 +41,6 @@ constexpr int SK_OUT = SK_BM * SK_OUT_PITCH;      // one staging tile
 constexpr int SK_LDS = SK_NBUF * SK_BUF + 2 * SK_OUT + 512;  // + scratch of the prefetches
 constexpr int SK_PF_DIST = 4;                     // tiles the L2 prefetch runs ahead
 constexpr int SK_PF_LOADS = 2;                    // 128-byte lines per row of B
-constexpr int SK_WALK = 16;                       // tiles along n per workgroup
 constexpr int SK_THREADS = 512;                   // 4 multiplying, 2 loading, 2 storing waves
 
 __global__ __launch_bounds__(SK_THREADS) void gemm_shortk_kernel(gemm_args_t a,
@@ -331,6 +333,29 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_shortk_kernel(gemm_args_t a,
     }
 }
 
+// Tiles along n that one workgroup walks, or 0 when the kernel that takes a workgroup per
+// tile is the better choice.  Measured with cold caches on b x s x s x 128 products, time of
+// the per-tile kernel / time of this one: walks of 16 tiles pay from 2048 workgroups on
+// (128 x 2048: 1.19); with fewer, walks of 8 do (64 x 2048: 1.08, 32 x 2048: 1.12,
+// 128 x 1024: 1.05, 32 x 1024: 1.19, 256 x 512: 1.20) down to about 512 workgroups; rows of
+// more than 16 tiles cut into several walks lose below 2048 workgroups (8 x 4096: 0.87-0.95,
+// 4 x 8192: 0.81-0.91).
+inline uint32_t shortk_walk(gemm_args_t const& a)
+{
+    uint64_t const tiles_m = (a.M + SK_BM - 1) / SK_BM, tiles_n = (a.N + SK_BN - 1) / SK_BN;
+    if (tiles_n < 4 || tiles_m * tiles_n * a.batch >= (1ull << 31)) return 0;
+    static uint64_t const scale = [] {
+        const char* env = std::getenv("ES_KM_GEMM_RESIDENT_MIN");  // tuning and tests: percent
+        return uint64_t(env ? std::max(1, std::atoi(env)) : 100);
+    }();
+    uint64_t const rows = tiles_m * a.batch;
+    uint64_t const walks16 = rows * ((tiles_n + 15) / 16);
+    if (walks16 * 100 >= 2048 * scale) return 16;
+    if (tiles_n > 16) return 0;
+    uint64_t const walks8 = rows * ((tiles_n + 7) / 8);
+    return walks8 * 100 >= 512 * scale ? 8 : 0;
+}
+
 // Both operands contiguous along a single k mode of exactly 128 elements, single m and n
 // modes, C contiguous along n, strides small enough for 32-bit in-tile offsets, and enough
 // rows of tiles for several workgroups per compute unit.
@@ -342,19 +367,14 @@ bool gemm_shortk_eligible(gemm_args_t const& a)
     if (a.gm.sx[0] <= 0 || a.gn.sx[0] <= 0) return false;
     if (uint64_t(a.gm.sx[0]) * 256 * 2 >= (1ull << 31)) return false;
     if (uint64_t(a.gn.sx[0]) * 256 * 2 >= (1ull << 31)) return false;
-    uint64_t const tiles_m = (a.M + SK_BM - 1) / SK_BM, tiles_n = (a.N + SK_BN - 1) / SK_BN;
-    uint64_t const walks = (tiles_n + SK_WALK - 1) / SK_WALK;  // workgroups per row of tiles
-    // Measured against the kernel that takes a workgroup per tile: ahead from about four
-    // workgroups per compute unit on (1.3x at 16 per compute unit), behind below that,
-    // where its long set-up (the rows of A) is not hidden by other workgroups
-    return tiles_n >= 4 && tiles_m * walks * a.batch >= 1024 &&
-           tiles_m * tiles_n * a.batch < (1ull << 31);
+    return shortk_walk(a) != 0;
 }
 
 void launch_gemm_shortk(gemm_args_t const& a0, hipStream_t stream)
 {
     gemm_args_t a = with_tile(a0, SK_BM, SK_BN);
-    uint32_t const tpb = a.tiles_n < SK_WALK ? a.tiles_n : SK_WALK;
+    uint32_t const walk = shortk_walk(a);
+    uint32_t const tpb = a.tiles_n < walk ? a.tiles_n : walk;
     uint32_t const chunks = (a.tiles_n + tpb - 1) / tpb;
     static bool const raised = [] {
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_shortk_kernel),
