@@ -112,11 +112,24 @@ void choose_tile(dtype_t dt, uint64_t M, uint64_t N, uint64_t K, uint64_t batch,
                                             {256, 128, 0.80, 1.00},
                                             {128, 128, 0.68, 1.00}};
     double best = 0;
+    uint64_t const nk = K * dtype_size(dt) / 64;
     for (tile_option_t const& o : options) {
         uint64_t tiles = ((M + o.bm - 1) / o.bm) * ((N + o.bn - 1) / o.bn) * batch;
-        uint64_t rounds = (tiles + 255) / 256;
-        double   t = double(rounds) * double(o.bm) * double(o.bn) /
-                   (dt == dtype_t::f16 ? o.eff16 : o.eff32);
+        // at most 128 tiles and a long reduction: plan_contraction will cut k into splits
+        // (same rule as there), which costs a pass over the fp32 partial tiles.  In units of
+        // tile area per matrix-core time: bytes moved at ~4 TB/s against 2 K flop per unit
+        // of area at the compute unit's share of ~1.2 PFLOP/s (f16) or ~0.14 PFLOP/s (f32)
+        uint64_t const S = (tiles <= 128 && nk >= 16) ? std::min<uint64_t>({256 / tiles, nk / 8, 64}) : 1;
+        double fold = 0;
+        if (S > 1) {
+            double const ratio = dt == dtype_t::f16 ? 1.17 : 0.14;
+            fold = (4.0 * double(S) + elem) * double(M) * double(N) * double(batch) * ratio /
+                   (2.0 * double(K));
+        }
+        uint64_t rounds = (tiles * S + 255) / 256;
+        double   t = double(rounds) * double(o.bm) * double(o.bn) / double(S) /
+                       (dt == dtype_t::f16 ? o.eff16 : o.eff32) +
+                   fold;
         if (best == 0 || t < best * 0.97) {  // near ties go to the larger tile (listed first)
             best = t;
             bm = o.bm;
