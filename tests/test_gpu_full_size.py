@@ -46,6 +46,32 @@ def test_c1_f32_matmul_2048_cubed(km):
     assert np.max(np.abs(C[rows] - want)) <= 1e-4 * max(scale, 1.0) * 4
 
 
+def test_f32_product_whose_result_is_streamed_past_the_caches(km):
+    # 4096 x 4096 f32 = 64 MiB: the size from which the result is stored with streaming
+    # stores (written as instructions); a short reduction keeps the check cheap
+    import torch
+
+    m, k = 4096, 256
+    g = torch.Generator(device="cuda").manual_seed(13)
+    a = torch.rand(m, k, device="cuda", generator=g) * 2 - 1
+    b = torch.rand(m, k, device="cuda", generator=g) * 2 - 1
+    c = torch.full((m, m), float("nan"), device="cuda")
+    e = E.from_str("ij,kj->ik", dict(i=m, j=k, k=m), "*[hole|f32@0,hole|f32@1]", "+")
+    run(km, e, c, [a, b])
+    torch.cuda.synchronize()
+    assert "load=direct_to_lds" in km.describe(e)
+    A, B, C = (t.cpu().numpy().astype(np.float64) for t in (a, b, c))
+    assert not np.isnan(C).any()              # every element was written
+    r = np.random.RandomState(14)
+    for _ in range(4):
+        v = r.uniform(-1, 1, m)
+        lhs, rhs = C @ v, A @ (B.T @ v)
+        assert np.max(np.abs(lhs - rhs)) <= 1e-4 * np.sqrt(np.mean(rhs * rhs))
+    rows = r.randint(0, m, 64)
+    want = A[rows] @ B.T
+    assert np.max(np.abs(C[rows] - want)) <= 1e-4 * np.sqrt(np.mean(want * want)) * 4
+
+
 def test_c2_elementwise_and_reductions_8192_squared(km):
     import torch
 
