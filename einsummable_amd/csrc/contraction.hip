@@ -328,6 +328,10 @@ std::shared_ptr<plan_t> plan_contraction(einsummable_t const& e, int)
                                                           : 0;
     }
     uint64_t const tiles = uint64_t(a.tiles_m) * a.tiles_n * Bt;
+    {
+        const char* env = std::getenv("ES_KM_GEMM_XCD_BATCH");  // tuning and tests
+        a.xcd_total = Bt > 1 && tiles < (1ull << 32) && !(env && env[0] == '0') ? uint32_t(tiles) : 0;
+    }
     uint64_t const nk = K * dtype_size(dt) / 64;
     if (p->planned_dma && nk >= 16) {
         uint64_t S = tiles <= 128 ? std::min<uint64_t>({256 / tiles, nk / 8, 64}) : 1;

@@ -49,6 +49,9 @@ struct gemm_args_t {
     // fit the memory-side cache with room to spare, else 0: they are then read once, by a
     // kernel of their own, right before the product (gemm_warm_operands).
     uint64_t    warm_a_bytes, warm_b_bytes;
+    // tiles_m * tiles_n * batch when the batch has more than one entry and the product fits
+    // 32 bits (the XCD renumbering then runs across batch entries), else 0
+    uint32_t    xcd_total;
     int         lin;
     // planned for the kernel that keeps A in registers and walks along n (K = 128, fp16)
     int         shortk;
@@ -894,6 +897,7 @@ inline gemm_args_t with_tile(gemm_args_t a, int bm, int bn)
     a.tiles_m = (a.M + uint32_t(bm) - 1) / uint32_t(bm);
     a.tiles_n = (a.N + uint32_t(bn) - 1) / uint32_t(bn);
     a.group_magic = 0;  // belongs to the tile counts it was computed for
+    a.xcd_total = 0;
     return a;
 }
 
