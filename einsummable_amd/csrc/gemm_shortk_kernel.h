@@ -335,25 +335,19 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_shortk_kernel(gemm_args_t a,
 
 // Tiles along n that one workgroup walks, or 0 when the kernel that takes a workgroup per
 // tile is the better choice.  Measured with cold caches on b x s x s x 128 products, time of
-// the per-tile kernel / time of this one: walks of 16 tiles pay from 2048 workgroups on
-// (128 x 2048: 1.19); with fewer, walks of 8 do (64 x 2048: 1.08, 32 x 2048: 1.12,
-// 128 x 1024: 1.05, 32 x 1024: 1.19, 256 x 512: 1.20) down to about 512 workgroups; rows of
-// more than 16 tiles cut into several walks lose below 2048 workgroups (8 x 4096: 0.87-0.95,
-// 4 x 8192: 0.81-0.91).
+// the per-tile kernel / time of this one, walks of 16 tiles: 1.09-1.23 from 1024 workgroups
+// on (128 x 2048, 64 x 2048, 32 x 4096, 4 x 8192), 1.02 for 128 x 1024; below that, and for
+// rows of four tiles, 0.86-0.97 (8 .. 32 x 2048, 8 x 4096, 256 x 512).
 inline uint32_t shortk_walk(gemm_args_t const& a)
 {
     uint64_t const tiles_m = (a.M + SK_BM - 1) / SK_BM, tiles_n = (a.N + SK_BN - 1) / SK_BN;
-    if (tiles_n < 4 || tiles_m * tiles_n * a.batch >= (1ull << 31)) return 0;
-    static uint64_t const scale = [] {
-        const char* env = std::getenv("ES_KM_GEMM_RESIDENT_MIN");  // tuning and tests: percent
-        return uint64_t(env ? std::max(1, std::atoi(env)) : 100);
+    if (tiles_n < 8 || tiles_m * tiles_n * a.batch >= (1ull << 31)) return 0;
+    static uint64_t const min_walks = [] {
+        const char* env = std::getenv("ES_KM_GEMM_RESIDENT_MIN");  // tuning and tests
+        return uint64_t(env ? std::max(1, std::atoi(env)) : 1024);
     }();
-    uint64_t const rows = tiles_m * a.batch;
-    uint64_t const walks16 = rows * ((tiles_n + 15) / 16);
-    if (walks16 * 100 >= 2048 * scale) return 16;
-    if (tiles_n > 16) return 0;
-    uint64_t const walks8 = rows * ((tiles_n + 7) / 8);
-    return walks8 * 100 >= 512 * scale ? 8 : 0;
+    uint64_t const walks = tiles_m * a.batch * ((tiles_n + 15) / 16);
+    return walks >= min_walks ? 16 : 0;
 }
 
 // Both operands contiguous along a single k mode of exactly 128 elements, single m and n

@@ -245,10 +245,10 @@ RESIDENT_A_CASES = [
     # stay in registers and a workgroup walks along n.  Full tiles, ragged m and n, a batch
     # of two modes with strides (heads stored between sequence and head dimension), more
     # than 16 tiles along n (several walks per row of tiles)
-    ("bid,bjd->bij", dict(b=128, i=1024, j=512, d=128)),
-    ("bid,bjd->bij", dict(b=130, i=1000, j=504, d=128)),
-    ("bihd,bjhd->bhij", dict(b=8, h=16, i=1024, j=512, d=128)),
-    ("bid,bjd->bij", dict(b=86, i=1024, j=5000, d=128)),
+    ("bid,bjd->bij", dict(b=128, i=1024, j=1024, d=128)),
+    ("bid,bjd->bij", dict(b=130, i=1000, j=1016, d=128)),
+    ("bihd,bjhd->bhij", dict(b=8, h=16, i=1024, j=1024, d=128)),
+    ("bid,bjd->bij", dict(b=43, i=1024, j=5000, d=128)),
 ]
 
 
