@@ -99,14 +99,13 @@ void choose_tile(dtype_t dt, uint64_t M, uint64_t N, uint64_t K, uint64_t batch,
         if (K >= 1024 && M >= 512 && N >= 512 && big_tiles >= 768) bm = bn = 256;
         return;
     }
-    // Streaming shapes (one operand read once, little reuse: attention's P.V) are bound by
-    // HBM; with many rounds of tiles the small tile's extra workgroups per compute unit keep
-    // more loads in flight
+    // Streaming shapes (one operand read once, little reuse: attention's P.V, a vector or a
+    // few rows against a weight matrix) are bound by HBM: the small tile's extra workgroups
+    // per compute unit keep more loads in flight
     double const elem = double(dtype_size(dt));
     double const intensity = 2.0 * double(M) * double(N) * double(K) /
                              ((double(M) * K + double(N) * K + double(M) * N) * elem);
-    uint64_t const small_tiles = ((M + 127) / 128) * ((N + 127) / 128) * batch;
-    if (dt == dtype_t::f16 && intensity < 150.0 && small_tiles >= 1024) return;
+    if (dt == dtype_t::f16 && intensity < 150.0) return;
     static tile_option_t const options[] = {{256, 256, 1.00, 1.00},
                                             {128, 256, 0.80, 1.00},
                                             {256, 128, 0.80, 1.00},

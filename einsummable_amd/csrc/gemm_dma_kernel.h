@@ -97,26 +97,13 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
     int const wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     int const wm = wave >> 1, wn = wave & 1;
 
-    // Workgroups go to the eight XCDs (each with its own L2) round robin in the order of their
-    // linear index.  The tiles are renumbered so that one XCD works on a contiguous run of
-    // them -- across batch entries too: with the run inside one batch entry only, every XCD
-    // held a piece of every entry and fetched that entry's operands for itself (attention's
-    // P.V, 16 tiles per head: 1.67 GiB left the L2s for 1.06 GiB of operands).
+    // one XCD (one L2) works on a contiguous run of tiles, across batch entries: attention's
+    // P.V, 16 tiles per head, moved 1.67 GiB out of the L2s for 1.06 GiB of operands while the
+    // run stayed inside one batch entry
     uint32_t const n_tiles = a.tiles_m * a.tiles_n;
     uint32_t       tile = blockIdx.x;
     uint32_t       bz = blockIdx.y;
-    if (a.xcd_total) {
-        uint32_t const linear = tile + n_tiles * bz;
-        uint32_t const per_xcd = a.xcd_total / 8;
-        if (linear < per_xcd * 8) {
-            uint32_t const run = (linear % 8) * per_xcd + linear / 8;
-            bz = run / n_tiles;
-            tile = run - bz * n_tiles;
-        }
-    } else {
-        uint32_t const per_xcd = n_tiles / 8;
-        if (tile < per_xcd * 8) tile = (tile % 8) * per_xcd + tile / 8;
-    }
+    xcd_renumber(a, n_tiles, tile, bz);
     constexpr uint32_t GROUP_M = 4;
     uint32_t const     in_group = GROUP_M * a.tiles_n;
     // all of this is uniform: a multiply-high and shifts stay on the scalar unit, while a

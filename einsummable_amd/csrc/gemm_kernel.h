@@ -80,6 +80,28 @@ __device__ __forceinline__ void group_offsets(group_t const& g, uint32_t i, int6
     }
 }
 
+// Workgroups go to the eight XCDs (each with its own L2) round robin in the order of their
+// linear index (x fastest, then the batch in y).  The tiles are renumbered so that one XCD
+// works on a contiguous run of them -- across batch entries when xcd_total is set: with the
+// run inside one batch entry only, every XCD holds a piece of every entry and fetches that
+// entry's operands for itself.
+__device__ __forceinline__ void xcd_renumber(gemm_args_t const& a, uint32_t n_tiles,
+                                             uint32_t& tile, uint32_t& bz)
+{
+    if (a.xcd_total) {
+        uint32_t const linear = tile + n_tiles * bz;
+        uint32_t const per_xcd = a.xcd_total / 8;
+        if (linear < per_xcd * 8) {
+            uint32_t const run = (linear % 8) * per_xcd + linear / 8;
+            bz = run / n_tiles;
+            tile = run - bz * n_tiles;
+        }
+    } else {
+        uint32_t const per_xcd = n_tiles / 8;
+        if (tile < per_xcd * 8) tile = (tile % 8) * per_xcd + tile / 8;
+    }
+}
+
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float    float16_t __attribute__((ext_vector_type(16)));
 typedef float    float4_t __attribute__((ext_vector_type(4)));
@@ -363,17 +385,14 @@ __global__ __launch_bounds__(256) void gemm_kernel(gemm_args_t a)
     // runs at the same time form a compact rectangle that shares its A and B panels in L2.
     uint32_t const n_tiles = a.tiles_m * a.tiles_n;
     uint32_t       tile = blockIdx.x;
-    {
-        uint32_t const per_xcd = n_tiles / 8;
-        if (tile < per_xcd * 8) tile = (tile % 8) * per_xcd + tile / 8;
-    }
+    uint32_t       bz = blockIdx.y;
+    xcd_renumber(a, n_tiles, tile, bz);
     constexpr uint32_t GROUP_M = 8;
     uint32_t const     in_group = GROUP_M * a.tiles_n;
     uint32_t const     first_m = (tile / in_group) * GROUP_M;
     uint32_t const     rows = (a.tiles_m - first_m) < GROUP_M ? (a.tiles_m - first_m) : GROUP_M;
     uint32_t const     tm = first_m + (tile % in_group) % rows;
     uint32_t const     tn = (tile % in_group) / rows;
-    uint32_t const     bz = blockIdx.y;
 
     int64_t boa, bob, boc;
     {
@@ -545,17 +564,14 @@ __global__ __launch_bounds__(256) void gemm_fast_kernel(gemm_args_t a)
 
     uint32_t const n_tiles = a.tiles_m * a.tiles_n;
     uint32_t       tile = blockIdx.x;
-    {
-        uint32_t const per_xcd = n_tiles / 8;
-        if (tile < per_xcd * 8) tile = (tile % 8) * per_xcd + tile / 8;
-    }
+    uint32_t       bz = blockIdx.y;
+    xcd_renumber(a, n_tiles, tile, bz);
     constexpr uint32_t GROUP_M = 8;
     uint32_t const     in_group = GROUP_M * a.tiles_n;
     uint32_t const     first_m = (tile / in_group) * GROUP_M;
     uint32_t const     rows = (a.tiles_m - first_m) < GROUP_M ? (a.tiles_m - first_m) : GROUP_M;
     uint32_t const     tm = first_m + (tile % in_group) % rows;
     uint32_t const     tn = (tile % in_group) / rows;
-    uint32_t const     bz = blockIdx.y;
 
     int64_t boa, bob, boc;
     {
@@ -897,7 +913,8 @@ inline gemm_args_t with_tile(gemm_args_t a, int bm, int bn)
     a.tiles_m = (a.M + uint32_t(bm) - 1) / uint32_t(bm);
     a.tiles_n = (a.N + uint32_t(bn) - 1) / uint32_t(bn);
     a.group_magic = 0;  // belongs to the tile counts it was computed for
-    a.xcd_total = 0;
+    uint64_t const total = uint64_t(a.tiles_m) * a.tiles_n * a.batch;
+    a.xcd_total = a.xcd_total && total < (1ull << 32) ? uint32_t(total) : 0;
     return a;
 }
 
