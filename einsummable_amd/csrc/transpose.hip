@@ -4,8 +4,8 @@
 // einsummable_t::is_permutation, src/einsummable/einsummable.cc:740-743) that keeps its
 // innermost mode is a strided row copy and is handled by the generated elementwise kernel.
 // When the innermost mode of the input is not the innermost mode of the output, a direct
-// copy is uncoalesced on one side.  Here a 64 x 64 tile over (input-inner mode, output-inner
-// mode) goes through LDS: rows are read along the input's contiguous mode and written along
+// copy is uncoalesced on one side.  Here a tile over (input-inner mode, output-inner mode),
+// 64 x 64 up to 256 x 64 elements, goes through LDS: rows are read along the input's contiguous mode and written along
 // the output's contiguous mode, so both sides move whole 128..512-byte row segments.  All
 // other modes form the batch.  Pure data movement: results are bit-identical to the CPU's
 // permute_t (src/base/permute_.h) and to the interpreter.
@@ -14,6 +14,8 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <cstdlib>
+#include <string>
 
 namespace es
 {
@@ -32,12 +34,13 @@ struct transpose_args_t {
     uint32_t    tiles_i, tiles_o;
     uint64_t    n_blocks;
     uint32_t    nb;                 // number of batch modes
+    uint32_t    plain_stores;       // results go through the L2 instead of streaming past it
     uint32_t    bsize[MAXB];        // innermost batch mode first
     int64_t     bsi[MAXB], bso[MAXB];
 };
 
 // Tile origin and batch offsets of a workgroup; false when the workgroup has no tile.
-template <int EDGE>
+template <int EDGE, int EDGE_O = EDGE>
 __device__ __forceinline__ bool locate(transpose_args_t const& a, uint32_t& i0, uint32_t& o0,
                                        int64_t& off_i, int64_t& off_o)
 {
@@ -47,7 +50,8 @@ __device__ __forceinline__ bool locate(transpose_args_t const& a, uint32_t& i0, 
     uint32_t const ti = t % a.tiles_i;
     t /= a.tiles_i;
     uint32_t const to = t % a.tiles_o;
-    uint32_t bidx = t / a.tiles_o;
+    t /= a.tiles_o;
+    uint32_t bidx = t;
     off_i = 0;
     off_o = 0;
 #pragma unroll
@@ -61,7 +65,7 @@ __device__ __forceinline__ bool locate(transpose_args_t const& a, uint32_t& i0, 
         }
     }
     i0 = ti * EDGE;
-    o0 = to * EDGE;
+    o0 = to * EDGE_O;
     return true;
 }
 
@@ -69,61 +73,70 @@ __device__ __forceinline__ bool locate(transpose_args_t const& a, uint32_t& i0, 
 // consecutive elements of an input row and, after the turn through LDS, stores V consecutive
 // elements of an output row.  Needs every row start on both sides 16-byte aligned (strides,
 // batch offsets, extents and base pointers: checked on the host).
-// The tile edge is 128 for 2-byte elements (256-byte row segments), 64 otherwise.
-template <typename T>
-struct vec_tile_t {
-    static constexpr int edge = sizeof(T) == 2 ? 128 : 64;
-};
-
-template <typename T>
+// The tile is TI elements of the input-inner mode by TO elements of the output-inner mode;
+// vec_shape() picks it.
+template <typename T, int TI, int TO>
 __global__ __launch_bounds__(256) void transpose_vec_kernel(transpose_args_t a)
 {
-    constexpr int TT = vec_tile_t<T>::edge;
     constexpr int V = 16 / int(sizeof(T));
-    constexpr int LPR = TT / V;      // lanes per tile row
+    constexpr int LPR = TI / V;      // lanes per tile row on the way in
     constexpr int RPP = 256 / LPR;   // tile rows per pass of the workgroup
+    constexpr int LPR_O = TO / V;    // the same on the way out
+    constexpr int RPP_O = 256 / LPR_O;
     // pitch: an odd number of 4-byte words, so that a column walks over all banks
-    constexpr int PITCH = sizeof(T) == 2 ? TT + 2 : TT + 1;
+    constexpr int PITCH = sizeof(T) == 2 ? TI + 2 : TI + 1;
     typedef T vecT __attribute__((ext_vector_type(V)));
-    __shared__ T tile[TT * PITCH];
+    __shared__ T tile[TO * PITCH];
 
     uint32_t i0, o0;
     int64_t  off_i, off_o;
-    if (!locate<TT>(a, i0, o0, off_i, off_o)) return;
+    if (!locate<TI, TO>(a, i0, o0, off_i, off_o)) return;
     T const* const in = static_cast<T const*>(a.in) + off_i;
     T* const       out = static_cast<T*>(a.out) + off_o;
-    uint32_t const col = (threadIdx.x % LPR) * V;
-    uint32_t const row = threadIdx.x / LPR;
-
+    {
+        uint32_t const col = (threadIdx.x % LPR) * V;
+        uint32_t const row = threadIdx.x / LPR;
 #pragma unroll
-    for (int p = 0; p != TT / RPP; ++p) {
-        uint32_t const ol = row + p * RPP;
-        uint32_t const o = o0 + ol, i = i0 + col;
-        if (o < a.n_o && i < a.n_i) {  // n_i is a multiple of V: a started vector is whole
-            vecT v = __builtin_nontemporal_load(
-                reinterpret_cast<vecT const*>(in + int64_t(o) * a.si_o + i));
-            if constexpr (sizeof(T) == 2) {
-                typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-                u32x4 w = __builtin_bit_cast(u32x4, v);
-                uint32_t* dst = reinterpret_cast<uint32_t*>(&tile[ol * PITCH + col]);
+        for (int p = 0; p != TO / RPP; ++p) {
+            uint32_t const ol = row + p * RPP;
+            uint32_t const o = o0 + ol, i = i0 + col;
+            if (o < a.n_o && i < a.n_i) {  // n_i is a multiple of V: a started vector is whole
+                vecT v = __builtin_nontemporal_load(
+                    reinterpret_cast<vecT const*>(in + int64_t(o) * a.si_o + i));
+                if constexpr (sizeof(T) == 2) {
+                    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+                    u32x4 w = __builtin_bit_cast(u32x4, v);
+                    uint32_t* dst = reinterpret_cast<uint32_t*>(&tile[ol * PITCH + col]);
 #pragma unroll
-                for (int j = 0; j != 4; ++j) dst[j] = w[j];
-            } else {
+                    for (int j = 0; j != 4; ++j) dst[j] = w[j];
+                } else {
 #pragma unroll
-                for (int j = 0; j != V; ++j) tile[ol * PITCH + col + j] = v[j];
+                    for (int j = 0; j != V; ++j) tile[ol * PITCH + col + j] = v[j];
+                }
             }
         }
     }
     __syncthreads();
+    {
+        uint32_t const col = (threadIdx.x % LPR_O) * V;
+        uint32_t const row = threadIdx.x / LPR_O;
 #pragma unroll
-    for (int p = 0; p != TT / RPP; ++p) {
-        uint32_t const il = row + p * RPP;
-        uint32_t const i = i0 + il, o = o0 + col;
-        if (i < a.n_i && o < a.n_o) {
-            vecT v;
+        for (int p = 0; p != TI / RPP_O; ++p) {
+            uint32_t const il = row + p * RPP_O;
+            uint32_t const i = i0 + il, o = o0 + col;
+            if (i < a.n_i && o < a.n_o) {
+                vecT v;
 #pragma unroll
-            for (int j = 0; j != V; ++j) v[j] = tile[(col + j) * PITCH + il];
-            __builtin_nontemporal_store(v, reinterpret_cast<vecT*>(out + int64_t(i) * a.so_i + o));
+                for (int j = 0; j != V; ++j) v[j] = tile[(col + j) * PITCH + il];
+                vecT* d = reinterpret_cast<vecT*>(out + int64_t(i) * a.so_i + o);
+                // written in assembly: with a plain store in the other arm the compiler merges
+                // the two and drops the streaming hint
+                if (a.plain_stores) {
+                    *d = v;
+                } else {
+                    asm volatile("global_store_dwordx4 %0, %1, off nt" : : "v"(d), "v"(v) : "memory");
+                }
+            }
         }
     }
 }
@@ -176,6 +189,31 @@ __global__ __launch_bounds__(256) void transpose_kernel(transpose_args_t a)
     }
 }
 
+// Tile of the 16-byte kernel, measured on 4096..16384-square matrices with cold and with warm
+// caches.  4-byte elements: 512-byte segments on the way in and 256-byte segments on the way
+// out beat the square tile by 4..12 % once there are enough tiles to fill the device.
+// 2-byte elements: the same holds only for matrices well beyond the memory-side cache (2..6 %
+// at 16384 x 16384; at 8192 x 8192 the square tile is 6 % faster).
+inline void vec_shape(int elem_size, uint32_t n_i, uint32_t n_o, uint64_t batch, uint32_t& edge_i,
+                      uint32_t& edge_o)
+{
+    uint64_t const bytes = 2ull * n_i * n_o * batch * uint64_t(elem_size);
+    const char*    env = std::getenv("ES_KM_TRANSPOSE_TILE");  // tuning and tests
+    bool const     force_square = env && std::string(env) == "square";
+    bool const     force_long = env && std::string(env) == "long";
+    edge_i = edge_o = 64;
+    if (elem_size == 2) {
+        edge_i = edge_o = 128;
+        if (!force_square && (force_long || (bytes >= (1ull << 30) && n_i >= 256))) {
+            edge_i = 256;
+            edge_o = 64;
+        }
+    } else if (elem_size == 4) {
+        uint64_t const tiles = uint64_t((n_i + 127) / 128) * ((n_o + 63) / 64) * batch;
+        if (!force_square && (force_long || tiles >= 2048)) edge_i = 128;
+    }
+}
+
 struct transpose_plan_t : plan_t {
     transpose_args_t args;
     int              elem_size;
@@ -190,9 +228,10 @@ struct transpose_plan_t : plan_t {
         bool const aligned = reinterpret_cast<uintptr_t>(a.in) % 16 == 0 &&
                              reinterpret_cast<uintptr_t>(a.out) % 16 == 0;
         bool const vec = vec_ok && aligned;
-        uint32_t const edge = vec && elem_size == 2 ? 128 : 64;
-        a.tiles_i = (a.n_i + edge - 1) / edge;
-        a.tiles_o = (a.n_o + edge - 1) / edge;
+        uint32_t edge_i = 64, edge_o = 64;
+        if (vec) vec_shape(elem_size, a.n_i, a.n_o, batch, edge_i, edge_o);
+        a.tiles_i = (a.n_i + edge_i - 1) / edge_i;
+        a.tiles_o = (a.n_o + edge_o - 1) / edge_o;
         uint64_t const blocks = uint64_t(a.tiles_i) * a.tiles_o * batch;
         a.n_blocks = blocks;
         // a grid dimension times the block size must stay below 2^32
@@ -200,16 +239,16 @@ struct transpose_plan_t : plan_t {
         unsigned gy = unsigned((blocks + gx - 1) / gx);
         dim3     grid(gx, gy), block(256);
         if (vec) {
-            switch (elem_size) {
-                case 2:
-                    hipLaunchKernelGGL((transpose_vec_kernel<uint16_t>), grid, block, 0, stream, a);
-                    break;
-                case 4:
-                    hipLaunchKernelGGL((transpose_vec_kernel<uint32_t>), grid, block, 0, stream, a);
-                    break;
-                default:
-                    hipLaunchKernelGGL((transpose_vec_kernel<uint64_t>), grid, block, 0, stream, a);
-                    break;
+            if (elem_size == 2 && edge_i == 256) {
+                hipLaunchKernelGGL((transpose_vec_kernel<uint16_t, 256, 64>), grid, block, 0, stream, a);
+            } else if (elem_size == 2) {
+                hipLaunchKernelGGL((transpose_vec_kernel<uint16_t, 128, 128>), grid, block, 0, stream, a);
+            } else if (elem_size == 4 && edge_i == 128) {
+                hipLaunchKernelGGL((transpose_vec_kernel<uint32_t, 128, 64>), grid, block, 0, stream, a);
+            } else if (elem_size == 4) {
+                hipLaunchKernelGGL((transpose_vec_kernel<uint32_t, 64, 64>), grid, block, 0, stream, a);
+            } else {
+                hipLaunchKernelGGL((transpose_vec_kernel<uint64_t, 64, 64>), grid, block, 0, stream, a);
             }
         } else {
             switch (elem_size) {
@@ -298,11 +337,21 @@ std::shared_ptr<plan_t> plan_transpose(einsummable_t const& e, int)
         for (uint32_t d = 0; d != a.nb; ++d) ok = ok && a.bsi[d] % V == 0 && a.bso[d] % V == 0;
         p->vec_ok = ok;
     }
+    // Streaming stores send each 128..256-byte segment to the memory by itself; through the
+    // L2 the segments that neighbouring tiles write to the same rows leave together.  Kernel
+    // durations, 8192 x 8192: 2-byte elements 61 -> 50 us, 4-byte elements 137 -> 95 us;
+    // 16384 x 16384: 262 -> 230 us and 512 -> 474 us.  Small transposes, whose result stays
+    // in the L2 anyway, are faster streaming (4096 x 4096 2-byte: 11.6 against 14.5 us).
+    a.plain_stores = 2 * e.out_nelem() * uint64_t(p->elem_size) >= (128ull << 20);
+    if (const char* env = std::getenv("ES_KM_TRANSPOSE_STORES")) {  // tuning and tests
+        a.plain_stores = std::string(env) == "cached";
+    }
     p->workspace_bytes = 0;
-    p->description = std::string("transpose_lds tile=") +
-                     (p->vec_ok && p->elem_size == 2 ? "128x128 " : "64x64 ") +
-                     (p->vec_ok ? "vec16 " : "") +
-                     "batch=" + std::to_string(batch);
+    uint32_t edge_i = 64, edge_o = 64;
+    if (p->vec_ok) vec_shape(p->elem_size, a.n_i, a.n_o, batch, edge_i, edge_o);
+    p->description = "transpose_lds tile=" + std::to_string(edge_i) + "x" + std::to_string(edge_o) +
+                     (p->vec_ok ? " vec16" : "") + (a.plain_stores ? " cached_stores" : "") +
+                     " batch=" + std::to_string(batch);
     return p;
 }
 

@@ -86,3 +86,51 @@ def test_vector_transpose_falls_back_when_a_buffer_is_misaligned(km):
     torch.cuda.synchronize()
     got = dout[3:3 + 72 * 136].cpu().numpy()
     assert_bits_equal(got, np.ascontiguousarray(x.T).reshape(-1), "misaligned transpose")
+
+
+def test_wide_tile_of_4_byte_transposes_with_ragged_edges(km):
+    # enough tiles for the 128 x 64 tile; neither extent is a multiple of the tile
+    shape, perm = (3, 3000, 2008), (0, 2, 1)
+    x = normal(rng(53), int(np.prod(shape)), np.float32).reshape(shape)
+    e = permute_einsummable(shape, perm, "f32")
+    got = run_einsummable(km, e, [x])
+    assert "tile=128x64 vec16 cached_stores" in km.describe(e), km.describe(e)
+    want = np.ascontiguousarray(np.transpose(x, perm)).reshape(-1)
+    assert_bits_equal(got, want, "permute %s %s" % (shape, perm))
+
+
+def test_transpose_beyond_a_gibibyte_takes_the_long_tile(km):
+    import torch
+    from helpers import stream_handle
+
+    # 2-byte elements: 256 x 64 tile; 23176 x 23176 is just past 1 GiB in + out, ragged
+    n_a, n_b = 23176, 23184
+    e = permute_einsummable((n_a, n_b), (1, 0), "f16")
+    km.build(e)
+    d = km.describe(e)
+    assert "tile=256x64 vec16 cached_stores" in d, d
+    g = torch.Generator(device="cuda").manual_seed(54)
+    x = torch.randint(0, 1 << 15, (n_a, n_b), device="cuda", dtype=torch.int16, generator=g)
+    y = torch.full((n_b, n_a), -1, device="cuda", dtype=torch.int16)
+    km(e, stream_handle(), y.data_ptr(), [x.data_ptr()])
+    torch.cuda.synchronize()
+    assert torch.equal(y, x.t())
+
+
+@pytest.mark.parametrize("stores", ["stream", "cached"])
+@pytest.mark.parametrize("dt,npdt,tile", [("f16", np.float16, "256x64"), ("f32", np.float32, "128x64")])
+def test_long_tiles_forced_on_small_ragged_transposes(monkeypatch, dt, npdt, tile, stores):
+    # the switches are read when a plan is made: a manager of its own, so that no plan made
+    # under them stays in the session's manager
+    monkeypatch.setenv("ES_KM_TRANSPOSE_TILE", "long")
+    monkeypatch.setenv("ES_KM_TRANSPOSE_STORES", stores)
+    km = ea.KernelManager(0)
+    r = rng(55)
+    for shape, perm in [((264, 72), (1, 0)), ((2, 520, 136), (0, 2, 1)), ((8, 3, 776), (2, 1, 0))]:
+        x = normal(r, int(np.prod(shape)), npdt).reshape(shape)
+        e = permute_einsummable(shape, perm, dt)
+        got = run_einsummable(km, e, [x])
+        d = km.describe(e)
+        assert ("tile=%s vec16" % tile) in d and ("cached_stores" in d) == (stores == "cached"), d
+        want = np.ascontiguousarray(np.transpose(x, perm)).reshape(-1)
+        assert_bits_equal(got, want, "permute %s %s" % (shape, perm))
