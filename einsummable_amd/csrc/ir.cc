@@ -535,8 +535,12 @@ einsummable_t einsummable_t::make(std::vector<uint64_t> join_shape,
     for (auto const& inn : inns) top = std::max(top, *std::max_element(inn.begin(), inn.end()));
     int join_rank = std::max(top + 1, out_rank);
     if (join_rank != int(join_shape.size())) throw ir_error("invalid join shape size");
+    // every element count and byte size derived from the shape must fit 64 bits
+    uint64_t total = 1;
     for (uint64_t d : join_shape) {
         if (d == 0) throw ir_error("einsummable: cannot have zero join size");
+        if (d >= (1ull << 58) / total) throw ir_error("einsummable: join shape too large");
+        total *= d;
     }
     for (auto const& inn : inns) {
         std::set<int> uniq(inn.begin(), inn.end());

@@ -194,6 +194,14 @@ class Einsummable:
         self.join_shape = [int(x) for x in join_shape]
         self.inns = [list(map(int, inn)) for inn in inns]
         self.out_rank = int(out_rank)
+        # aggregated modes are numbered in order of first appearance, as the reference's
+        # constructor does (src/einsummable/einsummable.cc:32-93): join_shape is indexed by
+        # the numbers after this step, so inn_shape() must see them too
+        renamed = {}
+        for inn in self.inns:
+            for i, m in enumerate(inn):
+                if m >= self.out_rank:
+                    inn[i] = renamed.setdefault(m, self.out_rank + len(renamed))
         self.join = join
         self.castable = castable
         flat, offs = [], [0]
@@ -276,8 +284,8 @@ def codegen_source(e, compile=False):
     rc = lib.es_km_codegen_source(*e._args, int(compile), ctypes.cast(buf, ctypes.c_void_p),
                                   1 << 16)
     if rc != OK:
-        raise KmError(rc, lib.es_km_last_error(None).decode())
-    return buf.value.decode()
+        raise KmError(rc, lib.es_km_last_error(None).decode("utf-8", "replace"))
+    return buf.value.decode("utf-8", "replace")
 
 
 def scalarop_roundtrip(text):
@@ -288,8 +296,8 @@ def scalarop_roundtrip(text):
     rc = lib.es_km_scalarop_roundtrip(text.encode(), ctypes.cast(buf, ctypes.c_void_p), 8192,
                                       ctypes.byref(od), ctypes.byref(n))
     if rc != OK:
-        raise KmError(rc, lib.es_km_last_error(None).decode())
-    return buf.value.decode(), od.value, n.value
+        raise KmError(rc, lib.es_km_last_error(None).decode("utf-8", "replace"))
+    return buf.value.decode("utf-8", "replace"), od.value, n.value
 
 
 def merge_adjacent_dims(e):
@@ -303,9 +311,9 @@ def merge_adjacent_dims(e):
     buf = ctypes.create_string_buffer(256)
     rc = lib.es_km_merge_adjacent_dims(*e._args, js, flat, offs, ctypes.byref(orank), buf, 256)
     if rc < 0:
-        raise KmError(rc, lib.es_km_last_error(None).decode())
+        raise KmError(rc, lib.es_km_last_error(None).decode("utf-8", "replace"))
     inns = [[flat[i] for i in range(offs[k], offs[k + 1])] for k in range(len(e.inns))]
-    return [int(js[i]) for i in range(rc)], inns, orank.value, buf.value.decode()
+    return [int(js[i]) for i in range(rc)], inns, orank.value, buf.value.decode("utf-8", "replace")
 
 
 class KernelManager:
@@ -316,7 +324,7 @@ class KernelManager:
         self._lib = load_library()
         self._h = self._lib.es_km_create(int(device))
         if not self._h:
-            raise KmError(ERR_DEVICE, self._lib.es_km_last_error(None).decode())
+            raise KmError(ERR_DEVICE, self._lib.es_km_last_error(None).decode("utf-8", "replace"))
 
     def close(self):
         if self._h:
@@ -330,7 +338,7 @@ class KernelManager:
             pass
 
     def _fail(self, rc):
-        raise KmError(rc, self._lib.es_km_last_error(self._h).decode())
+        raise KmError(rc, self._lib.es_km_last_error(self._h).decode("utf-8", "replace"))
 
     def build(self, e):
         """Workspace bytes, or None when unsupported (the reference returns nullopt)."""
@@ -354,7 +362,7 @@ class KernelManager:
         rc = self._lib.es_km_describe(self._h, *e._args, ctypes.cast(buf, ctypes.c_void_p), 256)
         if rc != OK:
             self._fail(rc)
-        return buf.value.decode()
+        return buf.value.decode("utf-8", "replace")
 
     def __call__(self, e, stream, out, inns, workspace=None):
         ptrs = (ctypes.c_void_p * max(len(inns), 1))(*inns)
@@ -423,7 +431,7 @@ class ApplyGraph:
     def _check(self, rc):
         if rc < 0:
             h = self._km._h if self._km is not None else None
-            raise KmError(rc, self._lib.es_km_last_error(h).decode())
+            raise KmError(rc, self._lib.es_km_last_error(h).decode("utf-8", "replace"))
         return rc
 
     @staticmethod
@@ -551,7 +559,7 @@ def memgraph_describe(wire):
     wire = bytes(wire)
     n = lib.es_km_memgraph_describe(wire, len(wire), None, 0)
     if n < 0:
-        raise KmError(int(n), lib.es_km_last_error(None).decode())
+        raise KmError(int(n), lib.es_km_last_error(None).decode("utf-8", "replace"))
     buf = ctypes.create_string_buffer(int(n) + 1)
     lib.es_km_memgraph_describe(wire, len(wire), buf, int(n) + 1)
-    return buf.value.decode()
+    return buf.value.decode("utf-8", "replace")

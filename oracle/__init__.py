@@ -138,9 +138,19 @@ def einsummable(join_shape, inns, out_rank, join, castable, inputs, mode=EXACT):
     """Run the interpreter; returns a flat array of the join's output dtype."""
     od, hole_dts = scalarop_info(join)
     arrs = [np.ascontiguousarray(x, dtype=NP_DTYPES[dt]) for x, dt in zip(inputs, hole_dts)]
-    for k, (a, inn) in enumerate(zip(arrs, inns)):
-        # modes are renumbered by first appearance, sizes follow the given join_shape
-        pass
+    # aggregated modes are renumbered by first appearance (einsummable.cc:32-93); sizes
+    # follow join_shape under the new numbers, and every input must hold exactly that many
+    renamed = {}
+    for a, inn in zip(arrs, inns):
+        n = 1
+        for m in inn:
+            if m >= out_rank:
+                m = renamed.setdefault(m, out_rank + len(renamed))
+            if 0 <= m < len(join_shape):
+                n *= int(join_shape[m])
+        if a.size != n:
+            raise ValueError("input of %d elements where modes %s of %s need %d"
+                             % (a.size, list(inn), list(join_shape), n))
     flat, offs = _flatten(inns)
     n_out = int(np.prod([join_shape[i] for i in range(out_rank)], dtype=np.int64))
     out = np.empty(n_out, dtype=NP_DTYPES[od])

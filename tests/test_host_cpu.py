@@ -121,6 +121,21 @@ def test_generated_source_is_deterministic_and_keyed_on_structure_not_shape():
     assert a == b  # extents travel as kernel arguments: one compile serves every shape
 
 
+def test_aggregated_modes_are_numbered_by_first_appearance():
+    # einsummable.cc:32-93: "jk,ij" written with j = 2, k = 1 becomes j = 1, k = 2, and
+    # join_shape is read under the new numbers
+    e = E([9, 7, 65], [[2], [1, 0]], 1, "+[hole|f32@0,hole|f32@1]", "+")
+    assert e.inns == [[1], [2, 0]]
+    assert e.inn_shape(0) == [7] and e.inn_shape(1) == [65, 9]
+    js, mi, mo, s = ea.merge_adjacent_dims(e)
+    assert (js, mi, mo) == oracle.merge_adjacent_dims([9, 7, 65], [[2], [1, 0]], 1)
+    with pytest.raises(ValueError, match="need 7"):
+        oracle.einsummable([9, 7, 65], [[2], [1, 0]], 1, e.join, "+",
+                           [np.zeros(65, np.float32), np.zeros(63, np.float32)])
+    with pytest.raises(ea.KmError, match="too large"):
+        ea.codegen_source(E([1 << 40, 1 << 40], [[0, 1]], 2, "hole|f32@0"))
+
+
 def test_descriptor_errors_map_to_codes():
     bad = [
         E([4, 4], [[0, 1]], 1, "hole|f32@0"),                 # aggregation without castable
