@@ -106,13 +106,22 @@ def run_c2(km, steps, warmup):
     for _ in range(warmup):
         for c in calls:
             c()
+    # The timed region carries events around the dominant kernel only (the first node): every
+    # event pair is two more packets between dependent kernels, and the step is what is timed.
+    # The other three nodes get their events in a second pass of the same steps.
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
-        for c, t in zip(calls, timers):
-            t.record(c)
+        timers[0].record(calls[0])
+        for c in calls[1:]:
+            c()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
+    for _ in range(steps):
+        calls[0]()
+        for c, t in zip(calls[1:], timers[1:]):
+            t.record(c)
+    torch.cuda.synchronize()
 
     total_bytes = sum(b for _, _, b in nodes)
     per_node = []
