@@ -109,12 +109,17 @@ def run_c2(km, steps, warmup):
     # The timed region carries events around the dominant kernel only (the first node): every
     # event pair is two more packets between dependent kernels, and the step is what is timed.
     # The other three nodes get their events in a second pass of the same steps.
+    # An event recorded straight after a launch is stamped when the stream reaches it, so the
+    # step closes with one more event: without it the dominant kernel's start stamp falls into
+    # the tail of the step before.
     torch.cuda.synchronize()
+    step_end = torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     for _ in range(steps):
         timers[0].record(calls[0])
         for c in calls[1:]:
             c()
+        step_end.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     for _ in range(steps):
