@@ -198,7 +198,8 @@ struct contraction_plan_t : plan_t {
 
 std::shared_ptr<plan_t> plan_contraction(einsummable_t const& e, int)
 {
-    if (!e.is_contraction()) return nullptr;
+    double alpha = 1.0;
+    if (!e.is_scaled_contraction(alpha)) return nullptr;
     dtype_t const dt = e.out_dtype();
     if (dt == dtype_t::c64) return nullptr;  // complex contractions use the generated kernels
     if (e.inn_dtype(0) != dt || e.inn_dtype(1) != dt) return nullptr;
@@ -317,6 +318,7 @@ std::shared_ptr<plan_t> plan_contraction(einsummable_t const& e, int)
     // against a weight matrix): several workgroups share a tile's k range and a second
     // kernel sums their fp32 partial tiles, which live in the workspace.
     a.splits = 1;
+    a.alpha = alpha;
     p->workspace_bytes = 0;
     a.lin = a.gm.n == 1 && a.gn.n == 1 && a.gk.n == 1 && a.gn.sy[0] == 1 && a.gm.sy[0] > 0 &&
             uint64_t(a.gm.sy[0]) * 256 * dtype_size(dt) < (1ull << 31);
@@ -367,7 +369,8 @@ std::shared_ptr<plan_t> plan_contraction(einsummable_t const& e, int)
                      " M=" + std::to_string(M) + " N=" + std::to_string(N) + " K=" +
                      std::to_string(K) + " batch=" + std::to_string(Bt) +
                      (a.splits > 1 ? " split_k=" + std::to_string(a.splits) : "") +
-                     (a.shortk ? " resident_a" : "") + (a.warm_a_bytes ? " warm_operands" : "");
+                     (a.shortk ? " resident_a" : "") + (a.warm_a_bytes ? " warm_operands" : "") +
+                     (alpha != 1.0 ? " scaled" : "");
     return p;
 }
 

@@ -447,6 +447,7 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
         return;
     }
     T* const C = static_cast<T*>(a.C) + boc;
+    typename tr::acc_elem const alpha = typename tr::acc_elem(a.alpha);
     constexpr int STRIP_PITCH = WN * int(sizeof(T)) + 16;
     constexpr int CPR = WN * int(sizeof(T)) / 16;
     wait_loads_and_lds<0>();
@@ -461,7 +462,7 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
             for (int e0 = 0; e0 < tr::NACC; e0 += 4) {
                 quad_t q;
 #pragma unroll
-                for (int t = 0; t != 4; ++t) q[t] = T(acc[i][j][e0 + t]);
+                for (int t = 0; t != 4; ++t) q[t] = T(acc[i][j][e0 + t] * alpha);
                 int n = j * MI + tr::acc_row(e0, lane);
                 *reinterpret_cast<quad_t*>(strip + (lane % MI) * STRIP_PITCH +
                                            n * int(sizeof(T))) = q;
@@ -557,7 +558,8 @@ __global__ __launch_bounds__(256) void gemm_fold_kernel(gemm_args_t a)
     group_offsets(a.gm, m, mo_a, mo_c);
     group_offsets(a.gn, n, no_b, no_c);
     typedef T quad_t __attribute__((ext_vector_type(4)));
-    quad_t out = {T(sum[0]), T(sum[1]), T(sum[2]), T(sum[3])};
+    float const alpha = float(a.alpha);
+    quad_t out = {T(sum[0] * alpha), T(sum[1] * alpha), T(sum[2] * alpha), T(sum[3] * alpha)};
     *reinterpret_cast<quad_t*>(static_cast<T*>(a.C) + boc + mo_c + no_c) = out;
 }
 

@@ -58,6 +58,9 @@ struct gemm_args_t {
     // floor(2^32 / (4 * tiles_n)) + 1 when tile index * 4 * tiles_n < 2^32 (then the high
     // half of tile * magic is the exact quotient), else 0
     uint32_t    group_magic;
+    // every sum is multiplied by this before it is rounded to the output type (1 for a plain
+    // product); split-K partial tiles stay unscaled, the fold applies it
+    double      alpha;
 };
 
 __device__ __forceinline__ void group_offsets(group_t const& g, uint32_t i, int64_t& ox,
@@ -486,6 +489,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(gemm_args_t a)
 
     // epilogue: lane holds, per tile, NACC values: n = acc_row(e, lane), m = lane % MI
     T* const C = static_cast<T*>(a.C) + boc;
+    typename tr::acc_elem const alpha = typename tr::acc_elem(a.alpha);
 #pragma unroll
     for (int i = 0; i != TM; ++i) {
         uint32_t m = tm * BM + wm * WM + i * MI + lane % MI;
@@ -506,7 +510,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(gemm_args_t a)
                             T v[4];
                         } q;
 #pragma unroll
-                        for (int t = 0; t != 4; ++t) q.v[t] = T(acc[i][j][e0 + t]);
+                        for (int t = 0; t != 4; ++t) q.v[t] = T(acc[i][j][e0 + t] * alpha);
                         *reinterpret_cast<quad_t*>(C + mo_c + no_c) = q;
                     }
                 } else {
@@ -516,7 +520,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(gemm_args_t a)
                         if (n < a.N) {
                             int64_t no_b, no_c;
                             group_offsets(a.gn, n, no_b, no_c);
-                            C[mo_c + no_c] = T(acc[i][j][e0 + t]);
+                            C[mo_c + no_c] = T(acc[i][j][e0 + t] * alpha);
                         }
                     }
                 }
@@ -804,6 +808,7 @@ __global__ __launch_bounds__(256) void gemm_fast_kernel(gemm_args_t a)
     slice(nk - 1, std::false_type{});
 
     T* const C = static_cast<T*>(a.C) + boc;
+    typename tr::acc_elem const alpha = typename tr::acc_elem(a.alpha);
     if (a.c_mode == 3) {
         // Wide epilogue: each wave turns MI rows of its tile through a private LDS strip so
         // that the global stores are 16 bytes per lane and whole row segments per wavefront
@@ -821,7 +826,7 @@ __global__ __launch_bounds__(256) void gemm_fast_kernel(gemm_args_t a)
                 for (int e0 = 0; e0 < tr::NACC; e0 += 4) {
                     quad_t q;
 #pragma unroll
-                    for (int t = 0; t != 4; ++t) q[t] = T(acc[i][j][e0 + t]);
+                    for (int t = 0; t != 4; ++t) q[t] = T(acc[i][j][e0 + t] * alpha);
                     int n = j * MI + tr::acc_row(e0, lane);
                     *reinterpret_cast<quad_t*>(strip + (lane % MI) * STRIP_PITCH +
                                                n * int(sizeof(T))) = q;
@@ -869,7 +874,7 @@ __global__ __launch_bounds__(256) void gemm_fast_kernel(gemm_args_t a)
                         typedef T quad_t __attribute__((ext_vector_type(4)));
                         quad_t q;
 #pragma unroll
-                        for (int t = 0; t != 4; ++t) q[t] = T(acc[i][j][e0 + t]);
+                        for (int t = 0; t != 4; ++t) q[t] = T(acc[i][j][e0 + t] * alpha);
                         *reinterpret_cast<quad_t*>(C + mo_c + no_c) = q;
                     }
                 } else {
@@ -879,7 +884,7 @@ __global__ __launch_bounds__(256) void gemm_fast_kernel(gemm_args_t a)
                         if (n < a.N) {
                             int64_t no_b, no_c;
                             group_offsets(a.gn, n, no_b, no_c);
-                            C[mo_c + no_c] = T(acc[i][j][e0 + t]);
+                            C[mo_c + no_c] = T(acc[i][j][e0 + t] * alpha);
                         }
                     }
                 }

@@ -255,6 +255,7 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_shortk_kernel(gemm_args_t a,
     uint32_t const m0 = tm * SK_BM + uint32_t(wm) * 64;
     // A fragments: tile row i, k-step s: row lane % 32, k chunk 2 s + lane / 32
     chunk_t fa[2][8];
+    float const alpha = float(a.alpha);
     {
         T const* const A = static_cast<T const*>(a.A) + boa;
 #pragma unroll
@@ -321,7 +322,7 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_shortk_kernel(gemm_args_t a,
                 for (int e0 = 0; e0 < tr::NACC; e0 += 4) {
                     quad_t q;
 #pragma unroll
-                    for (int u = 0; u != 4; ++u) q[u] = T(acc[i][j][e0 + u]);
+                    for (int u = 0; u != 4; ++u) q[u] = T(acc[i][j][e0 + u] * alpha);
                     int const m = wm * 64 + i * 32 + lane % 32;
                     int const n = wn * 64 + j * 32 + tr::acc_row(e0, lane);
                     *reinterpret_cast<quad_t*>(out + m * SK_OUT_PITCH + n * 2) = q;

@@ -492,6 +492,26 @@ bool scalarop_t::is_mul() const
            is_hole(root.children[1], 1);
 }
 
+bool scalarop_t::is_scaled_mul(double& scale) const
+{
+    auto product = [](node_t const& n) {
+        return n.kind == op_kind::mul &&
+               ((is_hole(n.children[0], 0) && is_hole(n.children[1], 1)) ||
+                (is_hole(n.children[0], 1) && is_hole(n.children[1], 0)));
+    };
+    scale = 1.0;
+    if (product(root)) return true;
+    if (root.kind != op_kind::mul) return false;
+    for (int c = 0; c != 2; ++c) {
+        node_t const& k = root.children[c];
+        if (k.kind == op_kind::constant && k.dtype != dtype_t::c64 && product(root.children[1 - c])) {
+            scale = k.re;
+            return true;
+        }
+    }
+    return false;
+}
+
 bool scalarop_t::is_add() const
 {
     return root.kind == op_kind::add && is_hole(root.children[0], 0) &&
@@ -666,6 +686,12 @@ bool einsummable_t::is_contraction() const
 {
     return inns.size() == 2 && has_aggregation() && !has_broadcast() && castable &&
            castable.value() == castable_t::add && join.is_mul();
+}
+
+bool einsummable_t::is_scaled_contraction(double& scale) const
+{
+    return inns.size() == 2 && has_aggregation() && !has_broadcast() && castable &&
+           castable.value() == castable_t::add && join.is_scaled_mul(scale);
 }
 
 uint64_t einsummable_t::out_nelem() const

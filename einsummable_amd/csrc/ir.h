@@ -89,6 +89,9 @@ struct scalarop_t {
     bool        has_variables() const;
     bool        is_identity() const;  // exactly hole@0
     bool        is_mul() const;       // exactly *[hole@0,hole@1]
+    // *[hole@0,hole@1], or that product times one real constant on either side (holes in
+    // either order); `scale` is the constant, 1 for the plain product
+    bool        is_scaled_mul(double& scale) const;
     bool        is_add() const;       // exactly +[hole@0,hole@1]
 };
 
@@ -117,6 +120,11 @@ struct einsummable_t {
     bool     is_straight_elementwise() const;
     bool     is_permutation() const;
     bool     is_contraction() const;
+    // is_contraction() with is_scaled_mul() in place of is_mul(): a product whose result is
+    // multiplied by a constant once, after the sum (the reference has no such form: it runs
+    // the scale as a node of its own, or passes it as cuTENSOR's alpha,
+    // gpu_kernel_manager.cc:1577-1609)
+    bool     is_scaled_contraction(double& scale) const;
     dtype_t  out_dtype() const { return join.out_dtype(); }
     dtype_t  inn_dtype(int k) const { return join.hole_dtypes[k].value(); }
     uint64_t out_nelem() const;

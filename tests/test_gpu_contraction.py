@@ -283,3 +283,66 @@ def test_resident_lhs_kernel_for_head_dimension_reductions(km, monkeypatch, case
     want = oracle_einsummable(sub, [np.ascontiguousarray(L).reshape(-1),
                                     np.ascontiguousarray(R).reshape(-1)], oracle.WIDE)
     assert_close(np.ascontiguousarray(got).reshape(-1), want, DT["f16"], what=spec)
+
+
+def scaled(spec, sizes, dt, const, form=0):
+    c = "constant{%s|%s}" % (dt, const)
+    prod = ["*[hole|%s@0,hole|%s@1]", "*[hole|%s@1,hole|%s@0]"][form & 1] % (dt, dt)
+    join = ("*[%s,%s]" % (c, prod)) if form < 2 else ("*[%s,%s]" % (prod, c))
+    return E.from_str(spec, sizes, join, "+")
+
+
+SCALED_CASES = [
+    # (spec, sizes, dtype, constant, what it must run on); the constant is the attention
+    # scale 1/sqrt(128) as the reference prints it (six digits, then rounded to the dtype)
+    ("bid,bjd->bij", dict(b=130, i=1000, j=1016, d=128), "f16", "0.0883789", "resident_a"),
+    ("bid,bjd->bij", dict(b=3, i=136, j=264, d=128), "f16", "0.0883789", "direct_to_lds"),
+    ("ij,kj->ik", dict(i=8, j=2048, k=264), "f16", "0.0883789", "split_k="),
+    ("ij,jk->ik", dict(i=130, j=264, k=136), "f32", "0.0883883", "C=wide"),
+    ("ij,jk->ik", dict(i=130, j=256, k=136), "f32", "0.0883883", "direct_to_lds"),
+    ("ij,kj->ik", dict(i=130, j=1008, k=136), "f32", "-2.5", "split_k="),
+    ("ij,jk->ik", dict(i=37, j=51, k=29), "f16", "0.0883789", "A=elem"),
+    ("ji,jk->ik", dict(i=64, j=96, k=80), "f64", "0.3", "contraction_mfma_f64"),
+]
+
+
+@pytest.mark.parametrize("case", range(len(SCALED_CASES)))
+def test_product_times_a_constant_is_one_contraction(km, case):
+    spec, sizes, dt, const, path = SCALED_CASES[case]
+    for form in range(4 if case == 1 else 1):
+        e = scaled(spec, sizes, dt, const, form)
+        r = rng(70 + case)
+        xs = [normal(r, int(np.prod(e.inn_shape(k))), NP[DT[dt]]) for k in range(2)]
+        got = run_einsummable(km, e, xs)
+        d = km.describe(e)
+        assert d.startswith("contraction_mfma_" + dt) and path in d and d.endswith(" scaled"), d
+        if case == 0:
+            # a slice against the oracle, and the whole against the unscaled product times
+            # the constant in fp32 (one rounding apart at most)
+            L = xs[0].reshape(130, 1000, 128)[-1:, -136:, :]
+            R = xs[1].reshape(130, 1016, 128)[-1:, -264:, :]
+            sub = scaled(spec, dict(b=1, i=136, j=264, d=128), dt, const, form)
+            want = oracle_einsummable(sub, [np.ascontiguousarray(L).reshape(-1),
+                                            np.ascontiguousarray(R).reshape(-1)], oracle.WIDE)
+            part = got.reshape(130, 1000, 1016)[-1:, -136:, -264:]
+            assert_close(np.ascontiguousarray(part).reshape(-1), want, DT[dt], what=spec)
+            plain = run_einsummable(km, contraction(spec, sizes, dt), xs).astype(np.float32)
+            assert_close(got, plain * np.float32(np.float16(float(const))), DT[dt], what="scaled")
+        else:
+            want = oracle_einsummable(e, xs, oracle.WIDE)
+            assert_close(got, want, DT[dt], what="%s %s [%s]" % (spec, e.join, d))
+
+
+def test_scale_of_one_and_swapped_holes_are_the_plain_product(km):
+    sizes = dict(i=136, j=256, k=72)
+    r = rng(80)
+    xs = [normal(r, 136 * 256, np.float16), normal(r, 256 * 72, np.float16)]
+    plain = run_einsummable(km, contraction("ij,jk->ik", sizes, "f16"), xs)
+    swapped = E.from_str("ij,jk->ik", sizes, "*[hole|f16@1,hole|f16@0]", "+")
+    got = run_einsummable(km, swapped, xs)
+    assert km.describe(swapped).startswith("contraction_mfma_f16")
+    np.testing.assert_array_equal(got.view(np.uint16), plain.view(np.uint16))
+    one = scaled("ij,jk->ik", sizes, "f16", "1")
+    got = run_einsummable(km, one, xs)
+    assert not km.describe(one).endswith(" scaled")
+    np.testing.assert_array_equal(got.view(np.uint16), plain.view(np.uint16))
