@@ -372,6 +372,39 @@ def run_c4(km, steps, warmup):
                      hbm_frac=round(work / ms / 1e6 / HBM_PEAK_GBPS, 4))
         rows.append(r)
     rows.append({"node": "c4 whole chain (7 nodes, no per-node events)", "ms": round(chain_ms, 4)})
+    # The same chain with the scale folded into the scores contraction (one node fewer and
+    # one pass over the 1 GiB score tensor less): the constant multiplies the fp32 sums
+    # before the single rounding to fp16.
+    import einsummable_amd as ea
+
+    folded = ea.Einsummable([b, h, s, s, d], [[0, 1, 2, 4], [0, 1, 3, 4]], 4,
+                            "*[constant{f16|0.0883789},*[hole|f16@0,hole|f16@1]]", "+")
+    assert km.build(folded) == 0
+    first = lambda: km(folded, stream, mem["S"].data_ptr(), [mem["Q"].data_ptr(), mem["K"].data_ptr()])
+    calls6 = [first] + calls[2:]
+    t_first = Timed()
+    for _ in range(warmup):
+        for c in calls6:
+            c()
+    torch.cuda.synchronize()
+    for _ in range(steps):
+        t_first.record(first)
+        for c in calls6[1:]:
+            c()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        for c in calls6:
+            c()
+    torch.cuda.synchronize()
+    chain6_ms = (time.perf_counter() - t0) / steps * 1e3
+    ms = t_first.mean_ms()
+    flop = nodes[0][4]
+    rows.append({"node": "c4 scores with the scale folded in", "kernel": km.describe(folded),
+                 "ms": round(ms, 5), "flop": flop, "TFLOPs": round(flop / ms / 1e9, 2),
+                 "mfma_frac": round(flop / ms / 1e9 / PEAK_TFLOPS["f16"], 4)})
+    rows.append({"node": "c4 whole chain, scale folded into the scores contraction (6 nodes)",
+                 "ms": round(chain6_ms, 4)})
     return rows
 
 
