@@ -128,6 +128,18 @@ def run_c2(km, steps, warmup):
             t.record(c)
     torch.cuda.synchronize()
 
+    # nodes (iii) and (iv) as the one fused einsummable ab,a->a: sum_b exp(x[a,b] - m[a])
+    import einsummable_amd as ea
+
+    fused = ea.Einsummable([n, n], [[0, 1], [0]], 1, EXP_SUB, "+")
+    assert km.build(fused) == 0
+    t_fused = Timed()
+    for _ in range(warmup):
+        km(fused, stream, s.data_ptr(), [x.data_ptr(), m.data_ptr()])
+    for _ in range(steps):
+        t_fused.record(lambda: km(fused, stream, s.data_ptr(), [x.data_ptr(), m.data_ptr()]))
+    torch.cuda.synchronize()
+
     total_bytes = sum(b for _, _, b in nodes)
     per_node = []
     for (name, e, nbytes), t in zip(nodes, timers):
@@ -135,6 +147,11 @@ def run_c2(km, steps, warmup):
         per_node.append({"node": name, "kernel": km.describe(e), "bytes": nbytes,
                          "ms": round(ms, 5), "GBps": round(nbytes / ms / 1e6, 1),
                          "hbm_frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4)})
+    fb, fms = n * n * 2 + 2 * n * 2, t_fused.mean_ms()
+    per_node.append({"node": "(iii)+(iv) fused ij,i->i sum exp(x-rowmax) [not part of the step]",
+                     "kernel": km.describe(fused), "bytes": fb, "ms": round(fms, 5),
+                     "GBps": round(fb / fms / 1e6, 1),
+                     "hbm_frac": round(fb / fms / 1e6 / HBM_PEAK_GBPS, 4)})
     return {"wall_s": wall, "bytes_per_step": total_bytes, "per_node": per_node,
             "tensors": (x, y, m)}
 
@@ -405,6 +422,43 @@ def run_c4(km, steps, warmup):
                  "mfma_frac": round(flop / ms / 1e9 / PEAK_TFLOPS["f16"], 4)})
     rows.append({"node": "c4 whole chain, scale folded into the scores contraction (6 nodes)",
                  "ms": round(chain6_ms, 4)})
+    # And with the softmax in the fused forms the reference's GPU manager special-cases
+    # (gpu_kernel_manager.cc:327-336, 377-405): row max, ab,a->a sum exp(x - m), then
+    # ab,a,a->ab exp(x - m) / l -- five nodes, 4 GiB of softmax traffic instead of 6.
+    rows_n = b * h * s
+    sumexp = ea.Einsummable([rows_n, s], [[0, 1], [0]], 1, EXP_SUB, "+")
+    norm = ea.Einsummable([rows_n, s], [[0, 1], [0], [0]], 2,
+                          "*[exp[+[hole|f16@0,*[constant{f16|-1},hole|f16@1]]],power{-1}[hole|f16@2]]")
+    assert km.build(sumexp) == 0 and km.build(norm) == 0
+    P = lambda k: mem[k].data_ptr()
+    calls5 = [first, calls[2],
+              lambda: km(sumexp, stream, P("l"), [P("S"), P("m")]),
+              lambda: km(norm, stream, P("S"), [P("S"), P("m"), P("l")]),
+              calls[6]]
+    t5 = [Timed() for _ in calls5]
+    for _ in range(warmup):
+        for c in calls5:
+            c()
+    torch.cuda.synchronize()
+    for _ in range(steps):
+        for c, t in zip(calls5, t5):
+            t.record(c)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        for c in calls5:
+            c()
+    torch.cuda.synchronize()
+    chain5_ms = (time.perf_counter() - t0) / steps * 1e3
+    mat = rows_n * s * 2
+    for name, e, t, nbytes in (("c4 sum exp(x - m) ab,a->a", sumexp, t5[2], mat + 2 * rows_n * 2),
+                               ("c4 exp(x - m) / l ab,a,a->ab", norm, t5[3], 2 * mat + 2 * rows_n * 2)):
+        ms = t.mean_ms()
+        rows.append({"node": name, "kernel": km.describe(e), "ms": round(ms, 5), "bytes": nbytes,
+                     "GBps": round(nbytes / ms / 1e6, 1),
+                     "hbm_frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4)})
+    rows.append({"node": "c4 whole chain, scale folded and softmax in the fused forms (5 nodes)",
+                 "ms": round(chain5_ms, 4)})
     return rows
 
 
@@ -654,7 +708,7 @@ def main():
     c2 = run_c2(km, args.steps, args.warmup)
     ms_per_step = c2["wall_s"] / args.steps * 1e3
     value = c2["bytes_per_step"] / (c2["wall_s"] / args.steps) / 1e9
-    dom = max(c2["per_node"], key=lambda p: p["bytes"])
+    dom = max(c2["per_node"][:4], key=lambda p: p["bytes"])
     roofline = {"bound": "hbm", "kernel": dom["node"] + " [" + dom["kernel"] + "]",
                 "achieved": dom["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                 "frac": round(dom["GBps"] / HBM_PEAK_GBPS, 4),
