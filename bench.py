@@ -343,6 +343,33 @@ def c4_nodes(b, h, s, d):
     ]
 
 
+def c4_fused_nodes(b, h, s, d):
+    """The same attention with the scale folded into the scores contraction (the constant
+    multiplies the fp32 sums before the one rounding to fp16) and the softmax in the fused
+    forms the reference's GPU manager special-cases (gpu_kernel_manager.cc:327-336, 377-405):
+    row max, ab,a->a sum exp(x - m), ab,a,a->ab exp(x - m) / l.  Five nodes, 4 GiB of softmax
+    traffic at the full size instead of 6 plus the 2 GiB of the scale node."""
+    import einsummable_amd as ea
+
+    E = ea.Einsummable
+    full = c4_nodes(b, h, s, d)
+    rows, flops = b * h * s, 2 * b * h * s * s * d
+    mat = rows * s * 2
+    return [
+        ("scores, scale folded in", E([b, h, s, s, d], [[0, 1, 2, 4], [0, 1, 3, 4]], 4,
+                                      "*[constant{f16|0.0883789},*[hole|f16@0,hole|f16@1]]", "+"),
+         "S", ["Q", "K"], flops, "flop"),
+        full[2],
+        ("sum exp(x - m) ab,a->a", E([rows, s], [[0, 1], [0]], 1, EXP_SUB, "+"), "l", ["S", "m"],
+         mat + 2 * rows * 2, "B"),
+        ("exp(x - m) / l ab,a,a->ab",
+         E([rows, s], [[0, 1], [0], [0]], 2,
+           "*[exp[+[hole|f16@0,*[constant{f16|-1},hole|f16@1]]],power{-1}[hole|f16@2]]"),
+         "S", ["S", "m", "l"], 2 * mat + 2 * rows * 2, "B"),
+        full[6],
+    ]
+
+
 def run_c4(km, steps, warmup):
     """C4: b=4, h=32, s=2048, d=128, f16 with fp32 accumulation.  The elementwise nodes write
     over their first input (the engine donates it), so the 1 GiB score tensor exists once."""
@@ -422,19 +449,12 @@ def run_c4(km, steps, warmup):
                  "mfma_frac": round(flop / ms / 1e9 / PEAK_TFLOPS["f16"], 4)})
     rows.append({"node": "c4 whole chain, scale folded into the scores contraction (6 nodes)",
                  "ms": round(chain6_ms, 4)})
-    # And with the softmax in the fused forms the reference's GPU manager special-cases
-    # (gpu_kernel_manager.cc:327-336, 377-405): row max, ab,a->a sum exp(x - m), then
-    # ab,a,a->ab exp(x - m) / l -- five nodes, 4 GiB of softmax traffic instead of 6.
-    rows_n = b * h * s
-    sumexp = ea.Einsummable([rows_n, s], [[0, 1], [0]], 1, EXP_SUB, "+")
-    norm = ea.Einsummable([rows_n, s], [[0, 1], [0], [0]], 2,
-                          "*[exp[+[hole|f16@0,*[constant{f16|-1},hole|f16@1]]],power{-1}[hole|f16@2]]")
-    assert km.build(sumexp) == 0 and km.build(norm) == 0
-    P = lambda k: mem[k].data_ptr()
-    calls5 = [first, calls[2],
-              lambda: km(sumexp, stream, P("l"), [P("S"), P("m")]),
-              lambda: km(norm, stream, P("S"), [P("S"), P("m"), P("l")]),
-              calls[6]]
+    # And with the softmax in the fused forms as well: five nodes.
+    fused = c4_fused_nodes(b, h, s, d)
+    for _, e, *_r in fused:
+        assert km.build(e) == 0
+    calls5 = [lambda e=e, o=o, i=i: km(e, stream, mem[o].data_ptr(), [mem[x].data_ptr() for x in i])
+              for _, e, o, i, _w, _u in fused]
     t5 = [Timed() for _ in calls5]
     for _ in range(warmup):
         for c in calls5:
@@ -450,12 +470,10 @@ def run_c4(km, steps, warmup):
             c()
     torch.cuda.synchronize()
     chain5_ms = (time.perf_counter() - t0) / steps * 1e3
-    mat = rows_n * s * 2
-    for name, e, t, nbytes in (("c4 sum exp(x - m) ab,a->a", sumexp, t5[2], mat + 2 * rows_n * 2),
-                               ("c4 exp(x - m) / l ab,a,a->ab", norm, t5[3], 2 * mat + 2 * rows_n * 2)):
+    for (name, e, _o, _i, nbytes, _u), t in list(zip(fused, t5))[2:4]:
         ms = t.mean_ms()
-        rows.append({"node": name, "kernel": km.describe(e), "ms": round(ms, 5), "bytes": nbytes,
-                     "GBps": round(nbytes / ms / 1e6, 1),
+        rows.append({"node": "c4 " + name, "kernel": km.describe(e), "ms": round(ms, 5),
+                     "bytes": nbytes, "GBps": round(nbytes / ms / 1e6, 1),
                      "hbm_frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4)})
     rows.append({"node": "c4 whole chain, scale folded and softmax in the fused forms (5 nodes)",
                  "ms": round(chain5_ms, 4)})

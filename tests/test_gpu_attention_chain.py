@@ -14,8 +14,9 @@ from helpers import assert_close, normal, rng, stream_handle, to_device
 pytestmark = pytest.mark.gpu
 
 
+@pytest.mark.parametrize("chain", ["c4_nodes", "c4_fused_nodes"])
 @pytest.mark.parametrize("b,h,s,d", [(1, 2, 136, 128), (2, 3, 72, 64)])
-def test_attention_chain_matches_oracle(km, b, h, s, d):
+def test_attention_chain_matches_oracle(km, b, h, s, d, chain):
     import torch
 
     r = rng(40)
@@ -25,7 +26,7 @@ def test_attention_chain_matches_oracle(km, b, h, s, d):
     host["m"] = np.zeros(b * h * s, np.float16)
     host["l"] = np.zeros(b * h * s, np.float16)
     dev = {k: to_device(v.copy()) for k, v in host.items()}
-    nodes = bench.c4_nodes(b, h, s, d)
+    nodes = getattr(bench, chain)(b, h, s, d)
     # bench.c4_nodes carries 1/sqrt(128) as the reference prints it; the chain is linear in
     # it up to the softmax, so the same constant is right for the parity check at any d
     for name, e, out, inns, _w, _u in nodes:

@@ -125,7 +125,8 @@ def test_c3a_permute_512_mib_and_its_inverse(km):
     assert torch.equal(y.view(torch.int16), x.permute(0, 2, 1, 3).contiguous().view(torch.int16))
 
 
-def test_c4_attention_chain_b4_h32_s2048_d128(km):
+@pytest.mark.parametrize("chain", ["c4_nodes", "c4_fused_nodes"])
+def test_c4_attention_chain_b4_h32_s2048_d128(km, chain):
     import torch
 
     b, h, s, d = 4, 32, 2048, 128
@@ -136,7 +137,7 @@ def test_c4_attention_chain_b4_h32_s2048_d128(km):
     mem["O"] = torch.empty(b, h, s, d, device="cuda", dtype=torch.float16)
     mem["m"] = torch.empty(b * h * s, device="cuda", dtype=torch.float16)
     mem["l"] = torch.empty(b * h * s, device="cuda", dtype=torch.float16)
-    nodes = bench.c4_nodes(b, h, s, d)
+    nodes = getattr(bench, chain)(b, h, s, d)
     heads = [(0, 0), (1, 17), (3, 31)]
     scores = {}
     for name, e, out, inns, _w, _u in nodes:
@@ -152,12 +153,14 @@ def test_c4_attention_chain_b4_h32_s2048_d128(km):
     for bh in heads:
         Q, K, V = (mem[k][bh].cpu().numpy().astype(np.float64) for k in ("Q", "K", "V"))
         logits = Q @ K.T
+        if chain == "c4_fused_nodes":       # its first node already holds the scaled logits
+            logits = logits * float(np.float16(0.0883789))
         got = scores[bh].astype(np.float64)
         scale = np.sqrt(np.mean(logits * logits))
         assert np.max(np.abs(got - logits) / np.maximum(np.abs(logits), scale)) <= 1e-2
         # the head end to end against double precision: every intermediate of the chain is
         # an fp16 tensor (unit round-off 4.9e-4), so individual outputs carry a few of those
-        z = logits * 0.0883789
+        z = logits * 0.0883789 if chain == "c4_nodes" else logits
         p = np.exp(z - z.max(axis=1, keepdims=True))
         want = (p / p.sum(axis=1, keepdims=True)) @ V
         out = mem["O"][bh].cpu().numpy().astype(np.float64)
