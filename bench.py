@@ -179,6 +179,71 @@ def cpu_baseline_c2(rows=8192):
                 "all 8192 rows" if rows == 8192 else "first %d of 8192 rows" % rows, dt)}
 
 
+def cpu_baselines_other_configs():
+    """Bounded samples of the other configurations on the host: the CPU oracle on one core
+    (kind "port") and, for the f32 matmul, the host BLAS behind torch.matmul on all the
+    threads torch uses (the reference's CPU manager calls MKL's sgemm there,
+    kernel_executor.cc:1293-1449).  A few seconds in all."""
+    import numpy as np
+    import torch
+
+    import oracle
+
+    out = {}
+    r = np.random.RandomState(1)
+    # C1: 64 of the 2048 rows of A through the oracle; the whole product through the BLAS
+    n, rows = 2048, 64
+    A = r.uniform(-1, 1, (n, n)).astype(np.float32)
+    B = r.uniform(-1, 1, (n, n)).astype(np.float32)
+    t0 = time.perf_counter()
+    oracle.einsummable([rows, n, n], [[0, 2], [2, 1]], 2, "*[hole|f32@0,hole|f32@1]", "+",
+                       [A[:rows].copy(), B], oracle.EXACT)
+    dt = time.perf_counter() - t0
+    out["c1_oracle"] = {"value": round(2 * rows * n * n / dt / 1e12, 5), "unit": "TFLOP/s",
+                        "cores": 1, "kind": "port",
+                        "sample": "%d of 2048 rows of A, %.1f s" % (rows, dt)}
+    ta, tb = torch.from_numpy(A), torch.from_numpy(B)
+    torch.matmul(ta, tb)
+    t0 = time.perf_counter()
+    for _ in range(3):
+        torch.matmul(ta, tb)
+    dt = (time.perf_counter() - t0) / 3
+    out["c1_host_blas"] = {"value": round(2 * n ** 3 / dt / 1e12, 4), "unit": "TFLOP/s",
+                           "cores": torch.get_num_threads(), "kind": "host_blas",
+                           "sample": "whole 2048^3 product, torch.matmul on the host, %.3f s" % dt}
+    # C3a: 2 of the 32 outer slices of the permute
+    a, b, c, d = 2, 2048, 32, 128
+    x = r.normal(0, 1, a * b * c * d).astype(np.float16)
+    t0 = time.perf_counter()
+    oracle.einsummable([a, c, b, d], [[0, 2, 1, 3]], 4, "hole|f16@0", None, [x], oracle.EXACT)
+    dt = time.perf_counter() - t0
+    out["c3a_oracle"] = {"value": round(2 * x.nbytes / dt / 1e9, 4), "unit": "GB/s", "cores": 1,
+                         "kind": "port", "sample": "2 of 32 outer slices, %.1f s" % dt}
+    # C3b: all 64 touches
+    nn, blk = 4096, 512
+    acc = np.zeros((nn, nn), np.float16)
+    blocks = [r.normal(0, 1, (blk, blk)).astype(np.float16) for _ in range(8)]
+    offs = [(int(r.randint(0, nn - blk + 1)), int(r.randint(0, nn - blk + 1))) for _ in range(64)]
+    t0 = time.perf_counter()
+    for k, (ro, co) in enumerate(offs):
+        oracle.touch([(blk, nn, 0, ro, blk), (blk, nn, 0, co, blk)], "+", acc, blocks[k % 8])
+    dt = time.perf_counter() - t0
+    out["c3b_oracle"] = {"value": round(64 * 3 * blk * blk * 2 / dt / 1e9, 4), "unit": "GB/s",
+                         "cores": 1, "kind": "port", "sample": "all 64 touches, %.2f s" % dt}
+    # C4: the scores contraction of one of the 128 (batch, head) pairs, 128 of its 2048 rows
+    s, dd, si = 2048, 128, 128
+    Q = r.normal(0, 1, (si, dd)).astype(np.float16)
+    K = r.normal(0, 1, (s, dd)).astype(np.float16)
+    t0 = time.perf_counter()
+    oracle.einsummable([si, s, dd], [[0, 2], [1, 2]], 2, "*[hole|f16@0,hole|f16@1]", "+", [Q, K],
+                       oracle.EXACT)
+    dt = time.perf_counter() - t0
+    out["c4_scores_oracle"] = {"value": round(2 * si * s * dd / dt / 1e12, 6), "unit": "TFLOP/s",
+                               "cores": 1, "kind": "port",
+                               "sample": "128 of 2048 rows of one of 128 heads, %.1f s" % dt}
+    return out
+
+
 def run_contraction(km, name, e, shapes, dtype, flops, steps, warmup):
     import torch
 
@@ -748,6 +813,8 @@ def main():
         others["mfma_f16_register_ceiling"] = run_mfma_peak(km)
         others["read_only_1GiB"] = run_read_ceiling(km, args.steps, args.warmup)
         others["column_reductions"] = run_col_reductions(km, args.steps, args.warmup)
+    if args.workload == "all" and not args.no_cpu_baseline:
+        others["cpu_baselines"] = cpu_baselines_other_configs()
     if args.workload in ("llama", "all"):
         others["llama7b_contractions"] = run_llama_contractions(km, max(args.steps // 5, 3),
                                                                 max(args.warmup // 5, 1))
