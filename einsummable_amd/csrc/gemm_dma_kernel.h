@@ -62,22 +62,28 @@ __device__ __forceinline__ void wait_loads_and_lds()
     asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" : : "n"(VM) : "memory");
 }
 
-template <typename T, int BM, int BN, int NS, int AMODE, int BMODE>
+// RB: bytes of k per row per slice, 64 or 128.  With 128 a slice is a whole cache line per
+// row (products that stream a large operand once read it at 5.9 instead of 3.6 TB/s in a
+// stand-alone walk of the same pattern), eight rows per load instruction instead of sixteen,
+// and four k-steps per slice instead of two.
+template <typename T, int BM, int BN, int NS, int AMODE, int BMODE, int RB = DMA_ROW>
 __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
 {
     using tr = traits_t<T>;
     constexpr int MI = tr::MI;
     constexpr int VL = tr::VL;
-    constexpr int RB = DMA_ROW;
     constexpr int BK = RB / int(sizeof(T));
+    constexpr int CPRW = RB / 16;       // 16-byte chunks per row of a slice
+    constexpr int ROWS_PI = 1024 / RB;  // rows per load instruction (operand along k)
     constexpr int STAGE = (BM + BN) * RB;
     constexpr int A_BYTES = BM * RB;
     constexpr int WM = BM / 2, WN = BN / 2;
     constexpr int TM = WM / MI, TN = WN / MI;
     constexpr int STEPS = BK / (tr::KG * VL);
-    // load instructions per thread per slice: one moves 16 rows per wavefront
-    constexpr int NLA = BM / 64, NLB = BN / 64;
-    static_assert(MI == 32 && tr::KG == 2 && STEPS == 2, "layout below assumes 32x32 tiles");
+    // load instructions per thread per slice: one moves 1 KiB per wavefront
+    constexpr int NLA = BM * RB / 4096, NLB = BN * RB / 4096;
+    static_assert(MI == 32 && tr::KG == 2 && (STEPS == 2 || STEPS == 4) && (RB == 64 || RB == 128),
+                  "layout below assumes 32x32 tiles");
     static_assert(BM % 64 == 0 && BN % 64 == 0, "");
     // An operand contiguous along m / n (mode 1) stays [k][m] / [k][n] in LDS: BK rows of
     // BM / BN elements
@@ -150,7 +156,12 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
     // Load instruction i of this wavefront covers rows (4 i + wave) * 16 + lane / 4 of the
     // tile; the lane's LDS slot is chunk lane % 4 of that row and holds global chunk
     // (lane % 4) ^ bits 2..3 of the row = (lane % 4) ^ ((lane / 16) % 4).
-    uint32_t const load_chunk = uint32_t((lane & 3) ^ ((lane >> 4) & 3));
+    // 128-byte rows: rows (4 i + wave) * 8 + lane / 8, slot lane % 8, and the swizzle is bits
+    // 1..3 of the row = (wave % 2) * 4 + lane / 16: sixteen consecutive rows of one k-chunk
+    // (two rows per 64 banks) again cover all banks once.
+    uint32_t const load_chunk =
+        RB == 64 ? uint32_t((lane & 3) ^ ((lane >> 4) & 3))
+                 : uint32_t((lane & 7) ^ (((lane >> 4) & 3) | ((wave & 1) << 2)));
     uint32_t       voa[NLA], vob[NLB];
     // [k][m] / [k][n] rows: the 16-byte chunks of a row are permuted so that the fragment
     // reads (which walk down k for a fixed m / n) spread over the banks; bits of the k row
@@ -163,7 +174,7 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
     for (int i = 0; i != NLA; ++i) {
         int64_t x, y;
         if constexpr (AMODE == 0) {
-            uint32_t r = tm * BM + uint32_t((4 * i + wave) * 16 + lane / 4);
+            uint32_t r = tm * BM + uint32_t((4 * i + wave) * ROWS_PI + lane / CPRW);
             r = r < a.M ? r : a.M - 1;
             group_offsets(a.gm, r, x, y);
             voa[i] = uint32_t(x) * uint32_t(sizeof(T));
@@ -181,7 +192,7 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
     for (int i = 0; i != NLB; ++i) {
         int64_t x, y;
         if constexpr (BMODE == 0) {
-            uint32_t r = tn * BN + uint32_t((4 * i + wave) * 16 + lane / 4);
+            uint32_t r = tn * BN + uint32_t((4 * i + wave) * ROWS_PI + lane / CPRW);
             r = r < a.N ? r : a.N - 1;
             group_offsets(a.gn, r, x, y);
             vob[i] = uint32_t(x) * uint32_t(sizeof(T));
@@ -236,7 +247,7 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
 
     // Fragment of k-step s for MFMA tile row r0 + lane % 32: k-chunk 2 s + lane / 32, found
     // in slot chunk ^ bits 2..3 of the row
-    int const f_sw = (lane >> 2) & 3;
+    int const f_sw = RB == 64 ? (lane >> 2) & 3 : ((lane % MI) >> 1) & 7;
     int       f_off[STEPS];
 #pragma unroll
     for (int s = 0; s != STEPS; ++s) {
@@ -375,14 +386,17 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
         uint32_t       ka = 0, kb = 0;
         if (ISSUE) k_offsets(k_begin + kt + NS, ka, kb);
 #pragma unroll
-        for (int q = 0; q != MMAS; ++q) {
-            int const p = q % PAIRS;
-            tr::mma_sub(acc[p / TN][p % TN], fb[0][p % TN], fa[0][p / TN], q / PAIRS);
+        for (int s = 0; s != STEPS - 1; ++s) {
 #pragma unroll
-            for (int r = q * R0; r != (q + 1) * R0; ++r) {
-                if (r < READS) read_frag(cur, 1, r, fa[1], fb[1]);
+            for (int q = 0; q != MMAS; ++q) {
+                int const p = q % PAIRS;
+                tr::mma_sub(acc[p / TN][p % TN], fb[s & 1][p % TN], fa[s & 1][p / TN], q / PAIRS);
+#pragma unroll
+                for (int r = q * R0; r != (q + 1) * R0; ++r) {
+                    if (r < READS) read_frag(cur, s + 1, r, fa[(s + 1) & 1], fb[(s + 1) & 1]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
-            __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
         for (int q = 0; q != MMAS; ++q) {
@@ -510,19 +524,31 @@ bool gemm_dma_eligible(gemm_args_t const& a)
            a.offsets_fit_32 != 0;
 }
 
-template <typename T, int BM, int BN, int NS, int AMODE, int BMODE>
+// The same with slices of 128 bytes per row: K a whole number of such slices, and every
+// split-K share (the kernel cuts K into shares of its own slices) at least `stages` of them.
+template <typename T>
+bool gemm_dma_wide_eligible(gemm_args_t const& a, uint32_t stages)
+{
+    constexpr uint32_t BK = 128 / sizeof(T);
+    uint32_t const     splits = a.splits > 1 ? a.splits : 1;
+    return gemm_dma_eligible<T>(a) && a.K % BK == 0 && a.K / BK / splits >= stages;
+}
+
+template <typename T, int BM, int BN, int NS, int AMODE, int BMODE, int RB = DMA_ROW>
 void launch_gemm_dma_kernel_mode(gemm_args_t const& a, hipStream_t stream)
 {
     static_assert(NS >= 2 && NS <= 4, "eligibility guarantees four slices");
-    constexpr int lds = NS * (BM + BN) * DMA_ROW;
+    constexpr int lds = NS * (BM + BN) * RB;
     static bool const raised = [] {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_dma_kernel<T, BM, BN, NS, AMODE, BMODE>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        (void)hipFuncSetAttribute(
+            reinterpret_cast<const void*>(&gemm_dma_kernel<T, BM, BN, NS, AMODE, BMODE, RB>),
+            hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         return true;
     }();
     (void)raised;
     dim3 grid(a.tiles_m * a.tiles_n, a.batch, a.splits > 1 ? a.splits : 1);
-    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, NS, AMODE, BMODE>), grid, dim3(256), lds, stream, a);
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, NS, AMODE, BMODE, RB>), grid, dim3(256), lds,
+                       stream, a);
 }
 
 // Second pass of a split-K contraction: C = sum over the splits' partial tiles, in split

@@ -55,6 +55,23 @@ void launch_gemm_f16(int bm, int bn, gemm_args_t const& a, hipStream_t stream)
         if (bm == 128 && bn == 256) return launch_gemm_dma_kernel<T, 128, 256, 4>(a, stream);
         // short reductions: three stages of a small tile keep three workgroups per compute
         // unit, whose loads, matrix work and stores overlap each other
+        if (bm == 128 && bn == 128 && a.wide_slices && a.a_mode == 0 &&
+            gemm_dma_wide_eligible<T>(a, uint32_t(a.wide_slices))) {
+            // a large operand streamed once: whole cache lines per row and slice
+            if (a.b_mode == 0) {
+                if (a.wide_slices == 2) {
+                    launch_gemm_dma_kernel_mode<T, 128, 128, 2, 0, 0, 128>(a, stream);
+                } else {
+                    launch_gemm_dma_kernel_mode<T, 128, 128, 3, 0, 0, 128>(a, stream);
+                }
+            } else if (a.wide_slices == 2) {
+                launch_gemm_dma_kernel_mode<T, 128, 128, 2, 0, 1, 128>(a, stream);
+            } else {
+                launch_gemm_dma_kernel_mode<T, 128, 128, 3, 0, 1, 128>(a, stream);
+            }
+            if (a.splits > 1) launch_gemm_fold<T>(a, stream);
+            return;
+        }
         if (bm == 128 && bn == 128) {
             return a.K < 512 ? launch_gemm_dma_kernel<T, 128, 128, 3>(a, stream)
                              : launch_gemm_dma_kernel<T, 128, 128, 4>(a, stream);

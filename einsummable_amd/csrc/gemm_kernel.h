@@ -58,6 +58,9 @@ struct gemm_args_t {
     // floor(2^32 / (4 * tiles_n)) + 1 when tile index * 4 * tiles_n < 2^32 (then the high
     // half of tile * magic is the exact quotient), else 0
     uint32_t    group_magic;
+    // 0, or the number of stages (2 or 3) of the direct-to-LDS kernel with 128-byte slices:
+    // planned for f16 products bound by the reads of a large operand
+    int         wide_slices;
     // every sum is multiplied by this before it is rounded to the output type (1 for a plain
     // product); split-K partial tiles stay unscaled, the fold applies it
     double      alpha;

@@ -346,3 +346,41 @@ def test_scale_of_one_and_swapped_holes_are_the_plain_product(km):
     got = run_einsummable(km, one, xs)
     assert not km.describe(one).endswith(" scaled")
     np.testing.assert_array_equal(got.view(np.uint16), plain.view(np.uint16))
+
+
+WIDE_SLICE_CASES = [
+    # products bound by the reads of one large operand take 128-byte slices by themselves;
+    # ragged m and n, both layouts of the small operand, a reduction of exactly two slices
+    ("bij,bjd->bid", dict(b=40, i=1000, j=1984, d=120)),
+    ("ij,kj->ik", dict(i=40000, j=1024, k=72)),
+    ("bij,bjd->bid", dict(b=300, i=136, j=128, d=64)),
+    ("abce,aebd->abcd", dict(a=2, b=24, c=520, e=576, d=128)),
+]
+
+
+@pytest.mark.parametrize("stages", ["", "3"])
+@pytest.mark.parametrize("case", range(len(WIDE_SLICE_CASES)))
+def test_whole_cache_line_slices_equal_half_line_slices_bitwise(monkeypatch, case, stages):
+    spec, sizes = WIDE_SLICE_CASES[case]
+    e = contraction(spec, sizes, "f16")
+    r = rng(90 + case)
+    xs = [normal(r, int(np.prod(e.inn_shape(k))), np.float16) for k in range(2)]
+    if stages:
+        monkeypatch.setenv("ES_KM_GEMM_WIDE_SLICES", stages)
+    wide = ea.KernelManager(0)
+    wide.build(e)
+    if stages == "3" and case == 2:
+        assert "slices=128B" not in wide.describe(e)     # two slices cannot fill three stages
+        return
+    assert "slices=128B" in wide.describe(e), wide.describe(e)
+    monkeypatch.setenv("ES_KM_GEMM_WIDE_SLICES", "0")
+    half = ea.KernelManager(0)
+    half.build(e)
+    assert "slices=128B" not in half.describe(e)
+    a = run_einsummable(wide, e, xs)
+    b = run_einsummable(half, e, xs)
+    # the k-steps run in the same order through the same matrix instructions
+    np.testing.assert_array_equal(a.view(np.uint16), b.view(np.uint16))
+    if case == 2:
+        want = oracle_einsummable(e, xs, oracle.WIDE)
+        assert_close(a, want, DT["f16"], what=spec)
