@@ -374,7 +374,9 @@ std::shared_ptr<plan_t> plan_contraction(einsummable_t const& e, int)
                                  ((double(M) * K + double(N) * K + double(M) * N) * elem);
         bool const can = dt == dtype_t::f16 && p->planned_dma && p->bm == 128 && p->bn == 128 &&
                          !a.shortk && a.a_mode == 0;
-        if (can && intensity < 150.0 && a.splits <= 1) a.wide_slices = 2;
+        // (a reduction of a few slices has nothing to pipeline with two stages: 2048 x 2048 x
+        // 128 per head went from 90 to 107 us)
+        if (can && intensity < 150.0 && a.splits <= 1 && K >= 512) a.wide_slices = 2;
         if (const char* env = std::getenv("ES_KM_GEMM_WIDE_SLICES")) {  // tuning and tests
             int const v = std::atoi(env);
             a.wide_slices = can && (v == 2 || v == 3) ? v : 0;

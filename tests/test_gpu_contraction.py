@@ -358,7 +358,7 @@ WIDE_SLICE_CASES = [
 ]
 
 
-@pytest.mark.parametrize("stages", ["", "3"])
+@pytest.mark.parametrize("stages", ["", "2", "3"])
 @pytest.mark.parametrize("case", range(len(WIDE_SLICE_CASES)))
 def test_whole_cache_line_slices_equal_half_line_slices_bitwise(monkeypatch, case, stages):
     spec, sizes = WIDE_SLICE_CASES[case]
@@ -369,8 +369,10 @@ def test_whole_cache_line_slices_equal_half_line_slices_bitwise(monkeypatch, cas
         monkeypatch.setenv("ES_KM_GEMM_WIDE_SLICES", stages)
     wide = ea.KernelManager(0)
     wide.build(e)
-    if stages == "3" and case == 2:
-        assert "slices=128B" not in wide.describe(e)     # two slices cannot fill three stages
+    if stages != "2" and case == 2:
+        # two slices cannot fill three stages, and by itself the planner keeps reductions
+        # this short on half-line slices
+        assert "slices=128B" not in wide.describe(e)
         return
     assert "slices=128B" in wide.describe(e), wide.describe(e)
     monkeypatch.setenv("ES_KM_GEMM_WIDE_SLICES", "0")
