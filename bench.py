@@ -68,6 +68,26 @@ class Timed:
         return sum(a.elapsed_time(b) for a, b in self.pairs) / max(len(self.pairs), 1)
 
 
+SETTLE_MS = 40.0
+
+
+def warm(fn, steps):
+    """Untimed warm-up of the workloads reported under "others": `steps` calls, then more
+    until SETTLE_MS of wall time have gone by.  The device's clocks need some tens of
+    milliseconds of load to settle: the f32 2048^3 product runs at 105 TFLOP/s over its first
+    60 launches after an idle moment and at 127 TFLOP/s from about the 150th on."""
+    import torch
+
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    while (time.perf_counter() - t0) * 1e3 < SETTLE_MS:
+        for _ in range(10):
+            fn()
+        torch.cuda.synchronize()
+
+
 def c2_nodes(n):
     import einsummable_amd as ea
 
@@ -134,8 +154,7 @@ def run_c2(km, steps, warmup):
     fused = ea.Einsummable([n, n], [[0, 1], [0]], 1, EXP_SUB, "+")
     assert km.build(fused) == 0
     t_fused = Timed()
-    for _ in range(warmup):
-        km(fused, stream, s.data_ptr(), [x.data_ptr(), m.data_ptr()])
+    warm(lambda: km(fused, stream, s.data_ptr(), [x.data_ptr(), m.data_ptr()]), warmup)
     for _ in range(steps):
         t_fused.record(lambda: km(fused, stream, s.data_ptr(), [x.data_ptr(), m.data_ptr()]))
     torch.cuda.synchronize()
@@ -263,9 +282,7 @@ def run_contraction(km, name, e, shapes, dtype, flops, steps, warmup):
     stream = torch.cuda.current_stream().cuda_stream
     call = lambda: km(e, stream, out.data_ptr(), [t.data_ptr() for t in ins],
                       (wbuf.data_ptr(), ws) if ws else None)
-    for _ in range(warmup):
-        call()
-    torch.cuda.synchronize()
+    warm(call, warmup)
     t = Timed()
     for _ in range(steps):
         t.record(call)
@@ -300,9 +317,7 @@ def run_c3(km, steps, warmup):
     assert km.build(e) == 0
     stream = torch.cuda.current_stream().cuda_stream
     call = lambda: km(e, stream, y.data_ptr(), [x.data_ptr()])
-    for _ in range(warmup):
-        call()
-    torch.cuda.synchronize()
+    warm(call, warmup)
     t = Timed()
     for _ in range(steps):
         t.record(call)
@@ -321,9 +336,7 @@ def run_c3(km, steps, warmup):
     y = torch.empty_like(x)
     assert km.build(e) == 0
     call = lambda: km(e, stream, y.data_ptr(), [x.data_ptr()])
-    for _ in range(warmup):
-        call()
-    torch.cuda.synchronize()
+    warm(call, warmup)
     t = Timed()
     for _ in range(steps):
         t.record(call)
@@ -348,9 +361,7 @@ def run_c3(km, steps, warmup):
         for tch, bl in zip(touches, blocks):
             km.touch(tch, stream, acc.data_ptr(), bl.data_ptr())
 
-    for _ in range(warmup):
-        all_touches()
-    torch.cuda.synchronize()
+    warm(all_touches, warmup)
     t = Timed()
     for _ in range(steps):
         t.record(all_touches)
@@ -365,9 +376,7 @@ def run_c3(km, steps, warmup):
     batch = ea.TouchBatch(touches)
     ptrs = [bl.data_ptr() for bl in blocks]
     call = lambda: km.touch_batch(batch, stream, acc.data_ptr(), ptrs)
-    for _ in range(warmup):
-        call()
-    torch.cuda.synchronize()
+    warm(call, warmup)
     t = Timed()
     for _ in range(steps):
         t.record(call)
@@ -455,10 +464,7 @@ def run_c4(km, steps, warmup):
     calls = [lambda e=e, o=o, i=i: km(e, stream, mem[o].data_ptr(), [mem[x].data_ptr() for x in i])
              for _, e, o, i, _w, _u in nodes]
     timers = [Timed() for _ in calls]
-    for _ in range(warmup):
-        for c in calls:
-            c()
-    torch.cuda.synchronize()
+    warm(lambda: [c() for c in calls], warmup)
     for _ in range(steps):
         for c, t in zip(calls, timers):
             t.record(c)
@@ -492,10 +498,7 @@ def run_c4(km, steps, warmup):
     first = lambda: km(folded, stream, mem["S"].data_ptr(), [mem["Q"].data_ptr(), mem["K"].data_ptr()])
     calls6 = [first] + calls[2:]
     t_first = Timed()
-    for _ in range(warmup):
-        for c in calls6:
-            c()
-    torch.cuda.synchronize()
+    warm(lambda: [c() for c in calls6], warmup)
     for _ in range(steps):
         t_first.record(first)
         for c in calls6[1:]:
@@ -521,10 +524,7 @@ def run_c4(km, steps, warmup):
     calls5 = [lambda e=e, o=o, i=i: km(e, stream, mem[o].data_ptr(), [mem[x].data_ptr() for x in i])
               for _, e, o, i, _w, _u in fused]
     t5 = [Timed() for _ in calls5]
-    for _ in range(warmup):
-        for c in calls5:
-            c()
-    torch.cuda.synchronize()
+    warm(lambda: [c() for c in calls5], warmup)
     for _ in range(steps):
         for c, t in zip(calls5, t5):
             t.record(c)
@@ -594,9 +594,7 @@ def run_c5(km, steps, warmup):
         if name.endswith("norm.weight"):
             t = t + 1.0
         run.mem[name].copy_(t.half().view(torch.uint8))
-    for _ in range(warmup):
-        run.run()
-    torch.cuda.synchronize()
+    warm(run.run, warmup)
     timers = [Timed() for _ in g.nodes]
     t0 = time.perf_counter()
     for _ in range(steps):
@@ -753,9 +751,7 @@ def run_copy(km, steps, warmup):
     t = ea.Touch([(n, n, 0, 0, n)], None, ea.F16)
     stream = torch.cuda.current_stream().cuda_stream
     call = lambda: km.touch(t, stream, y.data_ptr(), x.data_ptr())
-    for _ in range(warmup):
-        call()
-    torch.cuda.synchronize()
+    warm(call, warmup)
     tm = Timed()
     for _ in range(steps):
         tm.record(call)

@@ -377,11 +377,24 @@ std::shared_ptr<plan_t> plan_contraction(einsummable_t const& e, int)
         // (a reduction of a few slices has nothing to pipeline with two stages: 2048 x 2048 x
         // 128 per head went from 90 to 107 us)
         if (can && intensity < 150.0 && a.splits <= 1 && K >= 512) a.wide_slices = 2;
+        // fp32, at most one tile per compute unit (LDS is then no constraint): four stages of
+        // 128-byte slices halve the barriers per k; 2048^3 with B along n 105.7 -> 121.3
+        // TFLOP/s, with B along k 123.3 -> 125.4.  With more tiles than compute units two
+        // workgroups share one and only two stages fit: 4096^3 141.4 -> 142.8, not taken.
+        bool const can32 = dt == dtype_t::f32 && p->planned_dma && p->bm == 128 && p->bn == 128 &&
+                           a.a_mode == 0;
+        if (can32 && a.splits <= 1 && K >= 512 &&
+            uint64_t(a.tiles_m) * a.tiles_n * uint64_t(a.batch) <= 256) {
+            a.wide_slices = 4;
+        }
         if (const char* env = std::getenv("ES_KM_GEMM_WIDE_SLICES")) {  // tuning and tests
             int const v = std::atoi(env);
-            a.wide_slices = can && (v == 2 || v == 3) ? v : 0;
+            a.wide_slices = ((can && (v == 2 || v == 3)) || (can32 && v >= 2 && v <= 4)) ? v : 0;
         }
-        if (a.wide_slices && !gemm::gemm_dma_wide_eligible<_Float16>(a, uint32_t(a.wide_slices))) {
+        if (a.wide_slices &&
+            !(dt == dtype_t::f16
+                  ? gemm::gemm_dma_wide_eligible<_Float16>(a, uint32_t(a.wide_slices))
+                  : gemm::gemm_dma_wide_eligible<float>(a, uint32_t(a.wide_slices)))) {
             a.wide_slices = 0;
         }
     }

@@ -386,3 +386,29 @@ def test_whole_cache_line_slices_equal_half_line_slices_bitwise(monkeypatch, cas
     if case == 2:
         want = oracle_einsummable(e, xs, oracle.WIDE)
         assert_close(a, want, DT["f16"], what=spec)
+
+
+@pytest.mark.parametrize("spec", ["ij,jk->ik", "ij,kj->ik"])
+@pytest.mark.parametrize("stages", ["", "2", "3"])
+def test_whole_cache_line_slices_fp32(monkeypatch, spec, stages):
+    # at most one tile per compute unit and no split-K: four stages by default
+    sizes = dict(i=1500, j=1056, k=1700)
+    e = contraction(spec, sizes, "f32")
+    r = rng(95)
+    xs = [uniform(r, int(np.prod(e.inn_shape(k))), np.float32) for k in range(2)]
+    monkeypatch.setenv("ES_KM_GEMM_TILE", "128x128")    # 168 tiles: no split-K
+    if stages:
+        monkeypatch.setenv("ES_KM_GEMM_WIDE_SLICES", stages)
+    wide = ea.KernelManager(0)
+    wide.build(e)
+    assert "slices=128B" in wide.describe(e) and "split_k" not in wide.describe(e), wide.describe(e)
+    monkeypatch.setenv("ES_KM_GEMM_WIDE_SLICES", "0")
+    half = ea.KernelManager(0)
+    half.build(e)
+    assert "slices=128B" not in half.describe(e)
+    a = run_einsummable(wide, e, xs)
+    b = run_einsummable(half, e, xs)
+    np.testing.assert_array_equal(a.view(np.uint32), b.view(np.uint32))
+    if not stages:
+        want = oracle_einsummable(e, xs, oracle.WIDE)
+        assert_close(a, want, DT["f32"], what=spec)
