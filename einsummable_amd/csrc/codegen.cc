@@ -639,16 +639,22 @@ cg_kernel_t gen_reduce_row(einsummable_t const& e, int max_vec)
     s << "__device__ __forceinline__ " << ACC << " comb(" << ACC << " x, " << ACC
       << " y) { return " << combine_expr(cast, od, "x", "y") << "; }\n";
     if (split) {
+        // Second pass: one wavefront per output row.  Lane l adds slices l, l + 64, ... and
+        // the 64 sums meet in a fixed butterfly, so the result does not depend on timing (a
+        // thread of its own per row waits for one load after the other: 38 us for the 2048
+        // slices of a single row, as long as the first pass).
         g.k.entry2 = g.k.entry + "_fold";
+        g.k.grid2 = (n_out + 3) / 4;
         s << "extern \"C\" __global__ __launch_bounds__(" << BLOCK << ") void " << g.k.entry2
           << "(args_t a)\n{\n";
-        s << "    const idx_t row = ((idx_t)blockIdx.y * gridDim.x + blockIdx.x) * " << BLOCK
-          << " + threadIdx.x;\n";
+        s << "    const idx_t row = ((idx_t)blockIdx.y * gridDim.x + blockIdx.x) * 4 + threadIdx.x / 64;\n";
         s << "    if (row >= " << g.P(p_nout) << ") return;\n";
         s << "    " << ACC << " acc = " << identity_of(cast, od) << ";\n";
-        s << "    for (unsigned z = 0; z != " << S << "u; ++z) acc = comb(acc, a.ws[(size_t)z * "
+        s << "#pragma unroll 4\n";
+        s << "    for (unsigned z = threadIdx.x % 64; z < " << S << "u; z += 64) acc = comb(acc, a.ws[(size_t)z * "
           << g.P(p_nout) << " + row]);\n";
-        s << "    a.out[row] = " << g.store_cast("acc") << ";\n}\n";
+        s << "#pragma unroll\n    for (int m = 32; m >= 1; m >>= 1) acc = comb(acc, lane_xor(acc, m));\n";
+        s << "    if (threadIdx.x % 64 == 0) a.out[row] = " << g.store_cast("acc") << ";\n}\n";
     }
     s << "extern \"C\" __global__ __launch_bounds__(" << BLOCK << ") void " << g.k.entry << "(args_t a)\n{\n";
     s << "    const idx_t n_out = " << g.P(p_nout) << ";\n";
@@ -841,7 +847,10 @@ cg_kernel_t gen_reduce_col(einsummable_t const& e, int max_vec)
     // (grid z), each leaving partial results in the workspace; a second kernel folds the
     // slices in order, so the result does not depend on scheduling.
     uint64_t const outer = L.shape[O];
-    uint64_t const want_threads = 1ull << 16;  // measured: 32-64 K threads with 4 rows in flight each
+    // measured with the slice-parallel fold below: 128 K threads with 4 rows in flight each
+    // (8192 x 8192 f16: 4.2 TB/s with 64 K, 4.6 with 128 K, 4.9 with 256 K, where 2048 x 4096
+    // f32 and 64 x 2048 x 1024 f16 lose 6-9 %)
+    uint64_t const want_threads = 1ull << 17;
     uint64_t       S = 1;
     if (n_vec * 2 <= want_threads && outer >= 16) {
         S = std::min<uint64_t>({(want_threads + n_vec - 1) / n_vec, outer / 8, 1024});
@@ -875,19 +884,32 @@ cg_kernel_t gen_reduce_col(einsummable_t const& e, int max_vec)
     s << "__device__ __forceinline__ " << ACC << " comb(" << ACC << " x, " << ACC
       << " y) { return " << combine_expr(cast, od, "x", "y") << "; }\n";
     if (split) {
-        // second pass: fold the slices' partial results, in slice order
+        // Second pass: fold the slices' partial results.  A workgroup owns 16 output vectors;
+        // its 16 groups of lanes each add every 16th slice (a thread of its own per output
+        // would wait for one load after the other: 23 us for 256 slices of 1024 floats), then
+        // group 0 adds the 16 sums in group order, so the result does not depend on timing.
         g.k.entry2 = g.k.entry + "_fold";
+        g.k.grid2 = (n_vec + 15) / 16;
         s << "extern \"C\" __global__ __launch_bounds__(256) void " << g.k.entry2
           << "(args_t a)\n{\n";
-        s << "    const idx_t vid = ((idx_t)blockIdx.y * gridDim.x + blockIdx.x) * 256 + threadIdx.x;\n";
-        s << "    if (vid >= " << g.P(p_nvec) << ") return;\n";
+        s << "    __shared__ " << ACC << " sh[256 * V];\n";
+        s << "    const unsigned vl = threadIdx.x % 16, zl = threadIdx.x / 16;\n";
+        s << "    const idx_t vid = ((idx_t)blockIdx.y * gridDim.x + blockIdx.x) * 16 + vl;\n";
+        s << "    const bool live = vid < " << g.P(p_nvec) << ";\n";
         s << "    " << ACC << " acc[V];\n";
         s << "#pragma unroll\n    for (int j = 0; j != V; ++j) acc[j] = "
           << identity_of(cast, od) << ";\n";
-        s << "    for (unsigned z = 0; z != " << S << "u; ++z) {\n";
-        s << "        const " << ACC << "* part = a.ws + (size_t)z * " << g.P(p_nout)
+        s << "    if (live) {\n";
+        s << "#pragma unroll 4\n        for (unsigned z = zl; z < " << S << "u; z += 16) {\n";
+        s << "            const " << ACC << "* part = a.ws + (size_t)z * " << g.P(p_nout)
           << " + (size_t)vid * V;\n";
-        s << "#pragma unroll\n        for (int j = 0; j != V; ++j) acc[j] = comb(acc[j], part[j]);\n";
+        s << "#pragma unroll\n            for (int j = 0; j != V; ++j) acc[j] = comb(acc[j], part[j]);\n";
+        s << "        }\n    }\n";
+        s << "#pragma unroll\n    for (int j = 0; j != V; ++j) sh[threadIdx.x * V + j] = acc[j];\n";
+        s << "    __syncthreads();\n";
+        s << "    if (zl != 0 || !live) return;\n";
+        s << "    for (unsigned z = 1; z != 16; ++z) {\n";
+        s << "#pragma unroll\n        for (int j = 0; j != V; ++j) acc[j] = comb(acc[j], sh[(z * 16 + vl) * V + j]);\n";
         s << "    }\n";
         s << "    vec_t<" << storage_type(od) << ", V> res;\n";
         s << "#pragma unroll\n    for (int j = 0; j != V; ++j) res.v[j] = "
@@ -1141,6 +1163,10 @@ struct codegen_plan_t : plan_t {
         hipError_t err = hipModuleLaunchKernel(v.fn, gx, gy, unsigned(v.k.splits), v.k.block, 1, 1,
                                                0, stream, nullptr, config);
         if (err == hipSuccess && v.k.splits > 1) {
+            if (v.k.grid2) {
+                gx = unsigned(std::min<uint64_t>(v.k.grid2, gx_max));
+                gy = unsigned((v.k.grid2 + gx - 1) / gx);
+            }
             err = hipModuleLaunchKernel(v.fn2, gx, gy, 1, v.k.block, 1, 1, 0, stream, nullptr,
                                         config);
         }

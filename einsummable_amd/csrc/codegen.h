@@ -34,6 +34,7 @@ struct cg_kernel_t {
     // (grid z) and leave partial results in the workspace, which `entry2` then folds.
     int         splits = 1;
     std::string entry2;
+    uint64_t    grid2 = 0;               // workgroups of `entry2`; 0: the same as `grid`
     uint64_t    ws_bytes = 0;
 };
 
