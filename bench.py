@@ -689,12 +689,14 @@ def run_read_ceiling(km, steps, warmup):
     assert km.build(e) == 0
     stream = torch.cuda.current_stream().cuda_stream
     ours, lib = Timed(), Timed()
-    for i in range(warmup + steps):
-        t = ours if i >= warmup else Timed()
-        t.record(lambda: km(e, stream, m.data_ptr(), [x.data_ptr()]))
-    for i in range(warmup + steps):
-        t = lib if i >= warmup else Timed()
-        t.record(lambda: torch.amax(x, dim=1, out=m))
+    call = lambda: km(e, stream, m.data_ptr(), [x.data_ptr()])
+    warm(call, warmup)
+    for _ in range(steps):
+        ours.record(call)
+    call = lambda: torch.amax(x, dim=1, out=m)
+    warm(call, warmup)
+    for _ in range(steps):
+        lib.record(call)
     torch.cuda.synchronize()
     nbytes = rows * n * 2 + rows * 2
     return {"bytes": nbytes, "es_rowmax_GBps": round(nbytes / ours.mean_ms() / 1e6, 1),
@@ -725,10 +727,11 @@ def run_col_reductions(km, steps, warmup):
         x = torch.randn(n_in, device="cuda", dtype=dt)
         y = torch.empty(n_out, device="cuda", dtype=dt)
         t = Timed()
-        for i in range(warmup + steps):
-            (t if i >= warmup else Timed()).record(
-                lambda: km(e, stream, y.data_ptr(), [x.data_ptr()],
-                           (w.data_ptr(), ws) if ws else None))
+        call = lambda: km(e, stream, y.data_ptr(), [x.data_ptr()],
+                          (w.data_ptr(), ws) if ws else None)
+        warm(call, warmup)
+        for _ in range(steps):
+            t.record(call)
         torch.cuda.synchronize()
         nbytes = (n_in + n_out) * x.element_size()
         rows.append({"node": name, "kernel": km.describe(e), "workspace_bytes": ws,
