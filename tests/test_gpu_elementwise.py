@@ -309,3 +309,49 @@ def test_split_row_reductions(km, case):
     ws = km.build(e)
     assert ws is not None and ws > 0 and "splits=" in km.describe(e), km.describe(e)
     check(km, e, seed=80 + case, exact=exact, sd=0.5)
+
+
+STAGED = [
+    ("ab,ba->ab", dict(a=136, b=72), "+[hole|f16@0,hole|f16@1]"),
+    ("ab,ba->ab", dict(a=33, b=50), "*[hole|f32@0,hole|f32@1]"),                  # ragged: scalar paths
+    ("abc,acb->abc", dict(a=3, b=40, c=24), "*[hole|f16@0,hole|f16@1]"),
+    ("abcd,dcba,ab->abcd", dict(a=4, b=6, c=8, d=16), "+[hole|f32@0,*[hole|f32@1,hole|f32@2]]"),
+    ("ba->ab", dict(a=64, b=48), "*[constant{f16|2},hole|f16@0]"),
+    ("abc,cb->abc", dict(a=5, b=16, c=32), "+[hole|f64@0,hole|f64@1]"),           # transposed and broadcast
+    ("ab,ba,ba->ab", dict(a=40, b=56), "+[hole|c64@0,*[hole|c64@1,hole|c64@2]]"),
+]
+
+
+@pytest.mark.parametrize("case", range(len(STAGED)))
+def test_inputs_with_another_inner_mode_are_transposed_into_the_workspace(monkeypatch, case):
+    spec, sizes, join = STAGED[case]
+    monkeypatch.setenv("ES_KM_EW_STAGE_MIN", "1")       # by itself only from 4 MiB on
+    staged = ea.KernelManager(0)
+    e = E.from_str(spec, sizes, join)
+    ws = staged.build(e)
+    assert ws > 0 and staged.describe(e).startswith("staged ["), staged.describe(e)
+    got = check(staged, e, seed=120 + case)
+    monkeypatch.setenv("ES_KM_EW_STAGE_MIN", "0")
+    direct = ea.KernelManager(0)
+    assert direct.build(e) == 0 and direct.describe(e).startswith("elementwise")
+    # the same arithmetic on the same values, whichever way they were fetched
+    xs = inputs_for(e, rng(120 + case))
+    assert_bits_equal(got, run_einsummable(direct, e, xs), spec)
+
+
+def test_large_transposed_input_is_staged_by_default(km):
+    e = E.from_str("ab,ba->ab", dict(a=2048, b=1536), "+[hole|f16@0,hole|f16@1]")
+    ws = km.build(e)
+    assert ws == 2048 * 1536 * 2 and km.describe(e).startswith("staged ["), km.describe(e)
+    r = rng(130)
+    xs = [normal(r, 2048 * 1536, np.float16) for _ in range(2)]
+    got = run_einsummable(km, e, xs)
+    want = (xs[0].reshape(2048, 1536).astype(np.float32) +
+            xs[1].reshape(1536, 2048).T.astype(np.float32)).astype(np.float16)
+    assert_bits_equal(got, want.reshape(-1), "ab,ba->ab")
+    import torch
+    from helpers import stream_handle
+    d = torch.zeros(16, device="cuda", dtype=torch.float16)
+    with pytest.raises(ea.KmError) as ei:
+        km(e, stream_handle(), d.data_ptr(), [d.data_ptr(), d.data_ptr()])
+    assert ei.value.code == -3
