@@ -325,7 +325,7 @@ STAGED = [
 @pytest.mark.parametrize("case", range(len(STAGED)))
 def test_inputs_with_another_inner_mode_are_transposed_into_the_workspace(monkeypatch, case):
     spec, sizes, join = STAGED[case]
-    monkeypatch.setenv("ES_KM_EW_STAGE_MIN", "1")       # by itself only from 4 MiB on
+    monkeypatch.setenv("ES_KM_EW_STAGE_MIN", "1")       # by itself only from 2 M elements on
     staged = ea.KernelManager(0)
     e = E.from_str(spec, sizes, join)
     ws = staged.build(e)
