@@ -68,6 +68,14 @@ def random_einsummable(r):
     return ea.Einsummable(shape, inns, out_rank, join_for(r, n_inn, dt), castable), dt
 
 
+@pytest.mark.parametrize("seed", [100, 101, 102])
+def test_random_einsummables_with_every_transposed_input_staged(monkeypatch, seed):
+    # elementwise nodes bring inputs with another inner mode into the output's order through
+    # the workspace, by themselves only when the input is large: here always
+    monkeypatch.setenv("ES_KM_EW_STAGE_MIN", "1")
+    test_random_einsummables_match_the_oracle(ea.KernelManager(0), seed)
+
+
 @pytest.mark.parametrize("seed", range(12))
 def test_random_einsummables_match_the_oracle(km, seed):
     r = random.Random(1000 + seed)
