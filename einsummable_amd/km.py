@@ -1,4 +1,5 @@
 import ctypes
+import sys
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
@@ -322,6 +323,11 @@ class KernelManager:
 
     def __init__(self, device=0):
         self._lib = load_library()
+        # A process that also uses torch for device memory must let torch set the device up
+        # before the library's first HIP call (the other way round torch finds no GPU).
+        torch = sys.modules.get("torch")
+        if torch is not None and torch.cuda.is_available():
+            torch.cuda.init()
         self._h = self._lib.es_km_create(int(device))
         if not self._h:
             raise KmError(ERR_DEVICE, self._lib.es_km_last_error(None).decode("utf-8", "replace"))
