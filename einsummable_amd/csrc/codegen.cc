@@ -10,8 +10,13 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <future>
+#include <map>
 #include <mutex>
 #include <sstream>
+
+#include <sys/stat.h>
+#include <unistd.h>
 
 namespace es
 {
@@ -1068,9 +1073,129 @@ std::vector<char> compile_hip_source(std::string const& source, std::string cons
 namespace
 {
 
+// ---- code objects on disk.  A runtime compile costs a good part of a second per kernel, and
+// a server process builds the same einsummables every time it starts.  The code object of a
+// source is kept in a file named by a 128-bit hash of (runtime-compiler version, options,
+// source); the file repeats the length of that text so that a truncated or foreign file is not
+// taken for a hit.  ES_KM_CACHE_DIR names the directory ("off" or "" switches the cache off);
+// by default it is $XDG_CACHE_HOME/es_km or $HOME/.cache/es_km.  Files are written under a
+// temporary name and renamed, so concurrent processes never see half a file.
+
+constexpr char COMPILE_OPTIONS[] = "gfx950 -O3 -std=c++17 -packed-fp32-ops";
+
+std::string cache_dir()
+{
+    const char* env = std::getenv("ES_KM_CACHE_DIR");
+    if (env) {
+        std::string d = env;
+        if (d.empty() || d == "off" || d == "0") return "";
+        return d;
+    }
+    if (const char* x = std::getenv("XDG_CACHE_HOME")) {
+        if (*x) return std::string(x) + "/es_km";
+    }
+    if (const char* h = std::getenv("HOME")) {
+        if (*h) return std::string(h) + "/.cache/es_km";
+    }
+    return "";
+}
+
+uint64_t fnv1a(std::string const& text, uint64_t h)
+{
+    for (unsigned char c : text) {
+        h ^= c;
+        h *= 1099511628211ull;
+    }
+    return h;
+}
+
+std::string cache_text(std::string const& source)
+{
+    int major = 0, minor = 0;
+    hiprtcVersion(&major, &minor);
+    return "hiprtc " + std::to_string(major) + "." + std::to_string(minor) + "\n" +
+           COMPILE_OPTIONS + "\n" + source;
+}
+
+std::string cache_file(std::string const& dir, std::string const& text)
+{
+    char name[64];
+    std::snprintf(name, sizeof(name), "%016llx%016llx.co",
+                  (unsigned long long)fnv1a(text, 14695981039346656037ull),
+                  (unsigned long long)fnv1a(text, 0x9e3779b97f4a7c15ull));
+    return dir + "/" + name;
+}
+
+struct cache_header_t {
+    char     magic[8];  // "ESKMCO1\0"
+    uint64_t text_bytes;
+    uint64_t code_bytes;
+};
+
+bool read_cached(std::string const& path, uint64_t text_bytes, std::vector<char>& code)
+{
+    std::FILE* f = std::fopen(path.c_str(), "rb");
+    if (!f) return false;
+    cache_header_t h;
+    bool           ok = std::fread(&h, sizeof(h), 1, f) == 1 &&
+              std::memcmp(h.magic, "ESKMCO1", 8) == 0 && h.text_bytes == text_bytes &&
+              h.code_bytes > 0 && h.code_bytes < (1ull << 30);
+    if (ok) {
+        code.resize(size_t(h.code_bytes));
+        ok = std::fread(code.data(), 1, code.size(), f) == code.size() && std::fgetc(f) == EOF;
+    }
+    std::fclose(f);
+    return ok;
+}
+
+void write_cached(std::string const& dir, std::string const& path, uint64_t text_bytes,
+                  std::vector<char> const& code)
+{
+    // failures only mean that the next process compiles again
+    for (size_t at = dir.find('/', 1); at != std::string::npos; at = dir.find('/', at + 1)) {
+        ::mkdir(dir.substr(0, at).c_str(), 0755);
+    }
+    ::mkdir(dir.c_str(), 0755);
+    std::string tmp = path + ".tmp" + std::to_string(long(::getpid()));
+    std::FILE*  f = std::fopen(tmp.c_str(), "wb");
+    if (!f) return;
+    cache_header_t h;
+    std::memcpy(h.magic, "ESKMCO1", 8);
+    h.text_bytes = text_bytes;
+    h.code_bytes = code.size();
+    bool ok = std::fwrite(&h, sizeof(h), 1, f) == 1 &&
+              std::fwrite(code.data(), 1, code.size(), f) == code.size();
+    ok = (std::fclose(f) == 0) && ok;
+    if (!ok || std::rename(tmp.c_str(), path.c_str()) != 0) std::remove(tmp.c_str());
+}
+
+}  // namespace
+
+std::vector<char> code_object_for(std::string const& source, bool* from_disk)
+{
+    if (from_disk) *from_disk = false;
+    std::string const dir = cache_dir();
+    if (dir.empty()) return compile_hip_source(source, "es_generated.hip", "gfx950");
+    std::string const text = cache_text(source);
+    std::string const path = cache_file(dir, text);
+    std::vector<char> code;
+    if (read_cached(path, text.size(), code)) {
+        if (from_disk) *from_disk = true;
+        return code;
+    }
+    code = compile_hip_source(source, "es_generated.hip", "gfx950");
+    write_cached(dir, path, text.size(), code);
+    return code;
+}
+
+namespace
+{
+
+// Loaded modules of this process, one per (device, source): a module belongs to the device
+// that was current when it was loaded.
 struct module_cache_t {
-    std::mutex                                   mu;
-    std::unordered_map<std::string, hipModule_t> by_source;
+    std::mutex                                              mu;
+    std::map<std::pair<int, std::string>, hipModule_t> by_source;
 };
 
 module_cache_t& module_cache()
@@ -1085,23 +1210,33 @@ struct variant_t {
     hipFunction_t fn2 = nullptr;  // second pass of a split reduction
 };
 
-// Compiles (once per distinct source) and resolves the variant's entry points.
-void load_kernel(variant_t& v)
+bool module_loaded(int device, std::string const& source)
+{
+    auto&                       cache = module_cache();
+    std::lock_guard<std::mutex> lock(cache.mu);
+    return cache.by_source.count({device, source}) != 0;
+}
+
+// Loads the variant's module on `device` (once per distinct source; `code` may be empty when
+// the module is known to be loaded, otherwise it is the source's code object) and resolves
+// the entry points.
+void load_kernel(variant_t& v, int device, std::vector<char> const& code)
 {
     auto&                       cache = module_cache();
     std::lock_guard<std::mutex> lock(cache.mu);
     hipModule_t                 mod;
-    auto                        it = cache.by_source.find(v.k.source);
+    auto                        it = cache.by_source.find({device, v.k.source});
     if (it != cache.by_source.end()) {
         mod = it->second;
     } else {
-        std::vector<char> code = compile_hip_source(v.k.source, "es_generated.hip", "gfx950");
-        hipError_t        err = hipModuleLoadData(&mod, code.data());
+        std::vector<char> compiled;
+        if (code.empty()) compiled = code_object_for(v.k.source, nullptr);
+        hipError_t err = hipModuleLoadData(&mod, code.empty() ? compiled.data() : code.data());
         if (err != hipSuccess) {
             throw km_error(km_status::device,
                            std::string("hipModuleLoadData: ") + hipGetErrorString(err));
         }
-        cache.by_source.emplace(v.k.source, mod);
+        cache.by_source.emplace(std::make_pair(device, v.k.source), mod);
     }
     auto get = [&](std::string const& name) {
         hipFunction_t fn;
@@ -1119,8 +1254,7 @@ void load_kernel(variant_t& v)
 struct codegen_plan_t : plan_t {
     einsummable_t     e;
     variant_t         wide;
-    mutable variant_t narrow;  // compiled on first use with a misaligned buffer
-    mutable std::mutex mu;
+    variant_t         narrow;  // scalar accesses: for buffers that are not 16-byte aligned
 
     explicit codegen_plan_t(einsummable_t const& e_) : e(e_) {}
 
@@ -1197,17 +1331,13 @@ struct codegen_plan_t : plan_t {
             launch(wide, stream, out, inns, workspace);
             return;
         }
-        {
-            std::lock_guard<std::mutex> lock(mu);
-            if (!narrow.fn) load_kernel(narrow);  // generated at plan time, compiled here
-        }
         launch(narrow, stream, out, inns, workspace);
     }
 };
 
 }  // namespace
 
-std::shared_ptr<plan_t> plan_codegen(einsummable_t const& e, int)
+std::shared_ptr<plan_t> plan_codegen(einsummable_t const& e, int device)
 {
     cg_kernel_t k;
     try {
@@ -1219,10 +1349,23 @@ std::shared_ptr<plan_t> plan_codegen(einsummable_t const& e, int)
     if (8 * (1 + k.n_inns) + 8 * k.params.size() > 1000) return nullptr;
     auto p = std::make_shared<codegen_plan_t>(e);
     p->wide.k = std::move(k);
-    load_kernel(p->wide);
-    // the scalar variant is only compiled if a misaligned buffer ever shows up, but its
-    // workspace need is part of what build() reports
     p->narrow.k = generate_kernel(e, 1);
+    // Both variants are compiled and loaded here, the scalar one on a second thread while
+    // this one compiles the wide one: run() only ever launches.
+    std::future<std::vector<char>> narrow_code;
+    bool const narrow_distinct = p->narrow.k.source != p->wide.k.source;
+    if (narrow_distinct && !module_loaded(device, p->narrow.k.source)) {
+        narrow_code = std::async(std::launch::async, [src = p->narrow.k.source]() {
+            return code_object_for(src, nullptr);
+        });
+    }
+    try {
+        load_kernel(p->wide, device, {});
+    } catch (...) {
+        if (narrow_code.valid()) narrow_code.wait();
+        throw;
+    }
+    load_kernel(p->narrow, device, narrow_code.valid() ? narrow_code.get() : std::vector<char>());
     switch (p->wide.k.kind) {
         case cg_kind::elementwise:
             p->description = "elementwise";

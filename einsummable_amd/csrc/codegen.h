@@ -46,4 +46,8 @@ cg_kernel_t generate_kernel(einsummable_t const& e, int max_vec = 16);
 std::vector<char> compile_hip_source(std::string const& source, std::string const& name,
                                      std::string const& arch);
 
+// The code object of a generated source: read from the on-disk cache (ES_KM_CACHE_DIR, default
+// ~/.cache/es_km; "off" disables) or compiled and written there.  *from_disk reports a hit.
+std::vector<char> code_object_for(std::string const& source, bool* from_disk);
+
 }  // namespace es

@@ -412,6 +412,16 @@ void apply_graph_t::run(hipStream_t main, void* arena_) const
     size_t const ns = streams_.size();
     auto stream_at = [&](int s) { return s == 0 ? main : streams_[size_t(s)]; };
     if (ns > 1) {
+        // Forking the pool streams off a stream that is being captured into a HIP graph
+        // crashed inside the HIP runtime (a host-side segmentation fault during the capture):
+        // refused here, for every caller.  A graph finalized on one stream can be captured.
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        check(hipStreamIsCapturing(main, &capturing), "hipStreamIsCapturing");
+        if (capturing != hipStreamCaptureStatusNone) {
+            throw km_error(km_status::invalid,
+                           "apply graph: a run on more than one stream cannot be captured into "
+                           "a HIP graph; finalize the graph on one stream for that");
+        }
         check(hipEventRecord(fork_, main), "hipEventRecord");
         for (size_t s = 1; s != ns; ++s) {
             check(hipStreamWaitEvent(streams_[s], fork_, 0), "hipStreamWaitEvent");

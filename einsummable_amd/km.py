@@ -75,6 +75,17 @@ def load_library():
         raise ImportError(
             "%s is missing: build it with `python -m einsummable_amd.build`" % path
         )
+    # One HIP runtime per process.  PyTorch wheels bundle their own libamdhip64 / libhiprtc
+    # under the same sonames as /opt/rocm's: loaded first, they also satisfy this library's
+    # NEEDED entries; loaded second, they come in as a second runtime beside /opt/rocm's, and
+    # the second one to touch the device finds none.  The tests and bench.py take device
+    # memory and streams from torch, so torch goes first whenever it is installed.  (A C++
+    # host that links this library has no torch in it and uses /opt/rocm's runtime.)
+    if "torch" not in sys.modules:
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
     lib = ctypes.CDLL(path)
     lib.es_km_create.restype = ctypes.c_void_p
     lib.es_km_create.argtypes = [ctypes.c_int]

@@ -106,7 +106,9 @@ def assert_close(got, want, es_dtype, scale=None, what=""):
     with np.errstate(invalid="ignore"):   # inf - inf where both sides overflowed alike
         err = np.abs(got - want)
     bound = RTOL[es_dtype] * np.maximum(np.abs(want), scale)
-    bad = ~fine & ~(err <= bound)
+    # an infinite (or NaN) expectation is only met by that very value: `err <= bound` would
+    # read inf <= inf there and accept anything
+    bad = ~fine & (~np.isfinite(want) | ~(err <= bound))
     if bad.any():
         i = int(np.argmax(np.where(bad, err, 0)))
         raise AssertionError(

@@ -209,3 +209,15 @@ def test_exec_graph_rejects_forward_dependencies():
     g, unary, add, m = _plan_only_graph()
     with _pytest.raises(ea.KmError):
         g.add_einsummable(unary, [m(1), m(0)], deps=[3])
+
+
+def test_assert_close_does_not_accept_a_finite_value_for_an_infinite_one():
+    from helpers import assert_close
+
+    inf = np.inf
+    assert_close(np.array([1.0, -inf, inf, np.nan]), np.array([1.0, -inf, inf, np.nan]), ea.F32)
+    for got, want in (([1.0, 5.0], [1.0, -inf]), ([1.0, inf], [1.0, -inf]), ([1.0, 0.0], [1.0, inf]),
+                      ([1.0, -inf], [1.0, 2.0]), ([1.0, 3.0], [1.0, np.nan]),
+                      ([1.0, np.nan], [1.0, 3.0])):
+        with pytest.raises(AssertionError):
+            assert_close(np.array(got), np.array(want), ea.F32, what="must fail")
