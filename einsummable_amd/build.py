@@ -22,6 +22,7 @@ SOURCES = [
     "exec_graph.cc", "memgraph_wire.cc",
     "codegen.cc",
     "touch.hip",
+    "static_workspace.hip",
     "transpose.hip",
     "contraction.hip",
     "gemm_f16.hip",

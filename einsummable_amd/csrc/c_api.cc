@@ -8,6 +8,7 @@
 #include "memgraph_wire.h"
 #include "gemm_kernel.h"
 #include "kernel_manager.h"
+#include "static_workspace.h"
 
 #include <cstring>
 
@@ -241,6 +242,41 @@ int es_km_execute(es_km_t* h, const uint64_t* join_shape, int join_rank, const i
         std::optional<std::tuple<void*, uint64_t>> ws;
         if (workspace) ws = std::make_tuple(workspace, workspace_bytes);
         (*h->km)(e, static_cast<hipStream_t>(stream), out, v, ws);
+        return ES_KM_OK;
+    });
+}
+
+int es_km_execute_static_workspace(es_km_t* h, const uint64_t* join_shape, int join_rank,
+                                   const int* inns_flat, const int* inns_offsets, int n_inns,
+                                   int out_rank, const char* join_text, char castable,
+                                   void* stream, void* out, const void* const* inns,
+                                   int n_inn_ptrs)
+{
+    return guarded(h, [&]() -> int {
+        if (!h) throw es::ir_error("null handle");
+        check_descriptor(join_shape, join_rank, inns_flat, inns_offsets, n_inns, out_rank,
+                         join_text);
+        if (!out || !inns) throw es::ir_error("execute: null buffer");
+        es::plan_t const* p = h->km->find_raw(raw_key(join_shape, join_rank, inns_flat,
+                                                      inns_offsets, n_inns, out_rank, join_text,
+                                                      castable));
+        if (!p) {
+            p = h->km->plan_of(make_einsummable(join_shape, join_rank, inns_flat, inns_offsets,
+                                                n_inns, out_rank, join_text, castable));
+        }
+        if (!p) throw es::km_error(es::km_status::not_built, "execute: einsummable was not built");
+        if (p->workspace_bytes > es::STATIC_WORKSPACE_BYTES) {
+            throw es::km_error(es::km_status::workspace,
+                               "execute_static_workspace: this einsummable needs " +
+                                   std::to_string(p->workspace_bytes) +
+                                   " bytes of workspace, the library's own holds " +
+                                   std::to_string(es::STATIC_WORKSPACE_BYTES) +
+                                   "; use es_km_execute with a workspace of the caller");
+        }
+        void* ws = es::static_workspace(h->km->device());
+        if (!ws) throw es::km_error(es::km_status::device, "static workspace not initialised");
+        h->km->run_plan(*p, static_cast<hipStream_t>(stream), out, inns, n_inn_ptrs, ws,
+                        es::STATIC_WORKSPACE_BYTES);
         return ES_KM_OK;
     });
 }

@@ -1,6 +1,7 @@
 #include "kernel_manager.h"
 
 #include "launch.h"
+#include "static_workspace.h"
 
 #include <hip/hip_runtime.h>
 
@@ -117,6 +118,7 @@ kernel_manager_t::kernel_manager_t(int device) : device_(device)
                                               std::to_string(count) + " visible)");
     }
     hip_check(hipSetDevice(device), "hipSetDevice");
+    static_workspace_init(device);
 }
 
 kernel_manager_t::~kernel_manager_t() = default;

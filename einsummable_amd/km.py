@@ -17,6 +17,7 @@ EXPORTS = [
     "es_km_build",
     "es_km_workspace_size",
     "es_km_execute",
+    "es_km_execute_static_workspace",
     "es_km_describe",
     "es_km_touch",
     "es_km_touch_batch",
@@ -111,6 +112,12 @@ def load_library():
         ctypes.c_int,
         ctypes.c_void_p,
         ctypes.c_uint64,
+    ]
+    lib.es_km_execute_static_workspace.argtypes = [ctypes.c_void_p] + desc + [
+        ctypes.c_void_p,
+        ctypes.c_void_p,
+        ctypes.c_void_p,
+        ctypes.c_int,
     ]
     lib.es_km_describe.argtypes = [ctypes.c_void_p] + desc + [ctypes.c_void_p, ctypes.c_size_t]
     lib.es_km_touch.argtypes = [
@@ -386,6 +393,14 @@ class KernelManager:
         ws_ptr, ws_size = workspace if workspace else (None, 0)
         rc = self._lib.es_km_execute(self._h, *e._args, stream, out, ptrs, len(inns), ws_ptr,
                                      ws_size)
+        if rc != OK:
+            self._fail(rc)
+
+    def execute_static_workspace(self, e, stream, out, inns):
+        """Like __call__, with the library's own 64 MiB workspace: allocates nothing."""
+        ptrs = (ctypes.c_void_p * max(len(inns), 1))(*inns)
+        rc = self._lib.es_km_execute_static_workspace(self._h, *e._args, stream, out, ptrs,
+                                                      len(inns))
         if rc != OK:
             self._fail(rc)
 

@@ -78,6 +78,24 @@ int es_km_execute(es_km_t* km, const uint64_t* join_shape, int join_rank, const 
                   char castable, void* stream, void* out, const void* const* inns,
                   int n_inn_ptrs, void* workspace, uint64_t workspace_bytes);
 
+/* es_km_execute with the workspace supplied by the library: it allocates nothing.  No
+ * counterpart in the reference, whose callers take workspaces from a pool of device
+ * allocations (src/engine/gpu/workspace.cc:48-91).  It is for callers that cannot allocate
+ * when they execute: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * allocation.  The workspace is ES_KM_STATIC_WORKSPACE_BYTES of device memory that belongs to
+ * the library's code object on each device (held until the process ends); an einsummable
+ * whose build reported more fails with ES_KM_ERR_WORKSPACE, one that reported 0 runs as with
+ * es_km_execute.  Every call on a device uses the same memory and leaves its partial results
+ * there: calls that may overlap in time on one device (different streams, different threads)
+ * race; order them, or give all but one a workspace of their own through es_km_execute.
+ * Results are bit-identical to es_km_execute. */
+#define ES_KM_STATIC_WORKSPACE_BYTES (64ull << 20)
+int es_km_execute_static_workspace(es_km_t* km, const uint64_t* join_shape, int join_rank,
+                                   const int* inns_flat, const int* inns_offsets, int n_inns,
+                                   int out_rank, const char* join_text, char castable,
+                                   void* stream, void* out, const void* const* inns,
+                                   int n_inn_ptrs);
+
 /* Name of the kernel family chosen by build for this einsummable, e.g. "elementwise",
  * "reduce_row", "contraction_mfma_f16" (diagnostics; no counterpart in the reference apart
  * from its force_debug printouts, gpu_kernel_manager.cc:1008-1034). */
