@@ -107,8 +107,8 @@ void choose_tile(dtype_t dt, uint64_t M, uint64_t N, uint64_t K, uint64_t batch,
                              ((double(M) * K + double(N) * K + double(M) * N) * elem);
     if (dt == dtype_t::f16 && intensity < 150.0) return;
     static tile_option_t const options[] = {{256, 256, 1.00, 1.00},
-                                            {128, 256, 0.80, 1.00},
-                                            {256, 128, 0.80, 1.00},
+                                            {128, 256, 0.88, 1.00},
+                                            {256, 128, 0.88, 1.00},
                                             {128, 128, 0.68, 1.00}};
     double best = 0;
     uint64_t const nk = K * dtype_size(dt) / 64;
@@ -121,7 +121,7 @@ void choose_tile(dtype_t dt, uint64_t M, uint64_t N, uint64_t K, uint64_t batch,
         uint64_t const S = (tiles <= 128 && nk >= 16) ? std::min<uint64_t>({256 / tiles, nk / 8, 64}) : 1;
         double fold = 0;
         if (S > 1) {
-            double const ratio = dt == dtype_t::f16 ? 1.17 : 0.14;
+            double const ratio = dt == dtype_t::f16 ? 1.5 : 0.14;
             fold = (4.0 * double(S) + elem) * double(M) * double(N) * double(batch) * ratio /
                    (2.0 * double(K));
         }
@@ -398,6 +398,13 @@ std::shared_ptr<plan_t> plan_contraction(einsummable_t const& e, int)
             a.wide_slices = 0;
         }
     }
+    a.wave8 = 0;
+    if (dt == dtype_t::f16 && p->planned_dma && a.a_mode == 0 && a.b_mode == 0 && !a.shortk &&
+        !a.wide_slices && (p->bm == 256 || p->bn == 256) &&
+        gemm::gemm_dma_wide_eligible<_Float16>(a, p->bm == 256 && p->bn == 256 ? 2u : 3u)) {
+        const char* env = std::getenv("ES_KM_GEMM_WAVES");  // tuning and tests: 4 keeps the old kernel
+        a.wave8 = !(env && env[0] == '4');
+    }
     static const char* mode_name[] = {"k", "mn", "elem"};
     p->description = std::string("contraction_mfma_") + dtype_name(dt) + " tile=" +
                      std::to_string(p->bm) + "x" + std::to_string(p->bn) + " A=" +
@@ -408,7 +415,8 @@ std::shared_ptr<plan_t> plan_contraction(einsummable_t const& e, int)
                      std::to_string(K) + " batch=" + std::to_string(Bt) +
                      (a.splits > 1 ? " split_k=" + std::to_string(a.splits) : "") +
                      (a.shortk ? " resident_a" : "") + (a.warm_a_bytes ? " warm_operands" : "") +
-                     (a.wide_slices ? " slices=128B" : "") + (alpha != 1.0 ? " scaled" : "");
+                     (a.wide_slices ? " slices=128B" : "") +
+                     (a.wave8 ? " slices=128B waves=8" : "") + (alpha != 1.0 ? " scaled" : "");
     return p;
 }
 

@@ -7,8 +7,9 @@
 // workgroup of four wavefronts needs 256 accumulator registers per lane, which leaves no room
 // for register staging of the next slice; the direct-to-LDS loads need none.
 //
-//   * 4 wavefronts, 2 x 2, each owning (BM/2) x (BN/2) of C; 128 x 128 = 4 x 4 MFMA tiles =
-//     256 accumulators for the 256 x 256 tile.
+//   * WGM x WGN wavefronts, each owning (BM/WGM) x (BN/WGN) of C: 2 x 2 (128 x 128 = 4 x 4 MFMA
+//     tiles = 256 accumulators for the 256 x 256 tile), or eight of them, 2 x 4 or 4 x 2, two
+//     per SIMD, for the compute-bound f16 products (launch_gemm_f16 says which and why).
 //   * LDS: NS stages of (BM + BN) rows x 64 bytes.  Loads run NS - 1 slices ahead of the
 //     matrix work; one workgroup barrier per slice.
 //   * One load instruction moves 16 rows x 64 bytes; a wavefront's 64 x 16 bytes land
@@ -66,10 +67,12 @@ __device__ __forceinline__ void wait_loads_and_lds()
 // row (products that stream a large operand once read it at 5.9 instead of 3.6 TB/s in a
 // stand-alone walk of the same pattern), eight rows per load instruction instead of sixteen,
 // and four k-steps per slice instead of two.
-template <typename T, int BM, int BN, int NS, int AMODE, int BMODE, int RB = DMA_ROW>
-__global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
+template <typename T, int BM, int BN, int NS, int AMODE, int BMODE, int RB = DMA_ROW, int WGM = 2,
+          int WGN = 2>
+__global__ __launch_bounds__(64 * WGM * WGN) void gemm_dma_kernel(gemm_args_t a)
 {
     using tr = traits_t<T>;
+    constexpr int NW = WGM * WGN;  // wavefronts, WGM x WGN over the tile
     constexpr int MI = tr::MI;
     constexpr int VL = tr::VL;
     constexpr int BK = RB / int(sizeof(T));
@@ -77,11 +80,12 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
     constexpr int ROWS_PI = 1024 / RB;  // rows per load instruction (operand along k)
     constexpr int STAGE = (BM + BN) * RB;
     constexpr int A_BYTES = BM * RB;
-    constexpr int WM = BM / 2, WN = BN / 2;
+    constexpr int WM = BM / WGM, WN = BN / WGN;
     constexpr int TM = WM / MI, TN = WN / MI;
     constexpr int STEPS = BK / (tr::KG * VL);
     // load instructions per thread per slice: one moves 1 KiB per wavefront
-    constexpr int NLA = BM * RB / 4096, NLB = BN * RB / 4096;
+    constexpr int NLA = BM * RB / (NW * 1024), NLB = BN * RB / (NW * 1024);
+    static_assert(NLA >= 1 && NLB >= 1 && (NW == 4 || NW == 8), "whole load instructions");
     static_assert(MI == 32 && tr::KG == 2 && (STEPS == 2 || STEPS == 4) && (RB == 64 || RB == 128),
                   "layout below assumes 32x32 tiles");
     static_assert(BM % 64 == 0 && BN % 64 == 0, "");
@@ -101,7 +105,7 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
     int const tid = threadIdx.x;
     int const lane = tid & 63;
     int const wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    int const wm = wave >> 1, wn = wave & 1;
+    int const wm = wave / WGN, wn = wave % WGN;
 
     // one XCD (one L2) works on a contiguous run of tiles, across batch entries: attention's
     // P.V, 16 tiles per head, moved 1.67 GiB out of the L2s for 1.06 GiB of operands while the
@@ -153,10 +157,10 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
     T const* const A = uniform(static_cast<T const*>(a.A) + boa);
     T const* const B = uniform(static_cast<T const*>(a.B) + bob);
 
-    // Load instruction i of this wavefront covers rows (4 i + wave) * 16 + lane / 4 of the
+    // Load instruction i of this wavefront covers rows (NW i + wave) * 16 + lane / 4 of the
     // tile; the lane's LDS slot is chunk lane % 4 of that row and holds global chunk
     // (lane % 4) ^ bits 2..3 of the row = (lane % 4) ^ ((lane / 16) % 4).
-    // 128-byte rows: rows (4 i + wave) * 8 + lane / 8, slot lane % 8, and the swizzle is bits
+    // 128-byte rows: rows (NW i + wave) * 8 + lane / 8, slot lane % 8, and the swizzle is bits
     // 1..3 of the row = (wave % 2) * 4 + lane / 16: sixteen consecutive rows of one k-chunk
     // (two rows per 64 banks) again cover all banks once.
     uint32_t const load_chunk =
@@ -174,13 +178,13 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
     for (int i = 0; i != NLA; ++i) {
         int64_t x, y;
         if constexpr (AMODE == 0) {
-            uint32_t r = tm * BM + uint32_t((4 * i + wave) * ROWS_PI + lane / CPRW);
+            uint32_t r = tm * BM + uint32_t((NW * i + wave) * ROWS_PI + lane / CPRW);
             r = r < a.M ? r : a.M - 1;
             group_offsets(a.gm, r, x, y);
             voa[i] = uint32_t(x) * uint32_t(sizeof(T));
         } else {
             // this lane's slot: k row r of the slice, chunk c of that row
-            uint32_t const r = uint32_t(4 * i + wave) * RPIA + uint32_t(lane * 16) / RAM;
+            uint32_t const r = uint32_t(NW * i + wave) * RPIA + uint32_t(lane * 16) / RAM;
             uint32_t const c = (uint32_t(lane * 16) % RAM) / 16;
             uint32_t       m = tm * BM + (c ^ kn_swizzle(r)) * VL;
             m = m < a.M ? m : a.M - VL;  // M is a multiple of VL on this path
@@ -192,13 +196,13 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
     for (int i = 0; i != NLB; ++i) {
         int64_t x, y;
         if constexpr (BMODE == 0) {
-            uint32_t r = tn * BN + uint32_t((4 * i + wave) * ROWS_PI + lane / CPRW);
+            uint32_t r = tn * BN + uint32_t((NW * i + wave) * ROWS_PI + lane / CPRW);
             r = r < a.N ? r : a.N - 1;
             group_offsets(a.gn, r, x, y);
             vob[i] = uint32_t(x) * uint32_t(sizeof(T));
         } else {
             // this lane's slot: k row r of the slice, chunk c of that row
-            uint32_t const r = uint32_t(4 * i + wave) * RPI + uint32_t(lane * 16) / RBN;
+            uint32_t const r = uint32_t(NW * i + wave) * RPI + uint32_t(lane * 16) / RBN;
             uint32_t const c = (uint32_t(lane * 16) % RBN) / 16;
             uint32_t       n = tn * BN + (c ^ kn_swizzle(r)) * VL;
             n = n < a.N ? n : a.N - VL;  // N is a multiple of VL on this path
@@ -206,8 +210,37 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
             vob[i] = (uint32_t(x) + r * uint32_t(a.gk.sy[0])) * uint32_t(sizeof(T));
         }
     }
-    // byte offsets of the lane's 16-byte chunk of slice kt within a row of A / of B
-    auto k_offsets = [&](uint32_t kt, uint32_t& ka, uint32_t& kb) {
+    // Byte offsets of the lane's 16-byte chunk within a row of A / of B, slice after slice:
+    // next_k_offsets hands out those of the next slice in line (every slice's loads are
+    // issued in order).  With several k modes the digits of the slice's first k element are
+    // carried along and stepped by BK -- as long as the innermost mode holds whole slices, the
+    // usual case (a head dimension of 64 or 128) -- instead of decomposing every lane's k by
+    // division: those were some hundred vector instructions per slice in front of the
+    // matrix instructions (out-projection adbe,cde->abc: 0.082 -> 0.070 ms).
+    bool const k_walk = AMODE == 0 && BMODE == 0 && a.gk.n != 1 && a.gk.size[0] % BK == 0;
+    uint32_t   k_next = 0;  // slice index (within this workgroup's share) handed out next
+    uint32_t   k_dig[MAXG] = {0, 0, 0, 0};
+    uint32_t   k_wa = 0, k_wb = 0;        // element offsets of the slice's first k element
+    uint32_t   k_la = 0, k_lb = 0;        // the lane's own part, bytes
+    auto seek_k = [&](uint32_t first_slice) {
+        if (!k_walk) return;
+        int64_t x, y;
+        group_offsets(a.gk, first_slice * BK, x, y);
+        k_wa = uint32_t(x);
+        k_wb = uint32_t(y);
+        uint32_t i = first_slice * BK;
+#pragma unroll
+        for (int d = 0; d != MAXG; ++d) {
+            uint32_t const q = i / a.gk.size[d];
+            k_dig[d] = i - q * a.gk.size[d];
+            i = q;
+        }
+        k_la = load_chunk * VL * uint32_t(a.gk.sx[0]) * uint32_t(sizeof(T));
+        k_lb = load_chunk * VL * uint32_t(a.gk.sy[0]) * uint32_t(sizeof(T));
+    };
+    auto next_k_offsets = [&](uint32_t first_slice, uint32_t& ka, uint32_t& kb) {
+        uint32_t const kt = first_slice + k_next;
+        ++k_next;
         uint32_t const k = kt * BK + load_chunk * VL;
         if constexpr (AMODE == 1 || BMODE == 1) {  // one k mode (checked by the launcher)
             ka = AMODE == 1 ? kt * BK * uint32_t(a.gk.sx[0]) * uint32_t(sizeof(T))
@@ -216,6 +249,22 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
                             : k * uint32_t(sizeof(T));
         } else if (a.gk.n == 1) {  // contiguous in both operands on this path
             ka = kb = k * uint32_t(sizeof(T));
+        } else if (k_walk) {
+            ka = k_wa * uint32_t(sizeof(T)) + k_la;
+            kb = k_wb * uint32_t(sizeof(T)) + k_lb;
+            // step to the next slice: all of this is uniform
+            k_dig[0] += BK;
+            k_wa += BK * uint32_t(a.gk.sx[0]);
+            k_wb += BK * uint32_t(a.gk.sy[0]);
+#pragma unroll
+            for (int d = 0; d + 1 != MAXG; ++d) {
+                if (k_dig[d] == a.gk.size[d]) {
+                    k_dig[d] = 0;
+                    k_dig[d + 1] += 1;
+                    k_wa += uint32_t(a.gk.sx[d + 1]) - a.gk.size[d] * uint32_t(a.gk.sx[d]);
+                    k_wb += uint32_t(a.gk.sy[d + 1]) - a.gk.size[d] * uint32_t(a.gk.sy[d]);
+                }
+            }
         } else {
             int64_t x, y;
             group_offsets(a.gk, k, x, y);
@@ -228,10 +277,10 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
         uint32_t const st = kt % NS;
         if (q < NLA) {
             load_to_lds_16(A, voa[q] + ka,
-                           lds_base + st * STAGE + uint32_t(4 * q + wave) * 1024);
+                           lds_base + st * STAGE + uint32_t(NW * q + wave) * 1024);
         } else {
             load_to_lds_16(B, vob[q - NLA] + kb,
-                           lds_base + st * STAGE + A_BYTES + uint32_t(4 * (q - NLA) + wave) * 1024);
+                           lds_base + st * STAGE + A_BYTES + uint32_t(NW * (q - NLA) + wave) * 1024);
         }
     };
 
@@ -351,7 +400,6 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
     constexpr int MMAS = PAIRS * tr::SUB;
     constexpr int R0 = (READS + MMAS - 1) / MMAS;
     constexpr int R1 = (READS + MMAS - 2) / (MMAS - 1);
-    constexpr int L1 = (LOADS + MMAS - 2) / (MMAS - 1);
 
     // k slices of this workgroup: all of them, or this split's share (the first K/BK mod
     // splits shares are one slice longer); every share has at least NS slices
@@ -363,11 +411,12 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
         nk = q + (z < r ? 1 : 0);
     }
 
-    // prologue: four slices in flight, the first one landed
+    // prologue: NS slices in flight, the first one landed
+    seek_k(k_begin);
 #pragma unroll
     for (int s = 0; s != NS; ++s) {
         uint32_t ka, kb;
-        k_offsets(k_begin + uint32_t(s), ka, kb);
+        next_k_offsets(k_begin, ka, kb);
 #pragma unroll
         for (int q = 0; q != LOADS; ++q) issue(uint32_t(s), q, ka, kb);
     }
@@ -377,16 +426,31 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
     for (int q = 0; q != READS; ++q) read_frag(lds, 0, q, fa[0], fb[0]);
 
     // One slice.  YOUNGER = slices issued after slice kt+1 that may still be in flight when
-    // slice kt+1 is needed (-1: there is no slice kt+1); ISSUE: refill this stage with kt+4.
-    auto slice = [&](uint32_t kt, auto younger_tag, auto issue_tag) {
+    // slice kt+1 is needed (-1: there is no slice kt+1); ISSUE: refill this stage with slice
+    // kt+NS.  The loads of a slice are not issued in one burst: its first 1/STEPS goes out
+    // after the barrier in the last k-step of slice kt, the other parts during the first
+    // STEPS-1 k-steps of slice kt+1 (`prev`: slice kt-1+NS exists and this is not the first
+    // slice, whose predecessor's loads the prologue issued).  Eight wavefronts that each push
+    // all their loads of a slice right after the barrier fill the queue of the texture
+    // addresser, and a wavefront that cannot get a load accepted cannot issue matrix
+    // instructions either (8192^3, 256x256 tile: 72 % of the cycles had a matrix instruction
+    // in flight against 85 % without the loads and 87 % in a run whose loads all hit one line).
+    // (With two stages a load has one slice's time to land, and every part issued later
+    // cuts into it: 8192^3 runs 3 % slower spread out.  The whole slice then goes out after
+    // the barrier.)
+    constexpr bool SPREAD = NS >= 3;
+    auto part_lo = [](int p) { return SPREAD ? p * LOADS / STEPS : (p == 0 ? 0 : LOADS); };
+    uint32_t ka = 0, kb = 0;  // k offsets of the slice that is being issued
+    auto slice = [&](uint32_t kt, auto younger_tag, auto issue_tag, bool prev) {
         constexpr int  YOUNGER = decltype(younger_tag)::value;
         constexpr bool ISSUE = decltype(issue_tag)::value;
         char const*    cur = lds + (kt % NS) * STAGE;
         char const*    nxt = lds + ((kt + 1) % NS) * STAGE;
-        uint32_t       ka = 0, kb = 0;
-        if (ISSUE) k_offsets(k_begin + kt + NS, ka, kb);
+        if (!SPREAD) prev = false;
+        // ka, kb: still those of slice kt-1+NS, whose first part the slice before this one issued
 #pragma unroll
         for (int s = 0; s != STEPS - 1; ++s) {
+            int const lo = part_lo(s + 1), n = part_lo(s + 2) - part_lo(s + 1);
 #pragma unroll
             for (int q = 0; q != MMAS; ++q) {
                 int const p = q % PAIRS;
@@ -395,9 +459,17 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
                 for (int r = q * R0; r != (q + 1) * R0; ++r) {
                     if (r < READS) read_frag(cur, s + 1, r, fa[(s + 1) & 1], fb[(s + 1) & 1]);
                 }
+                if (prev) {
+#pragma unroll
+                    for (int r = lo + q * n / MMAS; r != lo + (q + 1) * n / MMAS; ++r) {
+                        issue(kt - 1 + NS, r, ka, kb);
+                    }
+                }
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
+        if (ISSUE) next_k_offsets(k_begin, ka, kb);  // slice kt+NS
+        constexpr int N0 = SPREAD ? LOADS / STEPS : LOADS;  // part 0
 #pragma unroll
         for (int q = 0; q != MMAS; ++q) {
             int const p = q % PAIRS;
@@ -414,8 +486,8 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
                         if (r < READS) read_frag(nxt, 0, r, fa[0], fb[0]);
                     }
 #pragma unroll
-                    for (int r = (q - 1) * L1; r != q * L1; ++r) {
-                        if (ISSUE && r < LOADS) issue(kt + NS, r, ka, kb);
+                    for (int r = (q - 1) * N0 / (MMAS - 1); r != q * N0 / (MMAS - 1); ++r) {
+                        if (ISSUE) issue(kt + NS, r, ka, kb);
                     }
                 }
             }
@@ -426,12 +498,13 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(gemm_args_t a)
         using std::integral_constant;
         uint32_t kt = 0;
         for (; kt + NS < nk; ++kt) {
-            slice(kt, integral_constant<int, NS - 2>{}, std::true_type{});
+            slice(kt, integral_constant<int, NS - 2>{}, std::true_type{}, kt != 0);
         }
         // the last NS slices refill nothing and have ever fewer loads behind them
         auto tail = [&](auto const& self, auto j_tag) {
             constexpr int J = decltype(j_tag)::value;
-            slice(kt++, integral_constant<int, NS - 2 - J>{}, std::false_type{});
+            slice(kt, integral_constant<int, NS - 2 - J>{}, std::false_type{}, J == 0 && kt != 0);
+            ++kt;
             if constexpr (J + 1 < NS) self(self, integral_constant<int, J + 1>{});
         };
         tail(tail, integral_constant<int, 0>{});
@@ -534,21 +607,23 @@ bool gemm_dma_wide_eligible(gemm_args_t const& a, uint32_t stages)
     return gemm_dma_eligible<T>(a) && a.K % BK == 0 && a.K / BK / splits >= stages;
 }
 
-template <typename T, int BM, int BN, int NS, int AMODE, int BMODE, int RB = DMA_ROW>
+template <typename T, int BM, int BN, int NS, int AMODE, int BMODE, int RB = DMA_ROW, int WGM = 2,
+          int WGN = 2>
 void launch_gemm_dma_kernel_mode(gemm_args_t const& a, hipStream_t stream)
 {
     static_assert(NS >= 2 && NS <= 4, "eligibility guarantees four slices");
     constexpr int lds = NS * (BM + BN) * RB;
     static bool const raised = [] {
         (void)hipFuncSetAttribute(
-            reinterpret_cast<const void*>(&gemm_dma_kernel<T, BM, BN, NS, AMODE, BMODE, RB>),
+            reinterpret_cast<const void*>(
+                &gemm_dma_kernel<T, BM, BN, NS, AMODE, BMODE, RB, WGM, WGN>),
             hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         return true;
     }();
     (void)raised;
     dim3 grid(a.tiles_m * a.tiles_n, a.batch, a.splits > 1 ? a.splits : 1);
-    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, NS, AMODE, BMODE, RB>), grid, dim3(256), lds,
-                       stream, a);
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, NS, AMODE, BMODE, RB, WGM, WGN>), grid,
+                       dim3(64 * WGM * WGN), lds, stream, a);
 }
 
 // Second pass of a split-K contraction: C = sum over the splits' partial tiles, in split

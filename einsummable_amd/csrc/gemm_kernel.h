@@ -61,6 +61,9 @@ struct gemm_args_t {
     // 0, or the number of stages (2 or 3) of the direct-to-LDS kernel with 128-byte slices:
     // planned for f16 products bound by the reads of a large operand
     int         wide_slices;
+    // f16, both operands along k, compute bound: eight wavefronts per workgroup on slices of
+    // 128 bytes (launch_gemm_f16)
+    int         wave8;
     // every sum is multiplied by this before it is rounded to the output type (1 for a plain
     // product); split-K partial tiles stay unscaled, the fold applies it
     double      alpha;

@@ -181,6 +181,40 @@ def test_big_tile_kernels(km, monkeypatch, case, tile):
         assert "tile=" + tile in d, d
 
 
+EIGHT_WAVE_CASES = [
+    # both operands along k, K a whole number of 128-byte slices: the eight-wavefront kernels
+    ("ij,kj->ik", dict(i=512, j=512, k=512)),                    # full tiles
+    ("ij,kj->ik", dict(i=264, j=448, k=520)),                    # ragged m and n, seven slices
+    ("ij,kj->ik", dict(i=40, j=192, k=24)),                      # one partial tile, three slices
+    ("bij,bkj->bik", dict(b=3, i=272, j=256, k=136)),
+    ("adbe,cde->abc", dict(a=2, d=4, b=136, e=64, c=264)),       # two k modes
+    ("ij,kj->ik", dict(i=8, j=4096, k=264)),                     # split-K, partial tiles folded
+]
+
+
+@pytest.mark.parametrize("tile", BIG_TILES)
+@pytest.mark.parametrize("case", range(len(EIGHT_WAVE_CASES)))
+def test_eight_wavefront_kernels_match_the_four_wavefront_ones_bitwise(km, monkeypatch, case, tile):
+    # same products summed in the same order: the bits must agree on random data, and both
+    # must agree with the oracle
+    spec, sizes = EIGHT_WAVE_CASES[case]
+    e = contraction(spec, sizes, "f16")
+    monkeypatch.setenv("ES_KM_GEMM_TILE", tile)
+    eight = ea.KernelManager(0)
+    eight.build(e)  # the planner reads its tuning variables when it plans
+    monkeypatch.setenv("ES_KM_GEMM_WAVES", "4")
+    four = ea.KernelManager(0)
+    four.build(e)
+    r = rng(90 + case)
+    xs = [uniform(r, int(np.prod(e.inn_shape(k))), np.float16) for k in range(2)]
+    a = run_einsummable(eight, e, xs)
+    b = run_einsummable(four, e, xs)
+    assert "waves=8" in eight.describe(e), eight.describe(e)
+    assert "waves=8" not in four.describe(e) and "tile=" + tile in four.describe(e), four.describe(e)
+    np.testing.assert_array_equal(a.view(np.uint16), b.view(np.uint16))
+    assert_close(a, oracle_einsummable(e, xs, oracle.WIDE), ea.F16, what=eight.describe(e))
+
+
 def test_big_tile_matches_small_tile_bitwise_on_exact_data(km, monkeypatch):
     # small integers: every product and partial sum is exact in fp32, so both tilings must
     # give the same bits whatever their summation order
