@@ -603,6 +603,11 @@ int es_km_graph_cross_stream_waits(es_km_graph_t* g)
     return g ? g->graph->n_cross_stream_waits() : ES_KM_ERR_INVALID;
 }
 
+int es_km_graph_launches(es_km_graph_t* g)
+{
+    return g ? g->graph->n_launches() : ES_KM_ERR_INVALID;
+}
+
 int es_km_graph_add_dummy(es_km_graph_t* g, uint64_t offset, uint64_t size, const int* deps,
                           int n_deps)
 {

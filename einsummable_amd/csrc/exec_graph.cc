@@ -311,6 +311,40 @@ void apply_graph_t::finalize(int n_streams)
         }
     }
 
+    // Runs of grouped touches.  The reference's engine launches the touches of a group one
+    // by one (gpu/exec_graph.cc:354-404); a launch costs more than a small window's copy, and
+    // each rereads and rewrites the output.  Nodes v, v+1, .. that are all touches of one
+    // group into the same output range (same dtype, same output extents) are folded into one
+    // touch_batch launch at v's place: nothing lies between them in launch order, every
+    // dependency of a later member is an earlier node, and the chain within the group has
+    // put them on one stream.
+    for (int v = 0; v < n;) {
+        node_t& head = nodes_[v];
+        int     end = v + 1;
+        if (head.kind == kind_t::touch && head.group >= 0) {
+            auto same = [&](node_t const& x) {
+                if (x.kind != kind_t::touch || x.group != head.group || x.stream != head.stream ||
+                    x.mems[0].offset != head.mems[0].offset || x.mems[0].size != head.mems[0].size ||
+                    x.touch.dtype != head.touch.dtype ||
+                    x.touch.selection.size() != head.touch.selection.size()) {
+                    return false;
+                }
+                for (size_t d = 0; d != x.touch.selection.size(); ++d) {
+                    if (x.touch.selection[d].d_out != head.touch.selection[d].d_out) return false;
+                }
+                return true;
+            };
+            while (end < n && same(nodes_[end])) ++end;
+        }
+        if (end - v >= 2) {
+            for (int m = v; m != end; ++m) {
+                nodes_[m].batch_head = v;
+                head.batch.push_back(m);
+            }
+        }
+        v = end;
+    }
+
     if (km_) {
         check(hipSetDevice(km_->device()), "hipSetDevice");
         streams_.assign(size_t(n_streams), nullptr);  // slot 0 is the caller's stream
@@ -350,6 +384,17 @@ void apply_graph_t::finalize(int n_streams)
         }
     }
     finalized_ = true;
+}
+
+int apply_graph_t::n_launches() const
+{
+    int count = 0;
+    for (node_t const& n : nodes_) {
+        if (n.kind == kind_t::dummy) continue;
+        if (n.batch_head >= 0 && n.batch_head != n.position) continue;
+        ++count;
+    }
+    return count;
 }
 
 void apply_graph_t::launch(node_t const& n, hipStream_t stream, char* arena) const
@@ -430,6 +475,28 @@ void apply_graph_t::run(hipStream_t main, void* arena_) const
     for (int v : order_) {
         node_t const&     n = nodes_[size_t(v)];
         hipStream_t const st = stream_at(n.stream);
+        if (n.batch_head >= 0) {
+            if (n.batch_head != v) continue;  // launched with its head
+            std::vector<touch_t>     touches;
+            std::vector<void const*> inns;
+            for (int m : n.batch) {
+                node_t const& nm = nodes_[size_t(m)];
+                for (int d : nm.waits) {
+                    check(hipStreamWaitEvent(st, events_[size_t(event_of_[size_t(d)])], 0),
+                          "hipStreamWaitEvent");
+                }
+                touches.push_back(nm.touch);
+                inns.push_back(arena + nm.mems[1].offset);
+            }
+            km_->touch_batch(touches, st, arena + n.mems[0].offset, inns);
+            for (int m : n.batch) {
+                if (nodes_[size_t(m)].record) {
+                    check(hipEventRecord(events_[size_t(event_of_[size_t(m)])], st),
+                          "hipEventRecord");
+                }
+            }
+            continue;
+        }
         for (int d : n.waits) {
             check(hipStreamWaitEvent(st, events_[size_t(event_of_[size_t(d)])], 0),
                   "hipStreamWaitEvent");

@@ -99,6 +99,8 @@ public:
     std::vector<int> const& deps_of(int id) const { return nodes_[id].deps; }
     // number of event waits run() enqueues (dependencies that cross streams)
     int n_cross_stream_waits() const { return n_waits_; }
+    // number of kernel / copy launches one run() makes (a run of grouped touches counts once)
+    int n_launches() const;
 
 private:
     enum class kind_t { einsummable, touch, constant, lowertri, copy, dummy, evict, load };
@@ -117,6 +119,12 @@ private:
         int                position = -1;
         int                stream = -1;
         bool               record = false;  // some dependent waits for this node's event
+        // Touches of one group that follow each other in launch order and write the same
+        // output run as one launch (kernel_manager_t::touch_batch), at the first one's
+        // place: `batch_head` is that node's id (-1: launched on its own), and the head
+        // holds the ids of all of them.
+        int                batch_head = -1;
+        std::vector<int>   batch;
     };
 
     int  insert(node_t&& n, std::vector<int> const& deps);

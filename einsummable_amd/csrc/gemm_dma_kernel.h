@@ -436,10 +436,11 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dma_kernel(gemm_args_t a)
     // instructions either (8192^3, 256x256 tile: 72 % of the cycles had a matrix instruction
     // in flight against 85 % without the loads and 87 % in a run whose loads all hit one line).
     // (With two stages a load has one slice's time to land, and every part issued later
-    // cuts into it: 8192^3 runs 3 % slower spread out.  The whole slice then goes out after
-    // the barrier.)
-    constexpr bool SPREAD = NS >= 3;
-    auto part_lo = [](int p) { return SPREAD ? p * LOADS / STEPS : (p == 0 ? 0 : LOADS); };
+    // cuts into it: 8192^3 on eight wavefronts runs 3 % slower in four parts than in one and
+    // 2 % faster in two; the four-wavefront kernels on two stages keep the single burst.)
+    constexpr bool SPREAD = true;
+    constexpr int  PARTS = NS >= 3 ? STEPS : (NW == 8 ? 2 : 1);
+    auto part_lo = [](int p) { return (p < PARTS ? p : PARTS) * LOADS / PARTS; };
     uint32_t ka = 0, kb = 0;  // k offsets of the slice that is being issued
     auto slice = [&](uint32_t kt, auto younger_tag, auto issue_tag, bool prev) {
         constexpr int  YOUNGER = decltype(younger_tag)::value;
@@ -469,7 +470,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dma_kernel(gemm_args_t a)
             }
         }
         if (ISSUE) next_k_offsets(k_begin, ka, kb);  // slice kt+NS
-        constexpr int N0 = SPREAD ? LOADS / STEPS : LOADS;  // part 0
+        constexpr int N0 = LOADS / PARTS;  // part 0
 #pragma unroll
         for (int q = 0; q != MMAS; ++q) {
             int const p = q % PAIRS;

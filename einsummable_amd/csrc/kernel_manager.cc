@@ -7,6 +7,7 @@
 
 #include <algorithm>
 #include <cstdlib>
+#include <cstring>
 
 namespace es
 {
@@ -392,11 +393,17 @@ void kernel_manager_t::touch_batch(std::vector<touch_t> const& touches_, hipStre
             }
         }
         // input vectors line up with output vectors when the window's origin has the same
-        // phase in both tensors and every input row starts on a vector boundary
-        bool v = wide && reinterpret_cast<uintptr_t>(inns[i]) % 16 == 0 &&
-                 it.base_inn % uint64_t(vmax) == it.lo[3] % uint32_t(vmax);
-        for (int s = 0; s != 3; ++s) v = v && (it.size[s] == 1 || it.str_inn[s] % uint64_t(vmax) == 0);
-        it.vec_inn = v ? 1 : 0;
+        // phase in both tensors and every input row starts on a vector boundary; with
+        // another phase (shift, in elements) the owner kernel still reads whole input vectors
+        bool rows = wide && reinterpret_cast<uintptr_t>(inns[i]) % 16 == 0;
+        for (int s = 0; s != 3; ++s) {
+            rows = rows && (it.size[s] == 1 || it.str_inn[s] % uint64_t(vmax) == 0);
+        }
+        uint64_t const shift = (it.base_inn + uint64_t(vmax) - it.lo[3] % uint32_t(vmax)) %
+                               uint64_t(vmax);
+        it.vec_inn = rows && shift == 0 ? 1 : 0;
+        it.vec_rows = rows ? 1 : 0;
+        it.shift = int(shift);
     }
     uint64_t out_str4[3];
     for (int s = 0; s != 3; ++s) {
@@ -412,11 +419,19 @@ void kernel_manager_t::touch_batch(std::vector<touch_t> const& touches_, hipStre
         return true;
     };
 
-    // Two ways to keep the sequential result.  Windows that mostly lie side by side are
-    // sorted into levels (a touch goes one level above the last earlier touch it overlaps);
-    // a level's windows are disjoint and run as one launch, each streaming at full width.
-    // Windows stacked on top of each other (the fan-in of partial sums) are folded by the
-    // owner of each output vector instead, which reads and writes the output once per launch.
+    // Two ways to keep the sequential result.  Usually the owner of each output vector folds
+    // the touches that cover it, in list order: one launch over the windows' bounding box, the
+    // output read and written once however many windows overlap.  When the windows are
+    // islands in a much larger box (the walk over the empty part would cost more than the
+    // touches), they are sorted into levels instead (a touch goes one level above the last
+    // earlier touch it overlaps); a level's windows are disjoint and run as one launch, each
+    // streaming through its own window.
+    int const    R = std::max(1, r);  // stored dimensions per item
+    size_t const cap = size_t(touch_list_capacity(R));
+    bool         strides_fit = true;
+    for (size_t i = 0; i != n; ++i) {
+        for (int s = 0; s != 3; ++s) strides_fit = strides_fit && items[i].str_inn[s] < (1ull << 32);
+    }
     constexpr size_t SPAN = 2048;  // the level search is quadratic: bounded spans of the list
     for (size_t span0 = 0; span0 < n; span0 += SPAN) {
         size_t const span_n = std::min(SPAN, n - span0);
@@ -437,9 +452,13 @@ void kernel_manager_t::touch_batch(std::vector<touch_t> const& touches_, hipStre
         }
         double box_volume = 1;
         for (int s = 0; s != 4; ++s) box_volume *= double(bhi[s] - blo[s]);
-        bool const stacked = span_volume >= 4.0 * box_volume;
+        bool by_owner = strides_fit && box_volume <= 8.0 * span_volume;
+        if (const char* env = std::getenv("ES_KM_TOUCH_BATCH")) {  // tuning and tests
+            if (env[0] == 'o') by_owner = strides_fit;  // owner computes
+            if (env[0] == 'l') by_owner = false;        // levels
+        }
 
-        if (!stacked) {
+        if (!by_owner) {
             std::vector<int> level(span_n, 0);
             int              top = 0;
             for (size_t i = 0; i != span_n; ++i) {
@@ -484,22 +503,40 @@ void kernel_manager_t::touch_batch(std::vector<touch_t> const& touches_, hipStre
             continue;
         }
 
-        for (size_t first = span0; first < span0 + span_n; first += TOUCH_BATCH_MAX) {
-            size_t const  cnt = std::min<size_t>(TOUCH_BATCH_MAX, span0 + span_n - first);
-            touch_batch_t b;
-            b.n = int(cnt);
-            b.vec = wide ? vmax : 1;
-            b.aligned = (wide && aligned) ? 1 : 0;
-            b.any_castable = 0;
+        // as many items per launch as the kernel arguments hold; consecutive launches keep
+        // the list order
+        for (size_t first = span0; first < span0 + span_n; first += cap) {
+            size_t const cnt = std::min(cap, span0 + span_n - first);
+            touch_list_t b;
+            b.n = uint32_t(cnt);
+            b.rank = uint32_t(R);
+            b.vec = uint32_t(wide ? vmax : 1);
+            bool     castable = false;
             uint64_t lo[4], hi[4];
             for (int s = 0; s != 4; ++s) {
                 lo[s] = ~0ull;
                 hi[s] = 0;
             }
+            uint32_t const W = uint32_t(touch_list_item_words(R));
+            int const      ND = R > 2 ? 4 : 2;
             for (size_t i = 0; i != cnt; ++i) {
                 touch_item_t const& it = items[first + i];
-                b.items[i] = it;
-                if (it.op) b.any_castable = 1;
+                uint32_t* const     w = b.w + i * W;
+                std::memset(w, 0, W * sizeof(uint32_t));
+                uint64_t const p = reinterpret_cast<uint64_t>(it.inn);
+                w[0] = uint32_t(p);
+                w[1] = uint32_t(p >> 32);
+                w[2] = uint32_t(it.base_inn);
+                w[3] = uint32_t(it.base_inn >> 32);
+                for (int d = 0; d != ND; ++d) {
+                    int const s = 4 - ND + d;
+                    w[4 + d] = it.lo[s];
+                    w[4 + ND + d] = it.size[s];
+                    if (d + 1 != ND) w[4 + 2 * ND + d] = uint32_t(it.str_inn[s]);
+                }
+                w[4 + 3 * ND - 1] =
+                    uint32_t(it.op) | (uint32_t(it.vec_rows) << 8) | (uint32_t(it.shift) << 16);
+                castable = castable || it.op != 0;
                 for (int s = 0; s != 4; ++s) {
                     lo[s] = std::min<uint64_t>(lo[s], it.lo[s]);
                     hi[s] = std::max<uint64_t>(hi[s], it.lo[s] + uint64_t(it.size[s]));
@@ -507,17 +544,21 @@ void kernel_manager_t::touch_batch(std::vector<touch_t> const& touches_, hipStre
             }
             lo[3] = lo[3] / uint64_t(b.vec) * uint64_t(b.vec);
             hi[3] = (hi[3] + uint64_t(b.vec) - 1) / uint64_t(b.vec) * uint64_t(b.vec);
-            b.n_vec = 1;
+            uint64_t rows = 1;
             for (int s = 0; s != 4; ++s) {
                 b.box_lo[s] = uint32_t(lo[s]);
                 b.box_size[s] = uint32_t(hi[s] - lo[s]);
-                b.n_vec *= (s == 3) ? (hi[s] - lo[s]) / uint64_t(b.vec) : (hi[s] - lo[s]);
-                if (s < 3) b.out_str[s] = out_str4[s];
+                if (s < 3) {
+                    b.out_str[s] = out_str4[s];
+                    rows *= hi[s] - lo[s];
+                }
             }
-            if (b.n_vec >= (1ull << 40)) {
+            uint64_t const vpr = (hi[3] - lo[3]) / uint64_t(b.vec);
+            b.chunks_per_row = uint32_t((vpr + TOUCH_LIST_BLOCK_HOST - 1) / TOUCH_LIST_BLOCK_HOST);
+            if (rows * b.chunks_per_row >= (1ull << 31)) {
                 throw km_error(km_status::invalid, "touch_batch: bounding box too large");
             }
-            launch_touch_batch(b, esz, int(dt), stream, out);
+            launch_touch_list(b, esz, int(dt), castable, stream, out);
             hip_check(hipGetLastError(), "touch_batch launch");
         }
     }

@@ -39,24 +39,44 @@ struct touch_item_t {
     int         op;          // 0 copy, 1 add, 2 mul, 3 min, 4 max
     int         vec_inn;     // level kernel: the input can be read as 16-byte vectors that
                              // line up with the output's vectors
+    int         vec_rows;    // owner kernel: every input row starts on a 16-byte boundary ...
+    int         shift;       // ... and the window lies this many elements off the output's
+                             // vector grid
 };
 
-constexpr int TOUCH_BATCH_MAX = 32;  // items per launch (kernel-argument budget)
+constexpr int TOUCH_BATCH_MAX = 32;  // items per level launch (kernel-argument budget)
 
-struct touch_batch_t {
-    int          n;
-    int          vec;           // elements per output vector
-    int          any_castable;  // some item reads the old output value
-    int          aligned;       // every window is vector aligned in both tensors
-    uint32_t     box_lo[4];     // bounding box of the windows
-    uint32_t     box_size[4];   // inner extent in elements
-    uint64_t     out_str[3];    // element strides of the output's outer dimensions
-    uint64_t     n_vec;
-    touch_item_t items[TOUCH_BATCH_MAX];
+// A list of touches for the owner-computes kernel, packed into the kernel arguments: every
+// workgroup (one wavefront) owns 64 consecutive output vectors of one row of the windows'
+// bounding box and folds, in list order, the items whose windows reach it.  Items of a list
+// whose touches have at most two dimensions are stored with two (12 words, leading extents
+// are 1 in every item), others with four (16 words): 64 or 60 touches travel in one launch.
+// Words of an item, ND = 2 or 4: input pointer (2), base_inn (2), lo[ND], size[ND],
+// str_inn[ND - 1] (elements, < 2^32), op | vec_rows << 8 | shift << 16.
+constexpr int TOUCH_LIST_WORDS = 960;
+constexpr int TOUCH_LIST_BLOCK_HOST = 64;  // output vectors per workgroup of the owner kernel
+
+struct touch_list_t {
+    uint32_t n;
+    uint32_t rank;            // 1..4: of the touches; > 2 selects the four-dimensional items
+    uint32_t vec;             // elements per output vector
+    uint32_t chunks_per_row;  // workgroups per row of the bounding box
+    uint32_t box_lo[4];       // bounding box of the windows, four normalised dimensions
+    uint32_t box_size[4];     // inner extent in elements, a multiple of vec
+    uint64_t out_str[3];      // element strides of the output's outer dimensions
+    uint32_t w[TOUCH_LIST_WORDS];
 };
 
-void launch_touch_batch(touch_batch_t const& b, int elem_size, int dtype_code, hipStream_t stream,
-                        void* out);
+inline int touch_list_item_words(int rank) { return rank > 2 ? 16 : 12; }
+
+inline int touch_list_capacity(int rank)
+{
+    int const fit = TOUCH_LIST_WORDS / touch_list_item_words(rank);
+    return fit < 64 ? fit : 64;  // the kernel finds its items with one 64-lane ballot
+}
+
+void launch_touch_list(touch_list_t const& b, int elem_size, int dtype_code, bool any_castable,
+                       hipStream_t stream, void* out);
 
 // A set of touches into one output tensor whose windows are pairwise disjoint: one launch,
 // blockIdx.y selects the touch, every touch streams through its own window.  Output vectors

@@ -6,13 +6,15 @@
 //
 // Layout: one thread moves one 16-byte vector (or one element when the windows are not
 // 16-byte aligned) of the innermost dimension; consecutive lanes take consecutive vectors of
-// a row, so every wavefront reads and writes whole 1 KiB row segments.  Each thread handles
-// UNROLL vectors 256 lanes apart, all loads issued before the first store.
+// a row, so every wavefront reads and writes whole 1 KiB row segments.  One vector per thread
+// (four per thread, 256 lanes apart, was 2.7 times slower on a 16 MiB copy), its loads issued
+// before its store.
 #include "launch.h"
 
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <cstddef>
 #include <cstring>
 
 namespace es
@@ -186,133 +188,6 @@ void launch_touch_op(touch_launch_t const& a, int op, hipStream_t stream, void* 
     }
 }
 
-// ---- batched touches
-
-// V: elements per output vector.  ALIGNED: every window starts and ends on a vector boundary
-// in both tensors, so inputs are read as vectors too; otherwise a window may cut through an
-// output vector and its input is read element by element under a per-element mask.
-template <typename T, int V, bool ALIGNED>
-__global__ __launch_bounds__(256) void touch_batch_kernel(touch_batch_t b, T* __restrict__ out)
-{
-    using vt = vec_t<T, V>;
-    uint64_t idx = uint64_t(blockIdx.x) * 256 + threadIdx.x;
-    if (idx >= b.n_vec) return;
-    // position inside the bounding box, then absolute output coordinates
-    uint32_t vpr = b.box_size[3] / V;
-    uint32_t c[4];
-    {
-        uint64_t r = idx;
-        c[3] = b.box_lo[3] + uint32_t(r % vpr) * V;
-        r /= vpr;
-        c[2] = b.box_lo[2] + uint32_t(r % b.box_size[2]);
-        r /= b.box_size[2];
-        c[1] = b.box_lo[1] + uint32_t(r % b.box_size[1]);
-        c[0] = b.box_lo[0] + uint32_t(r / b.box_size[1]);
-    }
-    uint64_t const oo = c[0] * b.out_str[0] + c[1] * b.out_str[1] + c[2] * b.out_str[2] + c[3];
-    // Workgroup-level culling on values that are uniform over the workgroup (scalar unit):
-    // when its 256 vectors lie in one row, an item whose window misses that row or that
-    // column range is skipped without any per-lane work.
-    uint64_t const first = uint64_t(blockIdx.x) * 256;
-    uint64_t const last = (first + 255 < b.n_vec ? first + 255 : b.n_vec - 1);
-    bool const     one_row = first / vpr == last / vpr;
-    uint32_t       u[3] = {0, 0, 0};
-    uint32_t       col_lo = 0, col_hi = 0;
-    if (one_row) {
-        uint64_t r = first;
-        col_lo = b.box_lo[3] + uint32_t(r % vpr) * V;
-        col_hi = b.box_lo[3] + uint32_t(last % vpr) * V + V;
-        r /= vpr;
-        u[2] = b.box_lo[2] + uint32_t(r % b.box_size[2]);
-        r /= b.box_size[2];
-        u[1] = b.box_lo[1] + uint32_t(r % b.box_size[1]);
-        u[0] = b.box_lo[0] + uint32_t(r / b.box_size[1]);
-    }
-    vt   val;
-    bool have = false;
-    // fully unrolled so that every item is read from the kernel arguments at a fixed offset
-    // (scalar loads); a dynamic index would make each thread copy the argument block to scratch
-#pragma unroll
-    for (int t = 0; t != TOUCH_BATCH_MAX; ++t) {
-        if (t >= b.n) break;
-        touch_item_t const& it = b.items[t];
-        if (one_row && !(u[0] - it.lo[0] < it.size[0] && u[1] - it.lo[1] < it.size[1] &&
-                         u[2] - it.lo[2] < it.size[2] && col_lo < it.lo[3] + it.size[3] &&
-                         col_hi > it.lo[3])) {
-            continue;
-        }
-        uint32_t d0 = c[0] - it.lo[0], d1 = c[1] - it.lo[1], d2 = c[2] - it.lo[2];
-        // columns [c3, c3 + V) against the window [lo3, lo3 + size3)
-        bool cols = c[3] < it.lo[3] + it.size[3] && c[3] + V > it.lo[3];
-        if (d0 < it.size[0] && d1 < it.size[1] && d2 < it.size[2] && cols) {
-            uint64_t const row = it.base_inn + d0 * it.str_inn[0] + d1 * it.str_inn[1] +
-                                 d2 * it.str_inn[2];
-            T const* const src = static_cast<T const*>(it.inn) + row;
-            vt   x;
-            bool in[V];
-            bool full = true;
-            if constexpr (ALIGNED) {
-                x = *reinterpret_cast<vt const*>(src + (c[3] - it.lo[3]));
-#pragma unroll
-                for (int j = 0; j != V; ++j) in[j] = true;
-            } else {
-#pragma unroll
-                for (int j = 0; j != V; ++j) {
-                    uint32_t d3 = c[3] + uint32_t(j) - it.lo[3];
-                    in[j] = d3 < it.size[3];
-                    full = full && in[j];
-                    if (in[j]) x.v[j] = src[d3];
-                }
-            }
-            if (!have && (it.op != OP_COPY || !full)) val = *reinterpret_cast<vt const*>(out + oo);
-#pragma unroll
-            for (int j = 0; j != V; ++j) {
-                if (!in[j]) continue;
-                switch (it.op) {
-                    case OP_COPY:
-                        val.v[j] = x.v[j];
-                        break;
-                    case OP_ADD:
-                        val.v[j] = apply<OP_ADD, T>(val.v[j], x.v[j]);
-                        break;
-                    case OP_MUL:
-                        val.v[j] = apply<OP_MUL, T>(val.v[j], x.v[j]);
-                        break;
-                    case OP_MIN:
-                        if constexpr (!(sizeof(T) == 8 && alignof(T) == 4)) {
-                            val.v[j] = apply<OP_MIN, T>(val.v[j], x.v[j]);
-                        }
-                        break;
-                    default:
-                        if constexpr (!(sizeof(T) == 8 && alignof(T) == 4)) {
-                            val.v[j] = apply<OP_MAX, T>(val.v[j], x.v[j]);
-                        }
-                        break;
-                }
-            }
-            have = true;
-        }
-    }
-    if (have) *reinterpret_cast<vt*>(out + oo) = val;
-}
-
-template <typename T>
-void launch_touch_batch_t(touch_batch_t const& b, hipStream_t stream, void* out)
-{
-    constexpr int VMAX = 16 / sizeof(T);
-    unsigned      blocks = unsigned((b.n_vec + 255) / 256);
-    if (b.vec == VMAX && b.aligned) {
-        hipLaunchKernelGGL((touch_batch_kernel<T, VMAX, true>), dim3(blocks), dim3(256), 0, stream,
-                           b, static_cast<T*>(out));
-    } else if (b.vec == VMAX) {
-        hipLaunchKernelGGL((touch_batch_kernel<T, VMAX, false>), dim3(blocks), dim3(256), 0,
-                           stream, b, static_cast<T*>(out));
-    } else {
-        hipLaunchKernelGGL((touch_batch_kernel<T, 1, true>), dim3(blocks), dim3(256), 0, stream, b,
-                           static_cast<T*>(out));
-    }
-}
-
 // ---- touches with pairwise disjoint windows, one per blockIdx.y
 
 template <typename T>
@@ -331,6 +206,236 @@ __device__ __forceinline__ T apply_dyn(int op, T out, T inn)
         default:
             if constexpr (!(sizeof(T) == 8 && alignof(T) == 4)) return apply<OP_MAX, T>(out, inn);
             return inn;
+    }
+}
+
+constexpr int TOUCH_LIST_BLOCK = TOUCH_LIST_BLOCK_HOST;
+
+// ---- a list of touches folded by the owner of each output vector
+//
+// One workgroup = one wavefront = 64 consecutive output vectors of one row of the bounding
+// box.  Lane t tests whether item t reaches the wavefront (at most 64 items per launch), the
+// ballot is the wavefront's list, and the items on it are folded in list order; everything
+// about an item except the lane's own column is uniform and sits in one wide scalar load.
+// What this replaces, on 64 accumulating windows of 512 x 512 at odd offsets of a 4096 x 4096
+// f16 output: the same fold unrolled over 32 items per launch (the code outgrew the
+// instruction cache: 2 x 77 us), a scalar walk over all items (several dependent scalar loads
+// each: 189 us), workgroups of 256 (seven items each on average, one latency chain after the
+// other: 48 us).
+//
+// R4: items keep four dimensions (16 words); otherwise two (12 words; leading extents are 1).
+// Words of an item, ND = 4 or 2: input pointer (2), base_inn (2), lo[ND], size[ND],
+// str_inn[ND - 1], op | vec_rows << 8 | shift << 16.
+template <typename T, int V, bool R4>
+__global__ __launch_bounds__(TOUCH_LIST_BLOCK) void touch_list_kernel(touch_list_t b,
+                                                                      T* __restrict__ out)
+{
+    using vt = vec_t<T, V>;
+    constexpr int ND = R4 ? 4 : 2;
+    constexpr int WI = R4 ? 16 : 12;
+    uint32_t       row = blockIdx.x / b.chunks_per_row;
+    uint32_t const chunk = blockIdx.x - row * b.chunks_per_row;
+    uint32_t       u[3] = {0, 0, 0};  // the row's coordinates, right-aligned
+    uint64_t       row_off = 0;
+    if constexpr (R4) {
+#pragma unroll
+        for (int s = 2; s >= 0; --s) {
+            uint32_t const q = row / b.box_size[s];
+            u[s] = b.box_lo[s] + (row - q * b.box_size[s]);
+            row = q;
+            row_off += u[s] * b.out_str[s];
+        }
+    } else {
+        u[2] = b.box_lo[2] + row;
+        row_off = u[2] * b.out_str[2];
+    }
+    uint32_t const box_hi3 = b.box_lo[3] + b.box_size[3];
+    uint32_t const col_lo = b.box_lo[3] + chunk * uint32_t(TOUCH_LIST_BLOCK) * V;
+    uint32_t const col_hi =
+        col_lo + uint32_t(TOUCH_LIST_BLOCK) * V < box_hi3 ? col_lo + uint32_t(TOUCH_LIST_BLOCK) * V : box_hi3;
+    uint32_t const c3 = col_lo + threadIdx.x * V;
+    bool const     live = c3 < box_hi3;
+    uint64_t const oo = row_off + c3;
+    // The item table is read through the kernel-argument pointer (`b` is the first argument):
+    // a run-time index into the by-value struct invites the compiler to copy the argument
+    // block into private memory first.
+    typedef uint32_t const __attribute__((address_space(4))) const_word_t;
+    typedef char const __attribute__((address_space(4))) const_byte_t;
+    const_word_t* const table = (const_word_t*)((const_byte_t*)__builtin_amdgcn_kernarg_segment_ptr() +
+                                                offsetof(touch_list_t, w));
+    uint64_t todo;
+    {
+        // every word is loaded before the first comparison (a test that stops at the first
+        // miss waits for one load after the other)
+        uint32_t const      t = threadIdx.x;
+        const_word_t* const it = table + (t < b.n ? t : 0u) * WI;
+        uint32_t            lo[ND], sz[ND];
+#pragma unroll
+        for (int d = 0; d != ND; ++d) {
+            lo[d] = it[4 + d];
+            sz[d] = it[4 + ND + d];
+        }
+        bool hit = (t < b.n) & (col_lo < lo[ND - 1] + sz[ND - 1]) & (col_hi > lo[ND - 1]);
+#pragma unroll
+        for (int d = 0; d != ND - 1; ++d) hit = hit & (u[3 - (ND - 1) + d] - lo[d] < sz[d]);
+        todo = __ballot(hit);
+    }
+    if (todo == 0) return;
+    // the old value is on its way while the first item's words arrive; lanes that no window
+    // reaches never store
+    vt val;
+    if (live) val = *reinterpret_cast<vt const*>(out + oo);
+    bool have = false;
+    // K items at a time: the words of all K, then the input vectors of all K, are under way
+    // before the first one is folded in -- one item after the other, each a chain of a scalar
+    // load, two vector loads and the update, a wavefront lived 14 k cycles for two items
+    constexpr int K = R4 ? 2 : 4;
+    while (todo) {
+        uint32_t w[K][WI];
+        bool     valid[K];
+#pragma unroll
+        for (int k = 0; k != K; ++k) {
+            valid[k] = todo != 0;
+            uint32_t const t = valid[k] ? uint32_t(__builtin_ctzll(todo)) : 0u;
+            if (valid[k]) todo &= todo - 1;
+            const_word_t* const it = table + t * WI;
+#pragma unroll
+            for (int i = 0; i != WI; ++i) w[k][i] = it[i];
+        }
+        uint32_t d[K][8];
+        uint32_t j_lo[K], j_hi[K];
+        bool     covered[K];
+        T const* elems[K];  // scalar path: the lane's first element
+#pragma unroll
+        for (int k = 0; k != K; ++k) {
+            uint32_t const lo3 = w[k][4 + ND - 1], sz3 = w[k][4 + 2 * ND - 1];
+            uint64_t       src_row = uint64_t(w[k][2]) | (uint64_t(w[k][3]) << 32);
+#pragma unroll
+            for (int dd = 0; dd != ND - 1; ++dd) {
+                src_row += uint64_t(u[3 - (ND - 1) + dd] - w[k][4 + dd]) * w[k][4 + 2 * ND + dd];
+            }
+            covered[k] = valid[k] && live && c3 < lo3 + sz3 && c3 + V > lo3;
+            // elements j_lo .. j_hi of this vector lie inside the window
+            j_lo[k] = c3 >= lo3 ? 0u : lo3 - c3;
+            j_hi[k] = c3 + V <= lo3 + sz3 ? uint32_t(V - 1) : lo3 + sz3 - 1 - c3;
+            uint32_t const flags = w[k][4 + 3 * ND - 1];
+            T const* const src =
+                reinterpret_cast<T const*>(uint64_t(w[k][0]) | (uint64_t(w[k][1]) << 32)) + src_row;
+            elems[k] = src + (int64_t(c3) - int64_t(lo3));
+#pragma unroll
+            for (int i = 0; i != 8; ++i) d[k][i] = 0;
+            if constexpr (V * sizeof(T) == 16) {
+                if (covered[k] && (flags & 0x100)) {
+                    // The input's rows are 16-byte aligned but the window sits `sh` elements
+                    // off the output's vector grid: the vector's elements come out of two
+                    // aligned input vectors, shifted by a whole number of bytes that is the
+                    // same for the whole item.  Neither vector is loaded unless one of its
+                    // elements is needed: an aligned 16-byte load that holds a valid element
+                    // cannot leave its page.
+                    uint32_t const sh = (flags >> 16) & 0xf;
+                    T const* const p0 = elems[k] - int64_t(sh);
+                    if (j_lo[k] + sh < uint32_t(V)) {
+                        vec_t<uint32_t, 4> const v0 = *reinterpret_cast<vec_t<uint32_t, 4> const*>(p0);
+#pragma unroll
+                        for (int i = 0; i != 4; ++i) d[k][i] = v0.v[i];
+                    }
+                    if (j_hi[k] + sh >= uint32_t(V)) {
+                        vec_t<uint32_t, 4> const v1 =
+                            *reinterpret_cast<vec_t<uint32_t, 4> const*>(p0 + V);
+#pragma unroll
+                        for (int i = 0; i != 4; ++i) d[k][4 + i] = v1.v[i];
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int k = 0; k != K; ++k) {
+            if (!covered[k]) continue;
+            uint32_t const flags = w[k][4 + 3 * ND - 1];
+            int const      op = int(flags & 0xff);
+            bool const     full = j_lo[k] == 0 && j_hi[k] == uint32_t(V - 1);
+            vt             x;
+            bool           by_vector = false;
+            if constexpr (V * sizeof(T) == 16) by_vector = (flags & 0x100) != 0;
+            if (by_vector) {
+                uint32_t const bytes = ((flags >> 16) & 0xf) * uint32_t(sizeof(T));
+                uint32_t const q = bytes >> 2, r = bytes & 3;
+                uint32_t       o[4];
+                switch (q) {  // uniform
+                    case 0:
+#pragma unroll
+                        for (int i = 0; i != 4; ++i) o[i] = __builtin_amdgcn_alignbyte(d[k][i + 1], d[k][i], r);
+                        break;
+                    case 1:
+#pragma unroll
+                        for (int i = 0; i != 4; ++i) o[i] = __builtin_amdgcn_alignbyte(d[k][i + 2], d[k][i + 1], r);
+                        break;
+                    case 2:
+#pragma unroll
+                        for (int i = 0; i != 4; ++i) o[i] = __builtin_amdgcn_alignbyte(d[k][i + 3], d[k][i + 2], r);
+                        break;
+                    default:
+#pragma unroll
+                        for (int i = 0; i != 4; ++i) o[i] = __builtin_amdgcn_alignbyte(d[k][i + 4], d[k][i + 3], r);
+                        break;
+                }
+                vec_t<uint32_t, 4> ov;
+#pragma unroll
+                for (int i = 0; i != 4; ++i) ov.v[i] = o[i];
+                if constexpr (V * sizeof(T) == 16) x = __builtin_bit_cast(vt, ov);
+            } else {
+#pragma unroll
+                for (int j = 0; j != V; ++j) {
+                    if (uint32_t(j) >= j_lo[k] && uint32_t(j) <= j_hi[k]) x.v[j] = elems[k][j];
+                }
+            }
+            have = true;
+            if (full) {
+                switch (op) {  // uniform
+                    case OP_COPY:
+                        val = x;
+                        break;
+                    case OP_ADD:
+#pragma unroll
+                        for (int j = 0; j != V; ++j) val.v[j] = apply_dyn<T>(OP_ADD, val.v[j], x.v[j]);
+                        break;
+                    default:
+#pragma unroll
+                        for (int j = 0; j != V; ++j) val.v[j] = apply_dyn<T>(op, val.v[j], x.v[j]);
+                        break;
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j != V; ++j) {
+                    if (uint32_t(j) >= j_lo[k] && uint32_t(j) <= j_hi[k]) {
+                        val.v[j] = apply_dyn<T>(op, val.v[j], x.v[j]);
+                    }
+                }
+            }
+        }
+    }
+    if (have) *reinterpret_cast<vt*>(out + oo) = val;
+}
+
+template <typename T>
+void launch_touch_list_t(touch_list_t const& b, hipStream_t stream, void* out)
+{
+    constexpr int  VMAX = 16 / sizeof(T);
+    uint64_t const rows = uint64_t(b.box_size[0]) * b.box_size[1] * b.box_size[2];
+    dim3 const     grid(unsigned(rows * b.chunks_per_row));
+    dim3 const     block(TOUCH_LIST_BLOCK);
+    T* const       o = static_cast<T*>(out);
+    bool const     r4 = b.rank > 2;
+    if (int(b.vec) == VMAX) {
+        if (r4) {
+            hipLaunchKernelGGL((touch_list_kernel<T, VMAX, true>), grid, block, 0, stream, b, o);
+        } else {
+            hipLaunchKernelGGL((touch_list_kernel<T, VMAX, false>), grid, block, 0, stream, b, o);
+        }
+    } else if (r4) {
+        hipLaunchKernelGGL((touch_list_kernel<T, 1, true>), grid, block, 0, stream, b, o);
+    } else {
+        hipLaunchKernelGGL((touch_list_kernel<T, 1, false>), grid, block, 0, stream, b, o);
     }
 }
 
@@ -503,29 +608,29 @@ void launch_touch(touch_launch_t const& a, int elem_size, int dtype_code, int op
     }
 }
 
-void launch_touch_batch(touch_batch_t const& b, int elem_size, int dtype_code, hipStream_t stream,
-                        void* out)
+void launch_touch_list(touch_list_t const& b, int elem_size, int dtype_code, bool any_castable,
+                       hipStream_t stream, void* out)
 {
-    if (b.n == 0 || b.n_vec == 0) return;
-    if (!b.any_castable) {
+    if (b.n == 0 || b.box_size[3] == 0) return;
+    if (!any_castable) {
         switch (elem_size) {
             case 2:
-                return launch_touch_batch_t<uint16_t>(b, stream, out);
+                return launch_touch_list_t<uint16_t>(b, stream, out);
             case 4:
-                return launch_touch_batch_t<uint32_t>(b, stream, out);
+                return launch_touch_list_t<uint32_t>(b, stream, out);
             default:
-                return launch_touch_batch_t<uint64_t>(b, stream, out);
+                return launch_touch_list_t<uint64_t>(b, stream, out);
         }
     }
     switch (dtype_code) {
         case 0:
-            return launch_touch_batch_t<_Float16>(b, stream, out);
+            return launch_touch_list_t<_Float16>(b, stream, out);
         case 1:
-            return launch_touch_batch_t<float>(b, stream, out);
+            return launch_touch_list_t<float>(b, stream, out);
         case 2:
-            return launch_touch_batch_t<double>(b, stream, out);
+            return launch_touch_list_t<double>(b, stream, out);
         default:
-            return launch_touch_batch_t<c64_t>(b, stream, out);
+            return launch_touch_list_t<c64_t>(b, stream, out);
     }
 }
 

@@ -39,6 +39,7 @@ EXPORTS = [
     "es_km_graph_run",
     "es_km_graph_node_info",
     "es_km_graph_cross_stream_waits",
+    "es_km_graph_launches",
     "es_km_graph_add_dummy",
     "es_km_graph_add_evict",
     "es_km_graph_add_load",
@@ -184,6 +185,7 @@ def load_library():
     lib.es_km_graph_run.argtypes = [V, V, V]
     lib.es_km_graph_node_info.argtypes = [V, I, V, V, V, I, V]
     lib.es_km_graph_cross_stream_waits.argtypes = [V]
+    lib.es_km_graph_launches.argtypes = [V]
     lib.es_km_graph_add_dummy.argtypes = [V, U64, U64, V, I]
     lib.es_km_graph_add_evict.argtypes = [V, U64, U64, I, V, I]
     lib.es_km_graph_add_load.argtypes = [V, I, U64, U64, V, I]
@@ -526,6 +528,9 @@ class ApplyGraph:
 
     def cross_stream_waits(self):
         return self._check(self._lib.es_km_graph_cross_stream_waits(self._g))
+
+    def launches(self):
+        return self._check(self._lib.es_km_graph_launches(self._g))
 
     def add_dummy(self, mem=(0, 0), deps=None):
         d, nd = self._deps(deps)

@@ -111,7 +111,7 @@ int es_km_describe(es_km_t* km, const uint64_t* join_shape, int join_rank, const
 int es_km_touch(es_km_t* km, const uint64_t* touchdims, int rank, char castable, int dtype,
                 void* stream, void* out, const void* inn);
 
-/* A group of touches into ONE output tensor in one call (one launch per 32 touches): the
+/* A group of touches into ONE output tensor in one call (one launch for up to 64 touches): the
  * result is bit-identical to calling es_km_touch on each, in list order, including where
  * windows overlap.  touchdims holds the selections back to back (ranks[i] x 5 values each),
  * castables[i] is '+','x','v','^' or 0, inns[i] the input of touch i.  All touches share the
@@ -229,6 +229,11 @@ int es_km_graph_run(es_km_graph_t* g, void* stream, void* arena);
 int es_km_graph_node_info(es_km_graph_t* g, int id, int* position, int* stream, int* deps, int cap,
                           int* n_deps);
 int es_km_graph_cross_stream_waits(es_km_graph_t* g);
+/* After finalize: launches one run makes.  Touches of one group that follow each other in
+ * insertion order and write the same output range count once: they run as one
+ * es_km_touch_batch launch, with the bytes of one launch per touch
+ * (src/engine/gpu/exec_graph.cc:354-404 issues them one by one). */
+int es_km_graph_launches(es_km_graph_t* g);
 
 /* Nodes that launch nothing and only carry dependencies (dummy_t, which the reference makes
  * of inputmem / inputsto / partialize / alloc / del nodes, src/engine/gpu/exec_graph.cc:94-97).

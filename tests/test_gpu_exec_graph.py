@@ -110,6 +110,48 @@ def test_touch_groups_first_member_initialises_then_members_accumulate_in_order(
     assert np.array_equal(arena[:n].cpu().numpy().view(np.uint16), want.view(np.uint16))
 
 
+@pytest.mark.parametrize("n_streams", [1, 3])
+def test_a_group_of_64_touches_runs_as_one_launch_with_the_oracles_bytes(km, n_streams):
+    # the memory-movement configuration as the engine would hold it: 64 accumulating touches
+    # of 512 x 512 blocks into windows of one 2048 x 2048 output at odd offsets, all of one
+    # group, each with its own input range; then a second group into another output
+    import torch
+
+    import oracle
+
+    r = rng(121)
+    n, blk, count = 2048, 512, 64
+    out_bytes, blk_bytes = n * n * 2, blk * blk * 2
+    blocks = [normal(r, blk * blk, np.float16) for _ in range(count)]
+    offs = [(int(r.randint(0, n - blk + 1)), int(r.randint(0, n - blk + 1))) for _ in range(count)]
+    arena = torch.empty((2 * out_bytes + count * blk_bytes) // 2, dtype=torch.float16, device="cuda")
+    arena[:2 * n * n] = 777.0                      # stale bytes: the first touch of a group replaces its window only
+    init = arena[:2 * n * n].cpu().numpy().copy()
+    for k, b in enumerate(blocks):
+        lo = (2 * out_bytes + k * blk_bytes) // 2
+        arena[lo:lo + blk * blk] = torch.from_numpy(b).cuda()
+    g = ea.ApplyGraph(km)
+    for which in range(2):
+        for k in range(count):
+            ro, co = offs[k] if which == 0 else offs[count - 1 - k]
+            t = ea.Touch([(blk, n, 0, ro, blk), (blk, n, 0, co, blk)], "+", ea.F16)
+            g.add_touch(t, 40 + which, [(which * out_bytes, out_bytes),
+                                        (2 * out_bytes + k * blk_bytes, blk_bytes)])
+    g.finalize(n_streams)
+    assert g.launches() == 2, g.launches()
+    g.run(stream_handle(), arena.data_ptr())
+    torch.cuda.synchronize()
+    got = arena[:2 * n * n].cpu().numpy()
+    for which in range(2):
+        want = init[which * n * n:(which + 1) * n * n].copy()
+        for k in range(count):
+            ro, co = offs[k] if which == 0 else offs[count - 1 - k]
+            dims = [(blk, n, 0, ro, blk), (blk, n, 0, co, blk)]
+            want = oracle.touch(dims, None if k == 0 else "+", want, blocks[k])
+        assert np.array_equal(got[which * n * n:(which + 1) * n * n].view(np.uint16),
+                              want.view(np.uint16)), which
+
+
 @pytest.mark.parametrize("n_streams", [1, 2, 4])
 def test_llama_layer_through_the_exec_graph_equals_node_by_node_launches(km, n_streams):
     import torch
