@@ -16,6 +16,9 @@ from .km import (  # noqa: F401
     Einsummable,
     KernelManager,
     KmError,
+    NodeCallback,
+    StreamPool,
+    WorkspacePool,
     Touch,
     TouchBatch,
     codegen_source,

@@ -19,7 +19,7 @@ SOURCES = [
     "ir.cc",
     "kernel_manager.cc",
     "c_api.cc",
-    "exec_graph.cc", "memgraph_wire.cc",
+    "exec_graph.cc", "memgraph_wire.cc", "pools.cc",
     "codegen.cc",
     "touch.hip",
     "static_workspace.hip",

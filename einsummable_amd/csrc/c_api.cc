@@ -8,6 +8,7 @@
 #include "memgraph_wire.h"
 #include "gemm_kernel.h"
 #include "kernel_manager.h"
+#include "pools.h"
 #include "static_workspace.h"
 
 #include <cstring>
@@ -15,6 +16,16 @@
 struct es_km {
     std::unique_ptr<es::kernel_manager_t> km;
     std::string                           last_error;
+};
+
+struct es_km_workspace_pool {
+    es::workspace_pool_t pool;
+    explicit es_km_workspace_pool(int device) : pool(device) {}
+};
+
+struct es_km_stream_pool {
+    es::stream_pool_t pool;
+    es_km_stream_pool(int device, int n) : pool(device, n) {}
 };
 
 struct es_km_graph {
@@ -601,6 +612,98 @@ int es_km_graph_node_info(es_km_graph_t* g, int id, int* position, int* stream, 
 int es_km_graph_cross_stream_waits(es_km_graph_t* g)
 {
     return g ? g->graph->n_cross_stream_waits() : ES_KM_ERR_INVALID;
+}
+
+int es_km_graph_launch_node(es_km_graph_t* g, int id, void* stream, void* arena, void* workspace,
+                            uint64_t workspace_bytes, int first_in_group,
+                            es_km_callback_t callback, void* user)
+{
+    return guarded(g ? g->owner : nullptr, [&]() -> int {
+        if (!g) throw es::ir_error("null graph");
+        if (!arena) throw es::ir_error("graph launch: null arena");
+        g->graph->launch_node(id, static_cast<hipStream_t>(stream), arena, workspace,
+                              workspace_bytes, first_in_group, callback, user);
+        return ES_KM_OK;
+    });
+}
+
+int es_km_graph_node_workspace(es_km_graph_t* g, int id, uint64_t* workspace_bytes)
+{
+    return guarded(g ? g->owner : nullptr, [&]() -> int {
+        if (!g) throw es::ir_error("null graph");
+        if (id < 0 || id >= g->graph->n_nodes()) throw es::ir_error("graph: no such node");
+        if (workspace_bytes) *workspace_bytes = g->graph->node_workspace(id);
+        return ES_KM_OK;
+    });
+}
+
+int es_km_graph_node_group(es_km_graph_t* g, int id)
+{
+    if (!g || id < 0 || id >= g->graph->n_nodes()) return -1;
+    return g->graph->kind_of(id) == 1 ? g->graph->group_of(id) : -1;
+}
+
+es_km_workspace_pool_t* es_km_workspace_pool_create(int device)
+{
+    try {
+        return new es_km_workspace_pool(device);
+    } catch (std::exception const& e) {
+        g_null_error = e.what();
+        return nullptr;
+    }
+}
+
+void es_km_workspace_pool_destroy(es_km_workspace_pool_t* p) { delete p; }
+
+void* es_km_workspace_pool_acquire(es_km_workspace_pool_t* p, uint64_t bytes, uint64_t* got_bytes)
+{
+    try {
+        if (!p) throw es::ir_error("null pool");
+        return p->pool.acquire(bytes, got_bytes);
+    } catch (std::exception const& e) {
+        g_null_error = e.what();
+        return nullptr;
+    }
+}
+
+int es_km_workspace_pool_release(es_km_workspace_pool_t* p, void* block)
+{
+    return guarded(nullptr, [&]() -> int {
+        if (!p) throw es::ir_error("null pool");
+        p->pool.release(block);
+        return ES_KM_OK;
+    });
+}
+
+int es_km_workspace_pool_blocks(es_km_workspace_pool_t* p)
+{
+    return p ? p->pool.n_blocks() : ES_KM_ERR_INVALID;
+}
+
+es_km_stream_pool_t* es_km_stream_pool_create(int device, int n_streams)
+{
+    try {
+        return new es_km_stream_pool(device, n_streams);
+    } catch (std::exception const& e) {
+        g_null_error = e.what();
+        return nullptr;
+    }
+}
+
+void es_km_stream_pool_destroy(es_km_stream_pool_t* p) { delete p; }
+
+void* es_km_stream_pool_try_acquire(es_km_stream_pool_t* p)
+{
+    return p ? static_cast<void*>(p->pool.try_acquire()) : nullptr;
+}
+
+int es_km_stream_pool_release(es_km_stream_pool_t* p, void* stream)
+{
+    return guarded(nullptr, [&]() -> int {
+        if (!p) throw es::ir_error("null pool");
+        p->pool.release(static_cast<hipStream_t>(stream));
+        return ES_KM_OK;
+    });
 }
 
 int es_km_graph_launches(es_km_graph_t* g)

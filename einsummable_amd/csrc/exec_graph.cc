@@ -96,6 +96,7 @@ int apply_graph_t::add_touch(touch_t const& t, int group, std::vector<mem_t> con
             if (nodes_[i].kind == kind_t::touch && nodes_[i].group == group) previous = i;
         }
     }
+    n.group_castable = t.castable;
     if (previous < 0) {
         n.touch.castable = std::nullopt;
     } else {
@@ -384,6 +385,53 @@ void apply_graph_t::finalize(int n_streams)
         }
     }
     finalized_ = true;
+}
+
+uint64_t apply_graph_t::node_workspace(int id) const
+{
+    node_t const& n = nodes_[size_t(id)];
+    if (n.kind != kind_t::einsummable || !km_) return 0;
+    return km_->workspace_size(n.e);
+}
+
+void apply_graph_t::launch_node(int id, hipStream_t stream, void* arena_, void* workspace,
+                                uint64_t workspace_bytes, int first_in_group,
+                                void (*callback)(void*), void* user) const
+{
+    if (!finalized_) throw km_error(km_status::not_built, "apply graph: launch before finalize");
+    if (!km_) throw km_error(km_status::device, "apply graph: planned without a kernel manager");
+    if (id < 0 || id >= int(nodes_.size())) throw km_error(km_status::invalid, "no such node");
+    char* const   arena = static_cast<char*>(arena_);
+    node_t const& n = nodes_[size_t(id)];
+    switch (n.kind) {
+        case kind_t::einsummable: {
+            plan_t const* p = km_->plan_of(n.e);
+            if (!p) throw km_error(km_status::not_built, "apply graph: einsummable not built");
+            std::vector<void const*> ptrs;
+            for (size_t i = 1; i != n.mems.size(); ++i) ptrs.push_back(arena + n.mems[i].offset);
+            km_->run_plan(*p, stream, arena + n.mems[0].offset, ptrs.data(), int(ptrs.size()),
+                          workspace, workspace_bytes);
+            break;
+        }
+        case kind_t::touch: {
+            touch_t t = n.touch;
+            if (n.group >= 0 && first_in_group >= 0) {
+                // the graph cleared the castable of the first member inserted; the caller's
+                // group manager says which one really runs first
+                if (first_in_group) {
+                    t.castable = std::nullopt;
+                } else if (!t.castable) {
+                    t.castable = n.group_castable;
+                }
+            }
+            (*km_)(t, stream, arena + n.mems[0].offset, arena + n.mems[1].offset);
+            break;
+        }
+        default:
+            launch(n, stream, arena);
+            break;
+    }
+    if (callback) check(hipLaunchHostFunc(stream, callback, user), "hipLaunchHostFunc");
 }
 
 int apply_graph_t::n_launches() const

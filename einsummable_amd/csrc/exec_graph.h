@@ -86,6 +86,23 @@ public:
     // `main` is ordered after all of it on return; nothing synchronises with the host.
     void run(hipStream_t main, void* arena) const;
 
+    // One node at a time, for a host event loop that keeps the dependencies itself (the
+    // reference's exec_state_t, src/engine/exec_state.cc:197-219): enqueues node `id` on
+    // `stream` -- no waits, no events; the caller launches a node when everything it depends
+    // on has reported back -- and, behind it on the same stream, a host function that calls
+    // `callback(user)` when the node's work is done (gpu_einsummable_t::launch and
+    // gpu_touch_t::launch, src/engine/gpu/exec_graph.cc:277-335, 354-404, with
+    // cudaStreamAddCallback).  The callback runs on a thread of the HIP runtime and must not
+    // call the HIP API.  `workspace`: at least node_workspace(id) bytes, the caller's (from
+    // its pool); unused by nodes that need none.  `first_in_group`: for a grouped touch, 1
+    // clears the castable (the first touch of a group to run initialises the output,
+    // managers.cc:3-21), 0 keeps it, -1 takes what insertion order said.  After finalize.
+    void launch_node(int id, hipStream_t stream, void* arena, void* workspace,
+                     uint64_t workspace_bytes, int first_in_group, void (*callback)(void*),
+                     void* user) const;
+    uint64_t node_workspace(int id) const;
+    int      group_of(int id) const { return nodes_[id].group; }
+
     int n_nodes() const { return int(nodes_.size()); }
     // smallest arena that holds every range a node touches
     uint64_t arena_bytes() const;
@@ -108,6 +125,7 @@ private:
         kind_t             kind;
         einsummable_t      e;
         touch_t            touch;
+        std::optional<castable_t> group_castable;  // as given, before the first member's is cleared
         int                group = -1;
         dtype_t            dtype = dtype_t::f32;
         uint64_t           bits0 = 0, bits1 = 0, n0 = 0, n1 = 0;

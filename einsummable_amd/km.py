@@ -40,6 +40,18 @@ EXPORTS = [
     "es_km_graph_node_info",
     "es_km_graph_cross_stream_waits",
     "es_km_graph_launches",
+    "es_km_graph_launch_node",
+    "es_km_graph_node_workspace",
+    "es_km_graph_node_group",
+    "es_km_workspace_pool_create",
+    "es_km_workspace_pool_destroy",
+    "es_km_workspace_pool_acquire",
+    "es_km_workspace_pool_release",
+    "es_km_workspace_pool_blocks",
+    "es_km_stream_pool_create",
+    "es_km_stream_pool_destroy",
+    "es_km_stream_pool_try_acquire",
+    "es_km_stream_pool_release",
     "es_km_graph_add_dummy",
     "es_km_graph_add_evict",
     "es_km_graph_add_load",
@@ -186,6 +198,22 @@ def load_library():
     lib.es_km_graph_node_info.argtypes = [V, I, V, V, V, I, V]
     lib.es_km_graph_cross_stream_waits.argtypes = [V]
     lib.es_km_graph_launches.argtypes = [V]
+    lib.es_km_graph_launch_node.argtypes = [V, I, V, V, V, U64, I, V, V]
+    lib.es_km_graph_node_workspace.argtypes = [V, I, V]
+    lib.es_km_graph_node_group.argtypes = [V, I]
+    lib.es_km_workspace_pool_create.restype = V
+    lib.es_km_workspace_pool_create.argtypes = [I]
+    lib.es_km_workspace_pool_destroy.argtypes = [V]
+    lib.es_km_workspace_pool_acquire.restype = V
+    lib.es_km_workspace_pool_acquire.argtypes = [V, U64, V]
+    lib.es_km_workspace_pool_release.argtypes = [V, V]
+    lib.es_km_workspace_pool_blocks.argtypes = [V]
+    lib.es_km_stream_pool_create.restype = V
+    lib.es_km_stream_pool_create.argtypes = [I, I]
+    lib.es_km_stream_pool_destroy.argtypes = [V]
+    lib.es_km_stream_pool_try_acquire.restype = V
+    lib.es_km_stream_pool_try_acquire.argtypes = [V]
+    lib.es_km_stream_pool_release.argtypes = [V, V]
     lib.es_km_graph_add_dummy.argtypes = [V, U64, U64, V, I]
     lib.es_km_graph_add_evict.argtypes = [V, U64, U64, I, V, I]
     lib.es_km_graph_add_load.argtypes = [V, I, U64, U64, V, I]
@@ -438,6 +466,62 @@ class KernelManager:
             self._fail(rc)
 
 
+NodeCallback = ctypes.CFUNCTYPE(None, ctypes.c_void_p)
+
+
+class WorkspacePool:
+    """gpu_workspace_manager_t (src/engine/gpu/workspace.cc:48-91) over the C ABI."""
+
+    def __init__(self, device=0):
+        self._lib = load_library()
+        self._p = self._lib.es_km_workspace_pool_create(int(device))
+        if not self._p:
+            raise KmError(ERR_DEVICE, self._lib.es_km_last_error(None).decode("utf-8", "replace"))
+
+    def acquire(self, nbytes):
+        got = ctypes.c_uint64(0)
+        ptr = self._lib.es_km_workspace_pool_acquire(self._p, int(nbytes), ctypes.byref(got))
+        if not ptr:
+            raise KmError(ERR_DEVICE, self._lib.es_km_last_error(None).decode("utf-8", "replace"))
+        return ptr, got.value
+
+    def release(self, ptr):
+        rc = self._lib.es_km_workspace_pool_release(self._p, ptr)
+        if rc != OK:
+            raise KmError(rc, self._lib.es_km_last_error(None).decode("utf-8", "replace"))
+
+    def blocks(self):
+        return self._lib.es_km_workspace_pool_blocks(self._p)
+
+    def close(self):
+        if self._p:
+            self._lib.es_km_workspace_pool_destroy(self._p)
+            self._p = None
+
+
+class StreamPool:
+    """streampool_manager_t (src/engine/gpu/stream_pool.cc:42-75) over the C ABI."""
+
+    def __init__(self, device=0, n_streams=4):
+        self._lib = load_library()
+        self._p = self._lib.es_km_stream_pool_create(int(device), int(n_streams))
+        if not self._p:
+            raise KmError(ERR_DEVICE, self._lib.es_km_last_error(None).decode("utf-8", "replace"))
+
+    def try_acquire(self):
+        return self._lib.es_km_stream_pool_try_acquire(self._p)
+
+    def release(self, stream):
+        rc = self._lib.es_km_stream_pool_release(self._p, stream)
+        if rc != OK:
+            raise KmError(rc, self._lib.es_km_last_error(None).decode("utf-8", "replace"))
+
+    def close(self):
+        if self._p:
+            self._lib.es_km_stream_pool_destroy(self._p)
+            self._p = None
+
+
 class ApplyGraph:
     """The exec-node layer (include/es_km.h, es_km_graph_*): apply / fill / copy nodes over
     one device arena with dependencies, placed on a pool of streams at finalize() and
@@ -531,6 +615,23 @@ class ApplyGraph:
 
     def launches(self):
         return self._check(self._lib.es_km_graph_launches(self._g))
+
+    def node_workspace(self, i):
+        ws = ctypes.c_uint64(0)
+        self._check(self._lib.es_km_graph_node_workspace(self._g, int(i), ctypes.byref(ws)))
+        return ws.value
+
+    def node_group(self, i):
+        return self._lib.es_km_graph_node_group(self._g, int(i))
+
+    def launch_node(self, i, stream, arena, workspace=None, first_in_group=-1, callback=None,
+                    user=None):
+        """Enqueue one node on `stream`; `callback` is a NodeCallback (keep it alive until it
+        has run) called with `user` (an int) when the node's work is done."""
+        ws_ptr, ws_size = workspace if workspace else (None, 0)
+        self._check(self._lib.es_km_graph_launch_node(
+            self._g, int(i), stream, arena, ws_ptr, ws_size, int(first_in_group),
+            ctypes.cast(callback, ctypes.c_void_p) if callback is not None else None, user))
 
     def add_dummy(self, mem=(0, 0), deps=None):
         d, nd = self._deps(deps)

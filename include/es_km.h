@@ -235,6 +235,49 @@ int es_km_graph_cross_stream_waits(es_km_graph_t* g);
  * (src/engine/gpu/exec_graph.cc:354-404 issues them one by one). */
 int es_km_graph_launches(es_km_graph_t* g);
 
+/* One node at a time, for a host event loop that keeps the dependencies itself.
+ *   gpu_einsummable_t::launch(resources, callback)   src/engine/gpu/exec_graph.cc:277-335
+ *   gpu_touch_t::launch (first-in-group decided by the group manager at run time)
+ *                                                    src/engine/gpu/exec_graph.cc:354-404,
+ *                                                    src/engine/managers.cc:3-21
+ *   gpu_constant_t / gpu_lowerTri_t / gpu_copy_t / gpu_evict_t / gpu_load_t ::launch
+ *                                                    src/engine/gpu/exec_graph.cc:600-690, 482-577
+ * Enqueues node `id` of a finalized graph on `stream` -- no waits and no events: the caller
+ * launches a node once every node it depends on (es_km_graph_node_info) has called back --
+ * followed on the same stream by a host function (hipLaunchHostFunc; the reference uses
+ * cudaStreamAddCallback) that calls callback(user) when the node's work is done.  The
+ * callback runs on a thread of the HIP runtime and must not call the HIP API; NULL asks for
+ * none.  workspace: at least es_km_graph_node_workspace(id) bytes, from the caller's pool,
+ * ignored by nodes that need none.  first_in_group, for a touch in a group: 1 clears its
+ * castable (the first touch of a group to run initialises the output), 0 keeps the castable
+ * it was added with, -1 takes what insertion order said (the first member inserted). */
+typedef void (*es_km_callback_t)(void* user);
+int es_km_graph_launch_node(es_km_graph_t* g, int id, void* stream, void* arena, void* workspace,
+                            uint64_t workspace_bytes, int first_in_group,
+                            es_km_callback_t callback, void* user);
+int es_km_graph_node_workspace(es_km_graph_t* g, int id, uint64_t* workspace_bytes);
+int es_km_graph_node_group(es_km_graph_t* g, int id);   /* the touch's group, or -1 */
+
+/* The resource pools such an event loop draws from.
+ *   gpu_workspace_manager_t: the first free block that is large enough, else a new device
+ *     allocation; released blocks are kept for reuse and freed with the pool
+ *                                                    src/engine/gpu/workspace.cc:48-91
+ *   streampool_t / streampool_manager_t: a fixed set of streams, try-acquire hands out a
+ *     free one or nothing                            src/engine/gpu/stream_pool.cc:8-75
+ * Both are safe to use from several threads. */
+typedef struct es_km_workspace_pool es_km_workspace_pool_t;
+typedef struct es_km_stream_pool    es_km_stream_pool_t;
+es_km_workspace_pool_t* es_km_workspace_pool_create(int device);
+void                    es_km_workspace_pool_destroy(es_km_workspace_pool_t* p);
+/* NULL on failure (es_km_last_error(NULL)); *got_bytes receives the block's real size */
+void* es_km_workspace_pool_acquire(es_km_workspace_pool_t* p, uint64_t bytes, uint64_t* got_bytes);
+int   es_km_workspace_pool_release(es_km_workspace_pool_t* p, void* block);
+int   es_km_workspace_pool_blocks(es_km_workspace_pool_t* p);
+es_km_stream_pool_t* es_km_stream_pool_create(int device, int n_streams);
+void                 es_km_stream_pool_destroy(es_km_stream_pool_t* p);
+void* es_km_stream_pool_try_acquire(es_km_stream_pool_t* p);   /* a hipStream_t, or NULL */
+int   es_km_stream_pool_release(es_km_stream_pool_t* p, void* stream);
+
 /* Nodes that launch nothing and only carry dependencies (dummy_t, which the reference makes
  * of inputmem / inputsto / partialize / alloc / del nodes, src/engine/gpu/exec_graph.cc:94-97).
  * The range is kept for inspection and takes no part in add_memory_dependencies. */

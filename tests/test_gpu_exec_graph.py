@@ -60,6 +60,41 @@ def add_nodes(g, nodes):
     return ids
 
 
+def oracle_run(nodes, init):
+    """The same node list applied one after the other by the CPU oracle; returns the arena."""
+    import oracle
+
+    arena = init.copy()
+    slot = lambda k: arena[k * N:(k + 1) * N]
+    seen_groups = set()
+    for kind, out, a, b in nodes:
+        if kind == "unary":
+            slot(out)[:] = oracle.einsummable([N], [[0]], 1, "*[constant{f32|0.5},hole|f32@0]",
+                                              None, [slot(a).copy()], oracle.EXACT)
+        elif kind == "binary":
+            slot(out)[:] = oracle.einsummable([N], [[0], [0]], 1, "+[hole|f32@0,hole|f32@1]", None,
+                                              [slot(a).copy(), slot(b).copy()], oracle.EXACT)
+        elif kind == "reduce":
+            slot(out)[:64] = oracle.einsummable([64, N // 64], [[0, 1]], 1, "hole|f32@0", "^",
+                                                [slot(a).copy()], oracle.EXACT)
+        elif kind == "copy":
+            slot(out)[:] = slot(a)
+        elif kind == "touch":
+            dims = [(128, 128, 0, 0, 128), (N // 128, N // 128, 3, 5, 40)]
+            o = np.ascontiguousarray(slot(out))
+            oracle.touch(dims, None, o, np.ascontiguousarray(slot(a)))
+            slot(out)[:] = o
+        elif kind == "group":
+            o = np.ascontiguousarray(slot(out))
+            oracle.touch([(N, N, 0, 0, N)], "+" if out in seen_groups else None, o,
+                         np.ascontiguousarray(slot(a)))
+            seen_groups.add(out)
+            slot(out)[:] = o
+        else:
+            slot(out)[:] = oracle.fill_constant(np.float32, 1.25, N)
+    return arena
+
+
 @pytest.mark.parametrize("seed", range(6))
 def test_random_graphs_give_the_sequential_bytes_on_any_number_of_streams(km, seed):
     import torch
@@ -85,6 +120,99 @@ def test_random_graphs_give_the_sequential_bytes_on_any_number_of_streams(km, se
     assert np.array_equal(results[0].view(np.uint32), results[1].view(np.uint32))
     assert np.array_equal(results[0].view(np.uint32), results[2].view(np.uint32))
     assert not np.array_equal(results[0], init)
+    # every operation of these graphs is a single exactly rounded f32 operation, a maximum or
+    # a move: the oracle's arena must hold the same values (a product may differ in the sign
+    # of a zero)
+    want = oracle_run(nodes, init)
+    assert np.array_equal(results[0], want)
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_a_host_event_loop_drives_the_nodes_one_by_one_through_completion_callbacks(km, seed):
+    # what the reference's exec_state_t does (src/engine/exec_state.cc:197-219): launch a
+    # node when everything it depends on has reported back, on a stream and with a workspace
+    # taken from pools, and learn of its completion through a callback behind it on the stream
+    import queue
+
+    import torch
+
+    r = rng(140 + seed)
+    n_slots = 12
+    nodes = random_graph(r, 60, n_slots)
+    init = normal(r, n_slots * N, np.float32)
+    g = ea.ApplyGraph(km)
+    ids = add_nodes(g, nodes)
+    g.add_memory_dependencies()
+    g.finalize(1)
+    deps = {i: set(g.node_info(i)[2]) for i in ids}
+    users = {i: [j for j in ids if i in deps[j]] for i in ids}
+    arena = torch.from_numpy(init.copy()).cuda()
+    torch.cuda.synchronize()
+
+    streams, workspaces = ea.StreamPool(0, 3), ea.WorkspacePool(0)
+    done = queue.Queue()
+    callback = ea.NodeCallback(lambda user: done.put(int(user) - 1))
+    waiting = {i: len(deps[i]) for i in ids}
+    ready = [i for i in ids if waiting[i] == 0]
+    held, started_groups, in_flight, finished, order = {}, set(), 0, 0, []
+    while finished != len(ids):
+        while ready:
+            s = streams.try_acquire()
+            if not s:
+                break
+            i = ready.pop(int(r.randint(0, len(ready))))     # any ready node may go next
+            need = g.node_workspace(i)
+            ws = workspaces.acquire(need) if need else None
+            group = g.node_group(i)
+            first = -1
+            if group >= 0:
+                first = 0 if group in started_groups else 1
+                started_groups.add(group)
+            g.launch_node(i, s, arena.data_ptr(), ws, first, callback, i + 1)
+            held[i] = (s, ws)
+            in_flight += 1
+            order.append(i)
+        i = done.get(timeout=60)
+        s, ws = held.pop(i)
+        streams.release(s)
+        if ws:
+            workspaces.release(ws[0])
+        in_flight -= 1
+        finished += 1
+        for j in users[i]:
+            waiting[j] -= 1
+            if waiting[j] == 0:
+                ready.append(j)
+    torch.cuda.synchronize()
+    assert in_flight == 0 and sorted(order) == sorted(ids)
+    assert order != sorted(order) or len(ids) < 3          # the loop did reorder independent nodes
+    got = arena.cpu().numpy()
+    assert np.array_equal(got, oracle_run(nodes, init))
+    streams.close()
+    workspaces.close()
+
+
+def test_workspace_and_stream_pools(km):
+    pool = ea.WorkspacePool(0)
+    a, size_a = pool.acquire(1 << 20)
+    b, size_b = pool.acquire(1 << 16)
+    assert a != b and size_a >= 1 << 20 and size_b >= 1 << 16 and pool.blocks() == 2
+    pool.release(a)
+    c, size_c = pool.acquire(1 << 10)                       # the first free block that is large enough
+    assert c == a and size_c == size_a and pool.blocks() == 2
+    with pytest.raises(ea.KmError):
+        pool.release(12345)
+    pool.release(b)
+    pool.release(c)
+    pool.close()
+    streams = ea.StreamPool(0, 2)
+    s0, s1 = streams.try_acquire(), streams.try_acquire()
+    assert s0 and s1 and s0 != s1 and streams.try_acquire() is None
+    streams.release(s0)
+    with pytest.raises(ea.KmError):
+        streams.release(s0)                                 # not out
+    assert streams.try_acquire() == s0
+    streams.close()
 
 
 def test_touch_groups_first_member_initialises_then_members_accumulate_in_order(km):
