@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the apply-node kernel path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c1|c3|c4|all]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c1|c3|c4|c5|llama|build|all]
 
 The headline workload is the fused elementwise + reduce configuration (f16, 8192 x 8192):
 one "step" runs its four apply nodes through the C-ABI kernel manager on buffers that are
@@ -12,8 +12,11 @@ already resident in HBM:
     (iv)  ij->i       row sum of (iii)
 `value` is algorithmic bytes per step / wall time per step (host launch cost included).
 `roofline` is the dominant kernel -- node (i) -- timed with events on the launch stream.
-`cpu_baseline` times the CPU oracle (a single-threaded C port of the reference semantics) on
-a bounded sample of the same workload.  Other workloads are reported under "others".
+`cpu_baseline` times the reference CPU executor's loops, ported as -O3 C with OpenMP
+(oracle/es_cpu_loops.c), over the same workload on all host cores; the same loops on one
+thread, the scalar interpreter and the other configurations' baselines are under
+"others.cpu_baselines".  Other workloads are reported under "others", and "others.targets"
+lists every numeric target with the worst measurement that answers it.
 """
 import argparse
 import json
@@ -43,7 +46,8 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="all",
-                    choices=["c2", "c1", "c3", "c4", "c5", "llama", "copy", "mfma_peak", "all"])
+                    choices=["c2", "c1", "c3", "c4", "c5", "llama", "copy", "mfma_peak", "build",
+                             "all"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     return ap.parse_args()
 
@@ -175,9 +179,49 @@ def run_c2(km, steps, warmup):
             "tensors": (x, y, m)}
 
 
-def cpu_baseline_c2(rows=8192):
-    """The CPU oracle (kind "port": a single-threaded C restatement of the reference's scalar
-    interpreter semantics) on the first `rows` rows of the same four nodes."""
+def cpu_loops_c2(threads, reps):
+    """The four C2 nodes through the -O3 / AVX2 / OpenMP loops of oracle/es_cpu_loops.c (a port
+    of the reference CPU executor's loops, kernel_executor.cc:786-914, 1163-1253) over the
+    whole 8192 x 8192 configuration: seconds per step."""
+    import numpy as np
+
+    import oracle
+
+    n = 8192
+    r = np.random.default_rng(0)
+    x = r.standard_normal((n, n), dtype=np.float32).astype(np.float16)
+    y = r.standard_normal((n, n), dtype=np.float32).astype(np.float16)
+
+    def step():
+        oracle.loops_relu_mul(x, y, threads)
+        m = oracle.loops_rowmax(x, threads)
+        ex = oracle.loops_exp_sub(x, m, threads)
+        oracle.loops_rowsum(ex, threads)
+
+    step()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        step()
+    return (time.perf_counter() - t0) / reps
+
+
+def cpu_baseline_c2():
+    """The reported CPU baseline of the headline configuration: the reference CPU executor's
+    loops as -O3 C (kind "port") on all host cores, whole workload."""
+    import oracle
+
+    n = 8192
+    cores = oracle.cpu_loops().es_cpu_max_threads()
+    dt = cpu_loops_c2(0, 3)
+    nbytes = n * n * 2 * (3 + 1 + 2 + 1) + 3 * n * 2
+    return {"value": round(nbytes / dt / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": "all four nodes over all 8192 rows, -O3 AVX2/F16C loops with OpenMP over "
+                      "rows, mean of 3 steps of %.3f s" % dt}
+
+
+def cpu_interpreter_c2(rows=512):
+    """The CPU oracle (a single-threaded C restatement of the reference's scalar interpreter,
+    every fp16 operation rounded in software) on the first `rows` rows of the same four nodes."""
     import numpy as np
 
     import oracle
@@ -194,8 +238,8 @@ def cpu_baseline_c2(rows=8192):
     dt = time.perf_counter() - t0
     nbytes = rows * n * 2 * (3 + 1 + 2 + 1) + 3 * rows * 2
     return {"value": round(nbytes / dt / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": "%s of the four nodes, %.1f s" % (
-                "all 8192 rows" if rows == 8192 else "first %d of 8192 rows" % rows, dt)}
+            "sample": "first %d of 8192 rows of the four nodes through the scalar interpreter, "
+                      "%.1f s" % (rows, dt)}
 
 
 def cpu_baselines_other_configs():
@@ -210,6 +254,54 @@ def cpu_baselines_other_configs():
 
     out = {}
     r = np.random.RandomState(1)
+    cores = oracle.cpu_loops().es_cpu_max_threads()
+    # C2 again: the loops on one thread (what one apply node of the reference gets), and the
+    # scalar interpreter
+    n2 = 8192
+    c2_bytes = n2 * n2 * 2 * (3 + 1 + 2 + 1) + 3 * n2 * 2
+    dt = cpu_loops_c2(1, 1)
+    out["c2_loops_1_thread"] = {"value": round(c2_bytes / dt / 1e9, 2), "unit": "GB/s", "cores": 1,
+                                "kind": "port", "sample": "all four nodes, all rows, %.2f s" % dt}
+    out["c2_interpreter"] = cpu_interpreter_c2()
+    # C3a through the row-copy loop, whole tensor, one thread and all cores
+    rg = np.random.default_rng(1)
+    xa = rg.standard_normal((32, 2048, 32, 128), dtype=np.float32).astype(np.float16)
+    for label, threads in (("1_thread", 1), ("all_cores", 0)):
+        oracle.loops_permute_acbd(xa[:2], threads)
+        t0 = time.perf_counter()
+        oracle.loops_permute_acbd(xa, threads)
+        dt = time.perf_counter() - t0
+        out["c3a_loops_" + label] = {"value": round(2 * xa.nbytes / dt / 1e9, 2), "unit": "GB/s",
+                                     "cores": threads or cores, "kind": "port",
+                                     "sample": "whole 32x2048x32x128 permute, %.3f s" % dt}
+    del xa
+    # C3b: all 64 touches through the row loop
+    accl = np.zeros((4096, 4096), np.float16)
+    blks = [rg.standard_normal((512, 512), dtype=np.float32).astype(np.float16) for _ in range(8)]
+    offl = [(int(r.randint(0, 3585)), int(r.randint(0, 3585))) for _ in range(64)]
+    for label, threads in (("1_thread", 1), ("all_cores", 0)):
+        t0 = time.perf_counter()
+        for _ in range(5):
+            for k, (ro, co) in enumerate(offl):
+                oracle.loops_touch_add(accl, blks[k % 8], ro, co, threads)
+        dt = (time.perf_counter() - t0) / 5
+        out["c3b_loops_" + label] = {"value": round(64 * 3 * 512 * 512 * 2 / dt / 1e9, 2),
+                                     "unit": "GB/s", "cores": threads or cores, "kind": "port",
+                                     "sample": "all 64 touches, mean of 5, %.4f s" % dt}
+    # f16 contractions on the host: fp32 GEMM on up-converted inputs (the reference's
+    # cblas_hgemm path is not available here), LLaMA projection 2048 x 4096 x 4096
+    pa = torch.from_numpy(rg.standard_normal((2048, 4096), dtype=np.float32))
+    pb = torch.from_numpy(rg.standard_normal((4096, 4096), dtype=np.float32))
+    torch.matmul(pa, pb.t())
+    t0 = time.perf_counter()
+    for _ in range(3):
+        torch.matmul(pa, pb.t())
+    dt = (time.perf_counter() - t0) / 3
+    out["f16_projection_host_blas_fp32"] = {
+        "value": round(2 * 2048 * 4096 * 4096 / dt / 1e12, 4), "unit": "TFLOP/s",
+        "cores": torch.get_num_threads(), "kind": "host_blas",
+        "sample": "2048x4096x4096 ij,kj->ik as fp32 on the host BLAS, %.3f s" % dt}
+    del pa, pb
     # C1: 64 of the 2048 rows of A through the oracle; the whole product through the BLAS
     n, rows = 2048, 64
     A = r.uniform(-1, 1, (n, n)).astype(np.float32)
@@ -263,7 +355,7 @@ def cpu_baselines_other_configs():
     return out
 
 
-def run_contraction(km, name, e, shapes, dtype, flops, steps, warmup):
+def run_contraction(km, name, e, shapes, dtype, flops, steps, warmup, yardstick=None):
     import torch
 
     tdt = {"f16": torch.float16, "f32": torch.float32, "f64": torch.float64}[dtype]
@@ -289,8 +381,21 @@ def run_contraction(km, name, e, shapes, dtype, flops, steps, warmup):
     torch.cuda.synchronize()
     ms = t.mean_ms()
     tf = flops / ms / 1e9
-    return {"node": name, "kernel": km.describe(e), "flop": flops, "ms": round(ms, 5),
-            "TFLOPs": round(tf, 2), "mfma_frac": round(tf / PEAK_TFLOPS[dtype], 4)}
+    row = {"node": name, "kernel": km.describe(e), "flop": flops, "ms": round(ms, 5),
+           "TFLOPs": round(tf, 2), "mfma_frac": round(tf / PEAK_TFLOPS[dtype], 4)}
+    nbytes = sum(t_.numel() * t_.element_size() for t_ in ins) + out.numel() * out.element_size()
+    row["hbm_frac"] = round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4)
+    if yardstick is not None:
+        # the vendor library's GEMM (torch.matmul -> hipBLASLt) on the same operands, as a
+        # yardstick only: nothing here calls it outside this measurement
+        fn = lambda: yardstick(*ins)
+        warm(fn, warmup)
+        t = Timed()
+        for _ in range(steps):
+            t.record(fn)
+        torch.cuda.synchronize()
+        row["torch_matmul_TFLOPs"] = round(flops / t.mean_ms() / 1e9, 2)
+    return row
 
 
 def run_c1(km, steps, warmup):
@@ -480,8 +585,13 @@ def run_c4(km, steps, warmup):
         ms = t.mean_ms()
         r = {"node": "c4 " + name, "kernel": km.describe(e), "ms": round(ms, 5)}
         if unit == "flop":
+            # both attention products are bound by HBM (1 GiB of scores written / read for
+            # 137 GFLOP): operand + result bytes over the time is the fraction that counts
+            nbytes = sum(mem[x].numel() * 2 for x in _i) + mem[_o].numel() * 2
             r.update(flop=work, TFLOPs=round(work / ms / 1e9, 2),
-                     mfma_frac=round(work / ms / 1e9 / PEAK_TFLOPS["f16"], 4))
+                     mfma_frac=round(work / ms / 1e9 / PEAK_TFLOPS["f16"], 4), bytes=nbytes,
+                     GBps=round(nbytes / ms / 1e6, 1),
+                     hbm_frac=round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4))
         else:
             r.update(bytes=work, GBps=round(work / ms / 1e6, 1),
                      hbm_frac=round(work / ms / 1e6 / HBM_PEAK_GBPS, 4))
@@ -568,8 +678,18 @@ def run_llama_contractions(km, steps, warmup):
         ("out proj adbe,cde->abc", E("adbe,cde->abc", dict(a=1, d=h, b=s, e=hd, c=d), mul, "+"),
          [(1, h, s, hd), (d, h, hd), (1, s, d)], 2 * s * d * d),
     ]
-    return [run_contraction(km, name, e, shapes, "f16", flops, steps, warmup)
-            for name, e, shapes, flops in cases]
+    import torch
+
+    nt = lambda a, b: torch.matmul(a, b.t())
+    yard = [nt, nt, nt, None, None, None]
+    rows = [run_contraction(km, name, e, shapes, "f16", flops, steps, warmup, y)
+            for (name, e, shapes, flops), y in zip(cases, yard)]
+    # the square products the tile rule and the roofline discussion refer to
+    E2 = ea.Einsummable.from_str
+    for n in (4096, 8192):
+        rows.append(run_contraction(km, "ij,kj->ik %d^3" % n, E2("ij,kj->ik", dict(i=n, j=n, k=n), mul, "+"),
+                                    [(n, n), (n, n), (n, n)], "f16", 2 * n ** 3, steps, warmup, nt))
+    return rows
 
 
 def run_c5(km, steps, warmup):
@@ -766,6 +886,82 @@ def run_copy(km, steps, warmup):
             "hbm_frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4)}
 
 
+BUILD_PROBE = r"""
+import json, sys, time
+sys.path.insert(0, %r)
+import torch
+import einsummable_amd as ea
+from einsummable_amd.llama_layer import LayerGraph
+torch.cuda.init()
+km = ea.KernelManager(0)
+g = LayerGraph()
+t0 = time.perf_counter()
+n = 0
+for node in g.nodes:
+    if node["kind"] == "einsummable":
+        km.build(node["e"])
+        n += 1
+print(json.dumps({"ms": (time.perf_counter() - t0) * 1e3, "einsummables": n}))
+"""
+
+
+def run_build_latency():
+    """Time of kernel_manager_t::build over the einsummables of the LLaMA-7B layer (runtime
+    compilation of the generated kernels is most of it), in a fresh process with an empty
+    code-object cache and again in a second process that finds the cache filled."""
+    import shutil
+    import subprocess
+    import tempfile
+
+    root = os.path.dirname(os.path.abspath(__file__))
+    cache = tempfile.mkdtemp(prefix="es_km_cache_")
+    out = {}
+    try:
+        env = dict(os.environ, ES_KM_CACHE_DIR=cache)
+        for label in ("first_process_empty_cache", "second_process_cache_on_disk"):
+            p = subprocess.run([sys.executable, "-c", BUILD_PROBE % root], env=env,
+                               capture_output=True, text=True, timeout=600)
+            if p.returncode != 0:
+                out[label] = {"error": p.stderr[-300:]}
+                continue
+            r = json.loads(p.stdout.strip().splitlines()[-1])
+            out[label] = {"build_ms": round(r["ms"], 1), "einsummables": r["einsummables"]}
+        out["code_objects_cached"] = len([f for f in os.listdir(cache) if f.endswith(".co")])
+    finally:
+        shutil.rmtree(cache, ignore_errors=True)
+    return out
+
+
+def targets_block(others):
+    """Every numeric target with the measurements that answer it, worst first, so that the
+    line cannot be read as its headline alone."""
+    mfma, hbm = [], []
+    for r in others.get("llama7b_contractions", []):
+        if "mfma_frac" in r and ("proj" in r["node"] or "w1" in r["node"] or "w2" in r["node"] or
+                                 "^3" in r["node"]):
+            mfma.append((r["mfma_frac"], r["node"], r.get("torch_matmul_TFLOPs")))
+    for key in ("c2_nodes", "c3", "c4", "column_reductions"):
+        for r in others.get(key, []):
+            if isinstance(r, dict) and "hbm_frac" in r and "[not part" not in r["node"]:
+                hbm.append((r["hbm_frac"], r["node"]))
+    mfma.sort()
+    hbm.sort()
+    out = {
+        "fp16_contractions_mfma_frac_target_0.60": {
+            "worst": mfma[0][0] if mfma else None, "best": mfma[-1][0] if mfma else None,
+            "rows": [{"node": n, "mfma_frac": f,
+                      "vendor_gemm_mfma_frac": round(t / PEAK_TFLOPS["f16"], 4) if t else None}
+                     for f, n, t in mfma]},
+        "memory_kernels_hbm_frac_target_0.70": {
+            "worst": hbm[0][0] if hbm else None,
+            "below_target": [{"node": n, "hbm_frac": f} for f, n in hbm if f < 0.70],
+            "at_or_above_target": len([1 for f, _ in hbm if f >= 0.70])},
+    }
+    if "c5" in others:
+        out["llama7b_layer_ms"] = others["c5"].get("layer_ms")
+    return out
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -817,6 +1013,9 @@ def main():
     if args.workload in ("llama", "all"):
         others["llama7b_contractions"] = run_llama_contractions(km, max(args.steps // 5, 3),
                                                                 max(args.warmup // 5, 1))
+    if args.workload in ("build", "all"):
+        others["build_latency_llama7b_layer"] = run_build_latency()
+    others["targets"] = targets_block(others)
 
     line = {
         "metric": "elementwise/reduce GB/s (apply-node kernel path; contraction TFLOP/s and "

@@ -323,3 +323,72 @@ def ref_permute(inn, out_perm):
         _u64(inn.shape), inn.ndim, _ints(out_perm), inn.dtype.itemsize,
         ctypes.c_void_p(out.ctypes.data), ctypes.c_void_p(inn.ctypes.data)))
     return out.reshape([inn.shape[p] for p in out_perm])
+
+
+# ---- optimised CPU loops for the reported CPU baseline (es_cpu_loops.c); benchmark
+# infrastructure like the rest of this package
+
+_loops = None
+
+
+def cpu_loops():
+    """The -O3 / AVX2 / OpenMP loops library (built on demand)."""
+    global _loops
+    if _loops is None:
+        path = os.path.join(_HERE, "libes_cpu_loops.so")
+        if not os.path.exists(path):
+            subprocess.run(["make", "-C", _HERE, "libes_cpu_loops.so"], check=True,
+                           capture_output=True)
+        lib = ctypes.CDLL(path)
+        P, Z, I = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int
+        lib.es_cpu_max_threads.restype = I
+        lib.es_cpu_relu_mul_f16.argtypes = [P, P, P, Z, I]
+        lib.es_cpu_rowmax_f16.argtypes = [P, P, Z, Z, I]
+        lib.es_cpu_exp_sub_f16.argtypes = [P, P, P, Z, Z, I]
+        lib.es_cpu_rowsum_f16.argtypes = [P, P, Z, Z, I]
+        lib.es_cpu_permute_acbd_2byte.argtypes = [P, P, Z, Z, Z, Z, I]
+        lib.es_cpu_touch_add_f16.argtypes = [P, Z, P, Z, Z, Z, Z, I]
+        _loops = lib
+    return _loops
+
+
+def _p(a):
+    assert a.flags["C_CONTIGUOUS"]
+    return ctypes.c_void_p(a.ctypes.data)
+
+
+def loops_relu_mul(x, y, threads=0):
+    out = np.empty_like(x)
+    cpu_loops().es_cpu_relu_mul_f16(_p(x), _p(y), _p(out), x.size, threads)
+    return out
+
+
+def loops_rowmax(x, threads=0):
+    out = np.empty(x.shape[0], np.float16)
+    cpu_loops().es_cpu_rowmax_f16(_p(x), _p(out), x.shape[0], x.shape[1], threads)
+    return out
+
+
+def loops_exp_sub(x, m, threads=0):
+    out = np.empty_like(x)
+    cpu_loops().es_cpu_exp_sub_f16(_p(x), _p(m), _p(out), x.shape[0], x.shape[1], threads)
+    return out
+
+
+def loops_rowsum(x, threads=0):
+    out = np.empty(x.shape[0], np.float16)
+    cpu_loops().es_cpu_rowsum_f16(_p(x), _p(out), x.shape[0], x.shape[1], threads)
+    return out
+
+
+def loops_permute_acbd(x, threads=0):
+    a, b, c, d = x.shape
+    out = np.empty((a, c, b, d), x.dtype)
+    cpu_loops().es_cpu_permute_acbd_2byte(_p(x), _p(out), a, b, c, d, threads)
+    return out
+
+
+def loops_touch_add(out, inn, ro, co, threads=0):
+    cpu_loops().es_cpu_touch_add_f16(_p(out), out.shape[1], _p(inn), inn.shape[0], inn.shape[1],
+                                     ro, co, threads)
+    return out

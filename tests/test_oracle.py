@@ -434,3 +434,29 @@ def test_fills_closed_form():
     # start == 0 on a square is numpy's tril
     m = oracle.fill_lowertri(np.float64, 1.0, 0.0, 6, 6, 0)
     assert np.array_equal(m, np.tril(np.ones((6, 6))))
+
+
+def test_cpu_baseline_loops_agree_with_the_oracle():
+    # the -O3 loops that bench.py times as the CPU baseline compute what the oracle computes
+    r = np.random.RandomState(5)
+    x = r.normal(0, 1, (37, 523)).astype(np.float16)
+    y = r.normal(0, 1, (37, 523)).astype(np.float16)
+    relu_mul = "*[ite_>=[constant{f16|0},hole|f16@0,constant{f16|0},hole|f16@0],hole|f16@1]"
+    want = oracle.einsummable([37, 523], [[0, 1], [0, 1]], 2, relu_mul, None, [x, y], oracle.EXACT)
+    for threads in (1, 3):
+        got = oracle.loops_relu_mul(x, y, threads)
+        assert np.array_equal(got.astype(np.float32), want.reshape(37, 523).astype(np.float32))
+        m = oracle.loops_rowmax(x, threads)
+        assert np.array_equal(m, x.max(axis=1))
+        e = oracle.loops_exp_sub(x, m, threads)
+        ref = np.exp(x.astype(np.float64) - m.astype(np.float64)[:, None])
+        assert np.allclose(e.astype(np.float64), ref, rtol=1e-2, atol=1e-7)
+        s = oracle.loops_rowsum(e, threads)
+        assert np.allclose(s.astype(np.float64), e.astype(np.float64).sum(axis=1), rtol=2e-3)
+        t = r.normal(0, 1, (3, 5, 4, 16)).astype(np.float16)
+        assert np.array_equal(oracle.loops_permute_acbd(t, threads), t.transpose(0, 2, 1, 3))
+        acc = r.normal(0, 1, (64, 96)).astype(np.float16)
+        blk = r.normal(0, 1, (20, 33)).astype(np.float16)
+        want_acc = oracle.touch([(20, 64, 0, 7, 20), (33, 96, 0, 11, 33)], "+", acc.copy(), blk)
+        assert np.array_equal(oracle.loops_touch_add(acc.copy(), blk, 7, 11, threads).view(np.uint16),
+                              want_acc.view(np.uint16))
