@@ -253,3 +253,21 @@ def test_load_errors():
     g.add_dummy()
     with pytest.raises(ea.KmError, match="must be empty"):
         g.load_memgraph(mp.to_wire(sample_memgraph()))
+
+
+def test_the_restated_schema_equals_the_reference_proto_field_for_field():
+    # tests/golden/einsummable_proto_fields.json is written from the reference's .proto text by
+    # tests/golden/make_proto_fields.py; the encoder of these tests is built from SCHEMA
+    import json
+    import os
+
+    import memgraph_proto
+
+    with open(os.path.join(os.path.dirname(__file__), "golden",
+                           "einsummable_proto_fields.json")) as f:
+        reference = json.load(f)
+    for message, fields in memgraph_proto.SCHEMA.items():
+        assert message in reference, message
+        mine = sorted((f[0], f[1], f[2], f[3], f[4] if len(f) == 5 else None) for f in fields)
+        theirs = sorted(tuple(f) for f in reference[message])
+        assert mine == theirs, (message, mine, theirs)
