@@ -575,6 +575,16 @@ int es_km_graph_add_memory_dependencies(es_km_graph_t* g)
     });
 }
 
+int es_km_graph_optimize(es_km_graph_t* g, int* n_absorbed)
+{
+    return guarded(g ? g->owner : nullptr, [&]() -> int {
+        if (!g) throw es::ir_error("null graph");
+        int const n = g->graph->optimize();
+        if (n_absorbed) *n_absorbed = n;
+        return ES_KM_OK;
+    });
+}
+
 int es_km_graph_finalize(es_km_graph_t* g, int n_streams)
 {
     return guarded(g ? g->owner : nullptr, [&]() -> int {
@@ -704,6 +714,18 @@ int es_km_stream_pool_release(es_km_stream_pool_t* p, void* stream)
         p->pool.release(static_cast<hipStream_t>(stream));
         return ES_KM_OK;
     });
+}
+
+int64_t es_km_graph_node_describe(es_km_graph_t* g, int id, char* out, uint64_t cap)
+{
+    if (!g || id < 0 || id >= g->graph->n_nodes()) return ES_KM_ERR_INVALID;
+    std::string const s = g->graph->describe(id);
+    if (out && cap) {
+        uint64_t const n = std::min<uint64_t>(cap - 1, s.size());
+        std::memcpy(out, s.data(), n);
+        out[n] = 0;
+    }
+    return int64_t(s.size());
 }
 
 int es_km_graph_launches(es_km_graph_t* g)

@@ -140,6 +140,15 @@ struct emitter_t {
             }
             case op_kind::convert: {
                 dtype_t from = n.children[0].dtype;
+                // A conversion to the dtype the value already has stands where two
+                // expressions were joined into one (scalarop_t::compose): the value is what a
+                // kernel would have stored and the next one loaded.  For f16 that is the
+                // rounding below; for the others the value is unchanged, but the compiler
+                // must not contract a product on one side with a sum on the other into one
+                // fused multiply-add, which rounds differently.
+                if (from == n.dtype && n.dtype != dtype_t::f16) {
+                    return define(n.dtype, "keep_apart(" + c[0] + ")");
+                }
                 if (n.dtype == dtype_t::f16) return define(n.dtype, "(float)(f16)(" + c[0] + ")");
                 if (n.dtype == dtype_t::f32) {
                     return define(n.dtype, from == dtype_t::f64 ? "(float)(" + c[0] + ")" : c[0]);
@@ -167,6 +176,17 @@ __device__ __forceinline__ c64 c_mul(c64 a, c64 b)
 {
     return c64{a.re * b.re - a.im * b.im, a.re * b.im + a.im * b.re};
 }
+__device__ __forceinline__ float keep_apart(float v)
+{
+    asm("" : "+v"(v));
+    return v;
+}
+__device__ __forceinline__ double keep_apart(double v)
+{
+    asm("" : "+v"(v));
+    return v;
+}
+__device__ __forceinline__ c64 keep_apart(c64 v) { return c64{keep_apart(v.re), keep_apart(v.im)}; }
 template <typename T, int N>
 struct __attribute__((aligned(sizeof(T) * N))) vec_t { T v[N]; };
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));

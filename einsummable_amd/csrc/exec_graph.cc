@@ -221,6 +221,17 @@ void apply_graph_t::storage_read(int storage_id, void* dst, uint64_t size) const
     std::memcpy(dst, s->host, size);
 }
 
+std::string apply_graph_t::describe(int id) const
+{
+    static const char* names[] = {"einsummable", "touch", "constant", "lowertri",
+                                  "copy",        "dummy", "evict",    "load"};
+    node_t const& n = nodes_[size_t(id)];
+    std::string   s = names[int(n.kind)];
+    for (mem_t const& m : n.mems) s += " " + std::to_string(m.offset) + ":" + std::to_string(m.size);
+    if (n.kind == kind_t::einsummable) s += " | " + n.e.key();
+    return s;
+}
+
 uint64_t apply_graph_t::arena_bytes() const
 {
     uint64_t need = 0;
@@ -252,6 +263,222 @@ void apply_graph_t::add_memory_dependencies()
         std::sort(nv.deps.begin(), nv.deps.end());
         nv.deps.erase(std::unique(nv.deps.begin(), nv.deps.end()), nv.deps.end());
     }
+}
+
+namespace
+{
+
+bool covers(mem_t const& a, mem_t const& b)
+{
+    return a.offset <= b.offset && b.offset + b.size <= a.offset + a.size;
+}
+
+bool same_range(mem_t const& a, mem_t const& b) { return a.offset == b.offset && a.size == b.size; }
+
+bool is_iota(std::vector<int> const& inn, int rank)
+{
+    if (int(inn.size()) != rank) return false;
+    for (int i = 0; i != rank; ++i) {
+        if (inn[size_t(i)] != i) return false;
+    }
+    return true;
+}
+
+bool is_increasing(std::vector<int> const& inn)
+{
+    for (size_t i = 1; i < inn.size(); ++i) {
+        if (inn[i] <= inn[i - 1]) return false;
+    }
+    return true;
+}
+
+// u: elementwise (no aggregation), every input straight or broadcast.
+bool absorbable_producer(einsummable_t const& u)
+{
+    if (u.has_aggregation() || u.join.has_variables()) return false;
+    for (auto const& inn : u.inns) {
+        if (!is_increasing(inn)) return false;
+    }
+    return true;
+}
+
+// The einsummable that computes v with u in place of its input k, or nothing when the two
+// do not line up.  v reads input k position by position over its join modes.
+std::optional<einsummable_t> merged(einsummable_t const& u, einsummable_t const& v, int k)
+{
+    int const Ru = int(u.join_shape.size());
+    int const Rv = int(v.join_shape.size());
+    if (u.out_dtype() != v.inn_dtype(k) || u.out_nelem() != v.inn_nelem(k)) return std::nullopt;
+    if (u.inns.size() + v.inns.size() - 1 > 6) return std::nullopt;
+    std::vector<std::vector<int>> u_inns = u.inns, v_inns = v.inns;
+    std::vector<uint64_t>         shape = v.join_shape;
+    int                           out_rank = v.out_rank;
+    auto all_iota = [](einsummable_t const& e) {
+        if (e.has_aggregation()) return false;
+        for (auto const& inn : e.inns) {
+            if (!is_iota(inn, int(e.join_shape.size()))) return false;
+        }
+        return true;
+    };
+    auto iota = [](int rank) {
+        std::vector<int> r(size_t(rank), 0);
+        for (int i = 0; i != rank; ++i) r[size_t(i)] = i;
+        return r;
+    };
+    if (u.join_shape == v.join_shape) {
+        // as they are
+    } else if (all_iota(v)) {
+        // v is a map over positions: it takes the shape u gives them
+        shape = u.join_shape;
+        out_rank = Ru;
+        for (auto& inn : v_inns) inn = iota(Ru);
+    } else if (all_iota(u)) {
+        for (auto& inn : u_inns) inn = iota(Rv);
+    } else {
+        return std::nullopt;
+    }
+    std::vector<std::vector<int>> inns = u_inns;
+    for (int i = 0; i != int(v_inns.size()); ++i) {
+        if (i != k) inns.push_back(v_inns[size_t(i)]);
+    }
+    try {
+        return einsummable_t::make(shape, inns, out_rank, scalarop_t::compose(v.join, k, u.join),
+                                   v.castable);
+    } catch (ir_error const&) {
+        return std::nullopt;
+    }
+}
+
+}  // namespace
+
+bool apply_graph_t::absorb_producer(int v)
+{
+    node_t& nv = nodes_[size_t(v)];
+    int const n = int(nodes_.size());
+    std::vector<int> candidates;  // indices into nv.mems
+    bool const copy = nv.kind == kind_t::touch;
+    if (copy) {
+        touch_t const t = nv.touch.simplify();
+        if (t.castable || t.selection.size() != 1) return false;
+        touchdim_t const& d = t.selection[0];
+        if (d.d_inn != d.size || d.d_out != d.size || d.offset_inn || d.offset_out) return false;
+        if (d.size * dtype_size(t.dtype) != nv.mems[0].size || nv.mems[1].size != nv.mems[0].size) {
+            return false;
+        }
+        for (int w = 0; nv.group >= 0 && w != n; ++w) {
+            if (w != v && nodes_[size_t(w)].kind == kind_t::touch && nodes_[size_t(w)].group == nv.group) {
+                return false;
+            }
+        }
+        candidates.push_back(1);
+    } else if (nv.kind == kind_t::einsummable) {
+        einsummable_t const& e = nv.e;
+        if (e.join.has_variables() || (e.has_aggregation() && e.inns.size() != 1)) return false;
+        for (int k = 0; k != int(e.inns.size()); ++k) {
+            if (is_iota(e.inns[size_t(k)], int(e.join_shape.size()))) candidates.push_back(k + 1);
+        }
+    }
+    for (int slot : candidates) {
+        mem_t const S = nv.mems[size_t(slot)];
+        if (S.size == 0) continue;
+        bool clean = true;
+        for (size_t i = 0; i != nv.mems.size(); ++i) {
+            if (int(i) != slot && overlaps(nv.mems[i], S)) clean = false;
+        }
+        if (!clean) continue;
+        // the node that wrote S: the last one before v to write any of it
+        int u = -1;
+        for (int w = v - 1; w >= 0 && u < 0; --w) {
+            node_t const& nw = nodes_[size_t(w)];
+            if (nw.kind == kind_t::dummy || nw.kind == kind_t::evict) continue;
+            if (overlaps(nw.mems[0], S)) u = w;
+        }
+        if (u < 0) continue;
+        node_t& nu = nodes_[size_t(u)];
+        if (nu.kind != kind_t::einsummable || !same_range(nu.mems[0], S)) continue;
+        if (!copy && !absorbable_producer(nu.e)) continue;
+        for (size_t i = 1; i != nu.mems.size(); ++i) {
+            // u reads at v's place now: not what it would write there, not its own old output
+            if (overlaps(nu.mems[i], nv.mems[0]) || overlaps(nu.mems[i], S)) clean = false;
+        }
+        // between the two: nobody else reads S, nobody writes what u reads
+        for (int w = u + 1; w < v && clean; ++w) {
+            node_t const& nw = nodes_[size_t(w)];
+            if (nw.kind == kind_t::dummy) continue;
+            for (size_t i = 1; i < nw.mems.size(); ++i) clean = clean && !overlaps(nw.mems[i], S);
+            if (nw.kind == kind_t::evict) continue;
+            for (size_t i = 1; i != nu.mems.size(); ++i) {
+                clean = clean && !overlaps(nw.mems[0], nu.mems[i]);
+            }
+        }
+        if (!clean) continue;
+        // after v: S is deleted before anybody reads or rewrites it
+        bool deleted = false;
+        for (int w = v + 1; w < n && clean && !deleted; ++w) {
+            node_t const& nw = nodes_[size_t(w)];
+            if (nw.kind == kind_t::dummy) {
+                deleted = covers(nw.mems[0], S) &&
+                          std::binary_search(nw.deps.begin(), nw.deps.end(), v);
+                continue;
+            }
+            for (size_t i = nw.kind == kind_t::evict ? 1 : 0; i < nw.mems.size(); ++i) {
+                clean = clean && !overlaps(nw.mems[i], S);
+            }
+        }
+        if (!clean || !deleted) continue;
+
+        einsummable_t fused = nu.e;
+        if (!copy) {
+            std::optional<einsummable_t> m = merged(nu.e, nv.e, slot - 1);
+            if (!m) continue;
+            fused = std::move(m.value());
+        }
+        if (km_ && !copy) {
+            try {
+                if (!km_->build(fused)) continue;
+            } catch (km_error const&) {
+                continue;
+            } catch (ir_error const&) {
+                continue;
+            }
+        }
+        std::vector<mem_t> mems{nv.mems[0]};
+        for (size_t i = 1; i != nu.mems.size(); ++i) mems.push_back(nu.mems[i]);
+        for (size_t i = 1; i != nv.mems.size(); ++i) {
+            if (!copy && int(i) != slot) mems.push_back(nv.mems[i]);
+        }
+        std::vector<int> deps = nv.deps;
+        deps.erase(std::remove(deps.begin(), deps.end(), u), deps.end());
+        deps.insert(deps.end(), nu.deps.begin(), nu.deps.end());
+        std::sort(deps.begin(), deps.end());
+        deps.erase(std::unique(deps.begin(), deps.end()), deps.end());
+        nv.kind = kind_t::einsummable;
+        nv.e = std::move(fused);
+        nv.mems = std::move(mems);
+        nv.deps = std::move(deps);
+        nv.group = -1;
+        nu.kind = kind_t::dummy;
+        nu.mems = {S};
+        // whoever waited for u to be done with its inputs waits for the node that reads them now
+        for (int w = v + 1; w < n; ++w) {
+            std::vector<int>& d = nodes_[size_t(w)].deps;
+            if (std::binary_search(d.begin(), d.end(), u) && !std::binary_search(d.begin(), d.end(), v)) {
+                d.insert(std::upper_bound(d.begin(), d.end(), v), v);
+            }
+        }
+        return true;
+    }
+    return false;
+}
+
+int apply_graph_t::optimize()
+{
+    if (finalized_) throw km_error(km_status::invalid, "apply graph: already finalized");
+    int absorbed = 0;
+    for (int v = 0; v != int(nodes_.size()); ++v) {
+        while (absorb_producer(v)) ++absorbed;
+    }
+    return absorbed;
 }
 
 void apply_graph_t::finalize(int n_streams)

@@ -78,6 +78,22 @@ public:
     // ranges imply (read after write, write after write, write after read).
     void add_memory_dependencies();
 
+    // Removes round trips through memory that the node list spells out but the results do not
+    // need, without changing one bit of what stays in memory.  A node v absorbs the node u
+    // that wrote one of its inputs when that range S is written by u alone, read by v alone
+    // and deleted afterwards -- a dummy that covers S and depends on v is read as S's del node
+    // (memgraph.h: del_t) -- and nothing between the two touches what u reads:
+    //  - v a touch that copies S whole (the formation / partialize copy that follows every
+    //    contraction and reduction, taskgraph.cc:3047-3061): u writes v's output itself;
+    //  - v an elementwise einsummable, or a reduction of one input, that takes S position by
+    //    position, and u elementwise: one einsummable whose join is v's with u's put in
+    //    place of the hole (scalarop_t::compose keeps the rounding a store and a load make).
+    // The merged node stands at v's place and u becomes a dummy, so ids, and dependencies on
+    // either, stay valid.  Einsummables the kernel manager cannot build stay as they are.
+    // Before finalize; returns the number of nodes absorbed.  The reference has no such pass
+    // at this level: its graphs reach the engine with these nodes in them.
+    int optimize();
+
     // Builds every einsummable on the kernel manager (throws km_error when one has no
     // kernel), fixes the launch order and places the nodes on `n_streams` streams.
     void finalize(int n_streams);
@@ -102,6 +118,10 @@ public:
                      void* user) const;
     uint64_t node_workspace(int id) const;
     int      group_of(int id) const { return nodes_[id].group; }
+
+    // "<kind> <range>..." -- the output first, "offset:size" each -- and for an einsummable
+    // its key (shape, castable, modes, join text) after " | "; for inspection and tests
+    std::string describe(int id) const;
 
     int n_nodes() const { return int(nodes_.size()); }
     // smallest arena that holds every range a node touches
@@ -146,6 +166,7 @@ private:
     };
 
     int  insert(node_t&& n, std::vector<int> const& deps);
+    bool absorb_producer(int v);
     void launch(node_t const& n, hipStream_t stream, char* arena) const;
 
     kernel_manager_t*        km_;

@@ -143,15 +143,15 @@ double probe_mfma_f16(void const* operands, void* scratch, int blocks, int iters
     if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) return -1.0;
     hipLaunchKernelGGL(mfma_probe_kernel, dim3(blocks), dim3(256), 0, stream,
                        static_cast<chunk_t const*>(operands), static_cast<float*>(scratch), 64);
-    hipEventRecord(e0, stream);
+    (void)hipEventRecord(e0, stream);
     hipLaunchKernelGGL(mfma_probe_kernel, dim3(blocks), dim3(256), 0, stream,
                        static_cast<chunk_t const*>(operands), static_cast<float*>(scratch), iters);
-    hipEventRecord(e1, stream);
+    (void)hipEventRecord(e1, stream);
     float ms = 0;
     bool  ok = hipEventSynchronize(e1) == hipSuccess &&
               hipEventElapsedTime(&ms, e0, e1) == hipSuccess && ms > 0;
-    hipEventDestroy(e0);
-    hipEventDestroy(e1);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
     if (!ok) return -1.0;
     double flop = double(blocks) * 4.0 * double(iters) * 8.0 * 32768.0;
     return flop / (double(ms) * 1e-3) / 1e12;

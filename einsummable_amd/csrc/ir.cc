@@ -444,6 +444,44 @@ scalarop_t scalarop_t::replace_variables(
     return ret;
 }
 
+namespace
+{
+void compose_in(node_t& n, int k, int n_inner, node_t const& inner)
+{
+    if (n.kind == op_kind::hole) {
+        if (n.arg == k) {
+            node_t c;
+            c.kind = op_kind::convert;
+            c.dtype = inner.dtype;
+            c.children.push_back(inner);
+            n = std::move(c);
+        } else {
+            n.arg = n_inner + (n.arg < k ? n.arg : n.arg - 1);
+        }
+        return;
+    }
+    for (node_t& c : n.children) compose_in(c, k, n_inner, inner);
+}
+}  // namespace
+
+scalarop_t scalarop_t::compose(scalarop_t const& outer, int k, scalarop_t const& inner)
+{
+    if (k < 0 || k >= outer.num_inputs() || !outer.hole_dtypes[size_t(k)]) {
+        throw ir_error("compose: the outer expression has no hole " + std::to_string(k));
+    }
+    if (outer.hole_dtypes[size_t(k)].value() != inner.out_dtype()) {
+        throw ir_error("compose: hole and inner expression differ in dtype");
+    }
+    scalarop_t ret;
+    ret.root = outer.root;
+    compose_in(ret.root, k, inner.num_inputs(), inner.root);
+    ret.hole_dtypes = inner.hole_dtypes;
+    for (int i = 0; i != outer.num_inputs(); ++i) {
+        if (i != k) ret.hole_dtypes.push_back(outer.hole_dtypes[size_t(i)]);
+    }
+    return ret;
+}
+
 scalar_bits_t parse_scalar(std::string const& text)
 {
     scalarop_t op = scalarop_t::parse("constant{" + text + "}");

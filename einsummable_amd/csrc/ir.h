@@ -83,6 +83,13 @@ struct scalarop_t {
     // einsummable.cc:221-233).  Variables not named stay.
     scalarop_t replace_variables(std::vector<std::pair<std::string, double>> const& values) const;
 
+    // `outer` with hole k replaced by the whole of `inner`, whose value passes through a
+    // conversion to inner's own output dtype first (what a store by one kernel and a load by
+    // the next do to it: a rounding for f16, nothing for the other dtypes, where the node
+    // still keeps the two expressions apart).  inner's holes keep their numbers; outer's other
+    // holes follow them in their old order.  Throws ir_error when the dtypes do not meet.
+    static scalarop_t compose(scalarop_t const& outer, int k, scalarop_t const& inner);
+
     std::string str() const;
     dtype_t     out_dtype() const { return root.dtype; }
     int         num_inputs() const { return int(hole_dtypes.size()); }

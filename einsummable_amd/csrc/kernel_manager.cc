@@ -340,16 +340,11 @@ void kernel_manager_t::touch_batch(std::vector<touch_t> const& touches_, hipStre
     int const esz = int(dtype_size(dt));
     int const vmax = 16 / esz;
 
-    // the output is walked in 16-byte vectors whenever its rows allow it; the windows
-    // themselves only need to be vector aligned for the inputs to be read as vectors too
+    // the output is walked in 16-byte vectors whenever its rows allow it
     bool out_wide = reinterpret_cast<uintptr_t>(out) % 16 == 0;
-    bool aligned = true;
     for (size_t i = 0; i != n; ++i) {
         touchdim_t const& last = ts[i].selection[r - 1];
         out_wide = out_wide && last.d_out % vmax == 0;
-        aligned = aligned && last.size % vmax == 0 && last.offset_inn % vmax == 0 &&
-                  last.offset_out % vmax == 0 && reinterpret_cast<uintptr_t>(inns[i]) % 16 == 0;
-        if (r > 1) aligned = aligned && last.d_inn % vmax == 0;
         for (auto const& d : ts[i].selection) {
             if (d.d_out >= (1ull << 32)) {
                 throw km_error(km_status::invalid, "touch_batch: extent beyond 2^32");

@@ -35,6 +35,8 @@ EXPORTS = [
     "es_km_graph_add_fill_lowertri",
     "es_km_graph_add_copy",
     "es_km_graph_add_memory_dependencies",
+    "es_km_graph_optimize",
+    "es_km_graph_node_describe",
     "es_km_graph_finalize",
     "es_km_graph_run",
     "es_km_graph_node_info",
@@ -193,6 +195,9 @@ def load_library():
                                                   U64, V, I]
     lib.es_km_graph_add_copy.argtypes = [V, U64, U64, U64, V, I]
     lib.es_km_graph_add_memory_dependencies.argtypes = [V]
+    lib.es_km_graph_optimize.argtypes = [V, ctypes.POINTER(ctypes.c_int)]
+    lib.es_km_graph_node_describe.restype = ctypes.c_int64
+    lib.es_km_graph_node_describe.argtypes = [V, I, ctypes.c_char_p, U64]
     lib.es_km_graph_finalize.argtypes = [V, I]
     lib.es_km_graph_run.argtypes = [V, V, V]
     lib.es_km_graph_node_info.argtypes = [V, I, V, V, V, I, V]
@@ -596,6 +601,13 @@ class ApplyGraph:
     def add_memory_dependencies(self):
         self._check(self._lib.es_km_graph_add_memory_dependencies(self._g))
 
+    def optimize(self):
+        """Absorbs whole-range copies and single-reader elementwise producers into their
+        neighbours (es_km_graph_optimize); returns how many nodes were absorbed."""
+        n = ctypes.c_int(0)
+        self._check(self._lib.es_km_graph_optimize(self._g, ctypes.byref(n)))
+        return n.value
+
     def finalize(self, n_streams=1):
         self._check(self._lib.es_km_graph_finalize(self._g, int(n_streams)))
 
@@ -609,6 +621,14 @@ class ApplyGraph:
         self._check(self._lib.es_km_graph_node_info(self._g, node, ctypes.byref(pos),
                                                     ctypes.byref(st), deps, 4096, ctypes.byref(n)))
         return pos.value, st.value, list(deps[:min(n.value, 4096)])
+
+    def describe(self, node):
+        """"<kind> <offset>:<size> ... | <einsummable key>" of a node."""
+        buf = ctypes.create_string_buffer(1 << 14)
+        n = self._lib.es_km_graph_node_describe(self._g, int(node), buf, len(buf))
+        if n < 0:
+            raise KmError(int(n), "no such node")
+        return buf.value.decode()
 
     def cross_stream_waits(self):
         return self._check(self._lib.es_km_graph_cross_stream_waits(self._g))

@@ -273,7 +273,11 @@ class ArenaRunner:
 
     ALIGN = 256
 
-    def __init__(self, km, graph, n_streams=4):
+    def __init__(self, km, graph, n_streams=4, optimize=False):
+        """`optimize`: every range that is neither an input nor the layer's output gets the
+        del node a memgraph holds for it (a dummy behind its last reader), and the exec graph
+        may then absorb whole-range copies and single-reader elementwise nodes into their
+        neighbours; what stays in memory keeps every bit."""
         import struct
 
         import torch
@@ -301,7 +305,18 @@ class ArenaRunner:
                 i = ag.add_lowertri_fill(n["dtype"], lo, up, n["nrow"], n["ncol"], n["start"],
                                          self.ranges[n["out"]])
             self.ids.append(i)
+        self.absorbed = 0
+        if optimize:
+            last_reader = {}
+            for i, n in zip(self.ids, graph.nodes):
+                for b in n.get("inns", [n["inn"]] if "inn" in n else []):
+                    last_reader[b] = i
+            for name, i in last_reader.items():
+                if name not in graph.inputs and name != graph.output:
+                    ag.add_dummy(self.ranges[name], [i])
         ag.add_memory_dependencies()
+        if optimize:
+            self.absorbed = ag.optimize()
         ag.finalize(n_streams)
         self.graph = ag
         self.n_streams = n_streams

@@ -216,6 +216,20 @@ int es_km_graph_add_copy(es_km_graph_t* g, uint64_t dst_offset, uint64_t src_off
  * write, write after read), for callers that hold no explicit edge list. */
 int es_km_graph_add_memory_dependencies(es_km_graph_t* g);
 
+/* Optional, before finalize: removes round trips through memory that change no stored bit.
+ * A touch that copies a whole range which one einsummable wrote and nobody else reads (the
+ * formation copy behind every contraction and reduction, src/einsummable/taskgraph.cc:
+ * 3047-3061) is dropped and the einsummable writes the copy's output; an elementwise
+ * einsummable, or a reduction of one input, whose input was written by an elementwise
+ * einsummable and is read by nobody else becomes one einsummable with both joins, the inner
+ * value rounded as the store between them rounded it.  Both need the range's del node
+ * (memgraph.h: del_t) in the graph, as a dummy that covers the range and depends on the
+ * reader: without it the range counts as a result and stays.  Node ids stay valid: the
+ * absorbed node becomes a dummy.  *n_absorbed (may be null) receives how many were absorbed.
+ * No counterpart in the reference, whose engine launches the nodes as the memgraph lists
+ * them. */
+int es_km_graph_optimize(es_km_graph_t* g, int* n_absorbed);
+
 /* Builds every einsummable (an unsupported one is an error here), places the nodes on
  * n_streams (1..16) streams.  The graph is immutable afterwards. */
 int es_km_graph_finalize(es_km_graph_t* g, int n_streams);
@@ -229,6 +243,11 @@ int es_km_graph_run(es_km_graph_t* g, void* stream, void* arena);
 int es_km_graph_node_info(es_km_graph_t* g, int id, int* position, int* stream, int* deps, int cap,
                           int* n_deps);
 int es_km_graph_cross_stream_waits(es_km_graph_t* g);
+/* Any time: a node as text, "<kind> <offset>:<size> ..." (the output range first) and, for an
+ * einsummable, " | [join shape]castable modes->out rank | join" (the join in the text form of
+ * scalarop's operator<<, src/einsummable/scalarop.cc:2881-3011).  Writes at most cap-1
+ * characters and a terminator; returns the full length, negative for a bad id. */
+int64_t es_km_graph_node_describe(es_km_graph_t* g, int id, char* out, uint64_t cap);
 /* After finalize: launches one run makes.  Touches of one group that follow each other in
  * insertion order and write the same output range count once: they run as one
  * es_km_touch_batch launch, with the bytes of one launch per touch

@@ -301,6 +301,52 @@ def test_llama_layer_through_the_exec_graph_equals_node_by_node_launches(km, n_s
         assert len({par.graph.node_info(i)[1] for i in par.ids}) > 1
 
 
+def surviving_buffers(runner):
+    """Names of the ranges some node still writes after the graph's optimisation pass."""
+    by_offset = {off: name for name, (off, _) in runner.ranges.items()}
+    names = set()
+    for i in runner.ids:
+        text = runner.graph.describe(i)
+        if not text.startswith("dummy"):
+            names.add(by_offset[int(text.split()[1].split(":")[0])])
+    return names
+
+
+@pytest.mark.parametrize("shape,n_streams", [
+    (dict(dim=256, n_heads=4, ffn=688, seq=128), 1),
+    (dict(dim=256, n_heads=4, ffn=688, seq=128), 4),
+    (dict(dim=192, n_heads=2, ffn=520, seq=72), 2),       # extents off the vector grid
+    (dict(), 4),                                          # LLaMA-7B: 4096, 32 heads, 11008, 2048
+])
+def test_optimized_layer_keeps_every_stored_bit(km, shape, n_streams):
+    """Formation copies absorbed into their producers and single-reader elementwise nodes
+    merged into their readers: fewer launches, and every range that is still written holds
+    exactly the bytes of the node-by-node run."""
+    import torch
+
+    g = LayerGraph(**shape)
+    vals = make_inputs(g, 11)
+    plain = ArenaRunner(km, g, n_streams)
+    fused = ArenaRunner(km, g, n_streams, optimize=True)
+    # 13 formation copies, and twelve links of elementwise chains: mean_eps -> rsqrt, x_rstd -> to_f16 ->
+    # weight (twice each), scores+mask -> to_f32, sub -> exp, div -> to_f16, silu -> gate,
+    # square -> sum of squares (twice)
+    assert fused.absorbed == 13 + 12, fused.absorbed
+    assert fused.graph.launches() == plain.graph.launches() - fused.absorbed
+    for k, v in vals.items():
+        plain.set_input(k, v)
+        fused.set_input(k, v)
+    plain.run()
+    fused.run()
+    torch.cuda.synchronize()
+    kept = surviving_buffers(fused)
+    assert g.output in kept and "sm.to_f16" in kept and "sm.exp" in kept
+    assert "scores" not in kept and "sm.sub" not in kept and "silu" not in kept
+    for name in sorted(kept):
+        a, b = plain.view(name), fused.view(name)
+        assert torch.equal(a, b), name
+
+
 @pytest.mark.parametrize("n_streams", [
     1,
     pytest.param(4, marks=pytest.mark.skip(

@@ -187,6 +187,107 @@ def test_exec_graph_memory_dependencies_and_stream_placement():
     assert g.cross_stream_waits() >= 2
 
 
+def test_exec_graph_optimize_absorbs_copies_and_single_reader_elementwise():
+    import einsummable_amd as ea
+
+    E = ea.Einsummable
+    g = ea.ApplyGraph(None)
+    m = lambda slot, nbytes=4096: (slot * 8192, nbytes)
+    mm = E.from_str("ij,kj->ik", dict(i=32, j=16, k=32), "*[hole|f32@0,hole|f32@1]", "+")
+    copy = ea.Touch([(1024, 1024, 0, 0, 1024)], None, ea.F32)
+    bsub = E([32, 32], [[0, 1], [0]], 2, "+[hole|f32@0,*[constant{f32|-1},hole|f32@1]]")
+    exp = E([1024], [[0]], 1, "exp[hole|f32@0]")
+    half = E([1024], [[0]], 1, "to_f16[hole|f32@0]")
+    rsum = E([32, 32], [[0, 1]], 1, "hole|f16@0", "+")
+    a = g.add_einsummable(mm, [m(2), m(0, 2048), m(1, 2048)])
+    b = g.add_touch(copy, -1, [m(3), m(2)])                  # formation of the product
+    da = g.add_dummy(m(2), [b])                              # del of the product's first home
+    c = g.add_einsummable(bsub, [m(4), m(3), m(9, 128)])
+    d = g.add_einsummable(exp, [m(5), m(4)])
+    dc = g.add_dummy(m(4), [d])
+    e = g.add_einsummable(half, [m(6, 2048), m(5)])
+    dd = g.add_dummy(m(5), [e])
+    f = g.add_einsummable(rsum, [m(7, 64), m(6, 2048)])      # a reduction of one input
+    de = g.add_dummy(m(6, 2048), [f])
+    keep = g.add_einsummable(exp, [m(8), m(3)])              # a second reader of b's output
+    g.add_memory_dependencies()
+    assert g.optimize() == 4
+    # the product writes the copy's output, at the copy's place
+    assert g.describe(a).startswith("dummy")
+    assert g.describe(b) == "einsummable 24576:4096 0:2048 8192:2048 | " + \
+        "[32,32,16]+ 0.2.,1.2.->2 | *[hole|f32@0,hole|f32@1]"
+    # b's output has two readers (c and keep): it stays, and so does keep
+    assert g.describe(keep).startswith("einsummable 65536:4096 24576:4096 |")
+    # c, d, e end in f: one reduction whose join holds all four, each stored value rounded
+    # as its store rounded it (to_f32 of an f32 marks a value that passed through memory)
+    for k in (c, d, e):
+        assert g.describe(k).startswith("dummy"), k
+    assert g.describe(f) == "einsummable 57344:64 24576:4096 73728:128 | [32,32]+ 0.1.,0.->1 | " + \
+        "to_f16[to_f16[to_f32[exp[to_f32[+[hole|f32@0,*[constant{f32|-1},hole|f32@1]]]]]]]"
+    g.finalize(2)
+    deps = g.node_info(f)[2]
+    assert b in deps                                         # inherited from c
+    assert g.launches() == 3                                 # b, f, keep
+
+
+def test_exec_graph_optimize_leaves_what_it_cannot_prove():
+    import einsummable_amd as ea
+
+    E = ea.Einsummable
+    exp = E([1024], [[0]], 1, "exp[hole|f32@0]")
+    sq = E([1024], [[0]], 1, "power{2}[hole|f32@0]")
+    m = lambda slot: (slot * 4096, 4096)
+
+    # no del node behind the reader: the range may be a result
+    g = ea.ApplyGraph(None)
+    a = g.add_einsummable(exp, [m(1), m(0)])
+    b = g.add_einsummable(sq, [m(2), m(1)])
+    g.add_memory_dependencies()
+    assert g.optimize() == 0
+
+    # a node between the two overwrites what the first one read
+    g = ea.ApplyGraph(None)
+    a = g.add_einsummable(exp, [m(1), m(0)])
+    w = g.add_einsummable(sq, [m(0), m(3)])
+    b = g.add_einsummable(sq, [m(2), m(1)])
+    g.add_dummy(m(1), [b])
+    g.add_memory_dependencies()
+    assert g.optimize() == 0
+
+    # the range is read again before it is deleted
+    g = ea.ApplyGraph(None)
+    a = g.add_einsummable(exp, [m(1), m(0)])
+    b = g.add_einsummable(sq, [m(2), m(1)])
+    c = g.add_einsummable(sq, [m(3), m(1)])
+    g.add_dummy(m(1), [b, c])
+    g.add_memory_dependencies()
+    assert g.optimize() == 0
+
+    # a permuting producer, a transposed reader, a contraction as reader: left alone
+    g = ea.ApplyGraph(None)
+    tr = E([32, 32], [[1, 0]], 2, "hole|f32@0")
+    mm = E.from_str("ij,jk->ik", dict(i=32, j=32, k=32), "*[hole|f32@0,hole|f32@1]", "+")
+    a = g.add_einsummable(tr, [m(1), m(0)])
+    b = g.add_einsummable(sq, [m(2), m(1)])
+    g.add_dummy(m(1), [b])
+    c = g.add_einsummable(tr, [m(3), m(2)])
+    g.add_dummy(m(2), [c])
+    d = g.add_einsummable(mm, [m(4), m(3), m(5)])
+    g.add_dummy(m(3), [d])
+    g.add_memory_dependencies()
+    assert g.optimize() == 0
+
+    # a later writer of the producer's input waits for the node that reads it now
+    g = ea.ApplyGraph(None)
+    a = g.add_einsummable(exp, [m(1), m(0)])
+    b = g.add_einsummable(sq, [m(2), m(1)])
+    d = g.add_dummy(m(1), [b])
+    w = g.add_einsummable(sq, [m(0), m(3)], deps=[a])
+    assert g.optimize() == 1
+    g.finalize(1)
+    assert b in g.node_info(w)[2]
+
+
 def test_exec_graph_single_stream_needs_no_events_and_groups_chain():
     import einsummable_amd as ea
 
