@@ -25,6 +25,7 @@ SOURCES = [
     "static_workspace.hip",
     "transpose.hip",
     "contraction.hip",
+    "complex_contraction.hip",
     "gemm_f16.hip",
     "gemm_f32.hip",
     "gemm_f64.hip",

@@ -143,6 +143,7 @@ std::optional<uint64_t> kernel_manager_t::build(einsummable_t const& e_)
     if (it != plans_.end()) return it->second->workspace_bytes;
 
     std::shared_ptr<plan_t> p = plan_contraction(e, device_);
+    if (!p) p = plan_complex_contraction(e, device_);
     if (!p) p = plan_transpose(e, device_);
     if (!p) p = plan_staged_elementwise(e, device_);
     if (!p) p = plan_codegen(e, device_);

@@ -93,6 +93,7 @@ private:
 // Planners (one translation unit each).  Each returns nullptr when the einsummable is not
 // of its kind; `e` has already been through merge_adjacent_dims.
 std::shared_ptr<plan_t> plan_contraction(einsummable_t const& e, int device);
+std::shared_ptr<plan_t> plan_complex_contraction(einsummable_t const& e, int device);
 std::shared_ptr<plan_t> plan_transpose(einsummable_t const& e, int device);
 std::shared_ptr<plan_t> plan_codegen(einsummable_t const& e, int device);
 

@@ -35,6 +35,10 @@ struct transpose_args_t {
     uint64_t    n_blocks;
     uint32_t    nb;                 // number of batch modes
     uint32_t    plain_stores;       // results go through the L2 instead of streaming past it
+    // 0: tiles in launch order, input-inner mode first (consecutive workgroups land on
+    // different XCDs); 1: every XCD takes one contiguous run of that order, so that the
+    // neighbours along a row share an L2; 2: the same with the output-inner mode first
+    uint32_t    order;
     uint32_t    bsize[MAXB];        // innermost batch mode first
     int64_t     bsi[MAXB], bso[MAXB];
 };
@@ -44,13 +48,25 @@ template <int EDGE, int EDGE_O = EDGE>
 __device__ __forceinline__ bool locate(transpose_args_t const& a, uint32_t& i0, uint32_t& o0,
                                        int64_t& off_i, int64_t& off_o)
 {
-    uint64_t const linear = uint64_t(blockIdx.y) * gridDim.x + blockIdx.x;
+    uint64_t linear = uint64_t(blockIdx.y) * gridDim.x + blockIdx.x;
     if (linear >= a.n_blocks) return false;  // uniform over the workgroup
+    if (a.order) {
+        uint64_t const per = a.n_blocks / 8;
+        if (linear < per * 8) linear = (linear % 8) * per + linear / 8;
+    }
     uint32_t t = uint32_t(linear);
-    uint32_t const ti = t % a.tiles_i;
-    t /= a.tiles_i;
-    uint32_t const to = t % a.tiles_o;
-    t /= a.tiles_o;
+    uint32_t ti, to;
+    if (a.order == 2) {
+        to = t % a.tiles_o;
+        t /= a.tiles_o;
+        ti = t % a.tiles_i;
+        t /= a.tiles_i;
+    } else {
+        ti = t % a.tiles_i;
+        t /= a.tiles_i;
+        to = t % a.tiles_o;
+        t /= a.tiles_o;
+    }
     uint32_t bidx = t;
     off_i = 0;
     off_o = 0;
@@ -192,21 +208,25 @@ __global__ __launch_bounds__(256) void transpose_kernel(transpose_args_t a)
 // Tile of the 16-byte kernel, measured on 4096..16384-square matrices with cold and with warm
 // caches.  4-byte elements: 512-byte segments on the way in and 256-byte segments on the way
 // out beat the square tile by 4..12 % once there are enough tiles to fill the device.
-// 2-byte elements: the same holds only for matrices well beyond the memory-side cache (2..6 %
-// at 16384 x 16384; at 8192 x 8192 the square tile is 6 % faster).
+// 2-byte elements: the long tile pays once each XCD works on one contiguous run of tiles
+// (8192 x 8192: 51.4 us square in launch order, 48.2 us long in runs; 16384 x 16384: 228 us
+// against 213 us long, in runs, output-inner mode first); 4-byte elements gain nothing from
+// the runs (91 us either way).
 inline void vec_shape(int elem_size, uint32_t n_i, uint32_t n_o, uint64_t batch, uint32_t& edge_i,
-                      uint32_t& edge_o)
+                      uint32_t& edge_o, uint32_t& order)
 {
     uint64_t const bytes = 2ull * n_i * n_o * batch * uint64_t(elem_size);
     const char*    env = std::getenv("ES_KM_TRANSPOSE_TILE");  // tuning and tests
     bool const     force_square = env && std::string(env) == "square";
     bool const     force_long = env && std::string(env) == "long";
     edge_i = edge_o = 64;
+    order = 0;
     if (elem_size == 2) {
         edge_i = edge_o = 128;
-        if (!force_square && (force_long || (bytes >= (1ull << 30) && n_i >= 256))) {
+        if (!force_square && (force_long || (bytes >= (128ull << 20) && n_i >= 256))) {
             edge_i = 256;
             edge_o = 64;
+            order = bytes >= (1ull << 30) ? 2 : 1;
         }
     } else if (elem_size == 4) {
         uint64_t const tiles = uint64_t((n_i + 127) / 128) * ((n_o + 63) / 64) * batch;
@@ -219,6 +239,7 @@ struct transpose_plan_t : plan_t {
     int              elem_size;
     uint64_t         batch;
     bool             vec_ok;  // extents, strides and batch offsets keep rows 16-byte aligned
+    bool             order_forced = false;
 
     void run(hipStream_t stream, void* out, void const* const* inns, void*, uint64_t) const override
     {
@@ -229,7 +250,11 @@ struct transpose_plan_t : plan_t {
                              reinterpret_cast<uintptr_t>(a.out) % 16 == 0;
         bool const vec = vec_ok && aligned;
         uint32_t edge_i = 64, edge_o = 64;
-        if (vec) vec_shape(elem_size, a.n_i, a.n_o, batch, edge_i, edge_o);
+        if (vec) {
+            uint32_t order = 0;
+            vec_shape(elem_size, a.n_i, a.n_o, batch, edge_i, edge_o, order);
+            if (!order_forced) a.order = order;
+        }
         a.tiles_i = (a.n_i + edge_i - 1) / edge_i;
         a.tiles_o = (a.n_o + edge_o - 1) / edge_o;
         uint64_t const blocks = uint64_t(a.tiles_i) * a.tiles_o * batch;
@@ -346,11 +371,17 @@ std::shared_ptr<plan_t> plan_transpose(einsummable_t const& e, int)
     if (const char* env = std::getenv("ES_KM_TRANSPOSE_STORES")) {  // tuning and tests
         a.plain_stores = std::string(env) == "cached";
     }
+    a.order = 0;
     p->workspace_bytes = 0;
     uint32_t edge_i = 64, edge_o = 64;
-    if (p->vec_ok) vec_shape(p->elem_size, a.n_i, a.n_o, batch, edge_i, edge_o);
+    if (p->vec_ok) vec_shape(p->elem_size, a.n_i, a.n_o, batch, edge_i, edge_o, a.order);
+    if (const char* env = std::getenv("ES_KM_TRANSPOSE_ORDER")) {  // tuning and tests
+        a.order = uint32_t(std::atoi(env)) % 3;
+        p->order_forced = true;
+    }
     p->description = "transpose_lds tile=" + std::to_string(edge_i) + "x" + std::to_string(edge_o) +
                      (p->vec_ok ? " vec16" : "") + (a.plain_stores ? " cached_stores" : "") +
+                     (a.order == 1 ? " xcd_runs" : a.order == 2 ? " xcd_runs_out_first" : "") +
                      " batch=" + std::to_string(batch);
     return p;
 }

@@ -12,7 +12,7 @@ from helpers import NP, assert_close, normal, oracle_einsummable, rng, run_einsu
 pytestmark = pytest.mark.gpu
 
 E = ea.Einsummable
-DT = {"f16": ea.F16, "f32": ea.F32, "f64": ea.F64}
+DT = {"f16": ea.F16, "f32": ea.F32, "f64": ea.F64, "c64": ea.C64}
 
 
 def contraction(spec, sizes, dt):
@@ -25,7 +25,11 @@ def check(km, spec, sizes, dt, seed=0, expect_mfma=True):
     r = rng(seed)
     xs = [uniform(r, int(np.prod(e.inn_shape(k))), NP[DT[dt]]) for k in range(2)]
     got = run_einsummable(km, e, xs)
-    if expect_mfma:
+    if expect_mfma and dt == "c64":
+        # the complex product runs as an fp32 product of twice the depth on the matrix cores
+        d = km.describe(e)
+        assert d.startswith("contraction_c64_as_f32") and "contraction_mfma_f32" in d, d
+    elif expect_mfma:
         assert km.describe(e).startswith("contraction_mfma_" + dt), km.describe(e)
     want = oracle_einsummable(e, xs, oracle.WIDE)
     assert_close(got, want, DT[dt], what="%s %s %s [%s]" % (spec, sizes, dt, km.describe(e)))
@@ -98,6 +102,71 @@ def test_multi_mode_groups(km, dt):
     check(km, "ipq,qpk->ik", dict(i=24, p=6, q=16, k=40), dt, seed=15)
     check(km, "xiyj,jk->xyik", dict(x=3, y=5, i=8, j=32, k=24), dt, seed=16)
     check(km, "ij,xjyk->iyxk", dict(x=3, y=5, i=8, j=32, k=24), dt, seed=17)
+
+
+@pytest.mark.parametrize("spec", MATMULS)
+def test_complex_matmul_spellings_run_on_the_matrix_cores(km, spec):
+    # every spelling: the left operand in place (summed mode innermost) or split into planes,
+    # the right one expanded along k or along n; the known-answer shape of tests/reference.h
+    check(km, spec, dict(i=64, j=96, k=80), "c64", seed=31)
+    check(km, spec, dict(i=37, j=51, k=29), "c64", seed=32)
+    check(km, spec, dict(i=3, j=4, k=5), "c64", seed=33)
+    check(km, spec, dict(i=130, j=264, k=136), "c64", seed=34)
+
+
+def test_complex_matmul_closed_form(km):
+    # (1 + i) times ones times (2 - i) ones: every entry is j * (1 + i)(2 - i) = j * (3 + i)
+    e = contraction("ij,jk->ik", dict(i=40, j=48, k=56), "c64")
+    lhs = np.full(40 * 48, 1 + 1j, np.complex64)
+    rhs = np.full(48 * 56, 2 - 1j, np.complex64)
+    got = run_einsummable(km, e, [lhs, rhs])
+    assert np.array_equal(got, np.full(40 * 56, 48 * (3 + 1j), np.complex64))
+
+
+COMPLEX_FORMS = [
+    ("bij,bjk->bik", dict(b=3, i=40, j=48, k=56), True),
+    ("bij,jk->bik", dict(b=3, i=40, j=48, k=56), True),
+    ("ibj,bjk->bik", dict(b=3, i=40, j=48, k=56), True),
+    ("bij,bkj->bki", dict(b=2, i=40, j=32, k=24), True),       # the left operand is expanded
+    ("aibj,akbj->abik", dict(a=2, b=3, i=24, j=32, k=40), True),
+    ("ipq,qpk->ik", dict(i=24, p=6, q=16, k=40), True),         # two summed modes, orders differ
+    ("xiyj,jk->xyik", dict(x=3, y=5, i=8, j=32, k=24), True),
+    ("ij,xjyk->iyxk", dict(x=3, y=5, i=8, j=32, k=24), True),
+    ("acbe,adbe->abcd", dict(a=1, b=4, c=72, d=88, e=64), True),
+    ("abce,aebd->abcd", dict(a=1, b=4, c=72, e=88, d=64), True),
+    ("bij,bjk->ikb", dict(b=4, i=24, j=16, k=40), False),       # batch innermost: generated kernel
+]
+
+
+@pytest.mark.parametrize("spec,sizes,mfma", COMPLEX_FORMS)
+def test_complex_contraction_forms(km, spec, sizes, mfma):
+    check(km, spec, sizes, "c64", seed=35, expect_mfma=mfma)
+    if not mfma:
+        assert not km.describe(contraction(spec, sizes, "c64")).startswith("contraction_c64")
+
+
+def test_complex_contraction_with_operands_off_the_vector_grid(km):
+    """Operands and output 8 bytes off a 16-byte boundary (a complex element's own alignment):
+    the expansion reads them as they lie, the fp32 product falls to its element paths."""
+    import torch
+    from helpers import stream_handle
+
+    e = contraction("ij,kj->ik", dict(i=72, j=40, k=56), "c64")
+    r = rng(36)
+    xs = [uniform(r, 72 * 40, np.complex64), uniform(r, 56 * 40, np.complex64)]
+    ws = km.build(e)
+    bufs = []
+    for x in xs:
+        t = torch.zeros(x.size + 1, dtype=torch.complex64, device="cuda")
+        t[1:] = torch.from_numpy(x).cuda()
+        bufs.append(t)
+    out = torch.zeros(72 * 56 + 1, dtype=torch.complex64, device="cuda")
+    w = torch.empty(max(ws, 1), dtype=torch.uint8, device="cuda")
+    km(e, stream_handle(), out.data_ptr() + 8, [b.data_ptr() + 8 for b in bufs], (w.data_ptr(), ws))
+    torch.cuda.synchronize()
+    want = oracle_einsummable(e, xs, oracle.WIDE)
+    assert_close(out[1:].cpu().numpy(), want, ea.C64, what="c64 off the vector grid")
+    assert out[0].item() == 0
 
 
 def test_one_sided_aggregation_is_not_a_gemm(km):

@@ -117,20 +117,25 @@ def test_transpose_beyond_a_gibibyte_takes_the_long_tile(km):
     assert torch.equal(y, x.t())
 
 
-@pytest.mark.parametrize("stores", ["stream", "cached"])
+@pytest.mark.parametrize("stores,order", [("stream", 0), ("cached", 1), ("cached", 2), ("stream", 2)])
 @pytest.mark.parametrize("dt,npdt,tile", [("f16", np.float16, "256x64"), ("f32", np.float32, "128x64")])
-def test_long_tiles_forced_on_small_ragged_transposes(monkeypatch, dt, npdt, tile, stores):
+def test_long_tiles_forced_on_small_ragged_transposes(monkeypatch, dt, npdt, tile, stores, order):
     # the switches are read when a plan is made: a manager of its own, so that no plan made
-    # under them stays in the session's manager
+    # under them stays in the session's manager.  `order`: the tile a workgroup takes (launch
+    # order; one run of tiles per XCD; the same with the output-inner mode first), on tile
+    # counts that do not divide by the eight XCDs
     monkeypatch.setenv("ES_KM_TRANSPOSE_TILE", "long")
     monkeypatch.setenv("ES_KM_TRANSPOSE_STORES", stores)
+    monkeypatch.setenv("ES_KM_TRANSPOSE_ORDER", str(order))
     km = ea.KernelManager(0)
     r = rng(55)
-    for shape, perm in [((264, 72), (1, 0)), ((2, 520, 136), (0, 2, 1)), ((8, 3, 776), (2, 1, 0))]:
+    for shape, perm in [((264, 72), (1, 0)), ((2, 520, 136), (0, 2, 1)), ((8, 3, 776), (2, 1, 0)),
+                        ((1032, 1160), (1, 0))]:
         x = normal(r, int(np.prod(shape)), npdt).reshape(shape)
         e = permute_einsummable(shape, perm, dt)
         got = run_einsummable(km, e, [x])
         d = km.describe(e)
         assert ("tile=%s vec16" % tile) in d and ("cached_stores" in d) == (stores == "cached"), d
+        assert ("xcd_runs" in d) == (order != 0) and ("out_first" in d) == (order == 2), d
         want = np.ascontiguousarray(np.transpose(x, perm)).reshape(-1)
         assert_bits_equal(got, want, "permute %s %s" % (shape, perm))
