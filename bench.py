@@ -29,7 +29,8 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E
-PEAK_TFLOPS = {"f16": 2500.0, "f32": 157.3, "f64": 78.6}
+# c64 products run as fp32 products of twice the depth: real flops against the fp32 peak
+PEAK_TFLOPS = {"f16": 2500.0, "f32": 157.3, "f64": 78.6, "c64": 157.3}
 
 # HBM bytes per launch of the dominant kernel (C2 node (i)) from two rocprofv3 --pmc runs:
 # FETCH_SIZE 131084.9 KiB x 1.9998 + WRITE_SIZE 131076.0 KiB x 1.0000, the factors being what
@@ -47,7 +48,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="all",
                     choices=["c2", "c1", "c3", "c4", "c5", "llama", "copy", "mfma_peak", "build",
-                             "all"])
+                             "colred", "all"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     return ap.parse_args()
 
@@ -358,7 +359,8 @@ def cpu_baselines_other_configs():
 def run_contraction(km, name, e, shapes, dtype, flops, steps, warmup, yardstick=None):
     import torch
 
-    tdt = {"f16": torch.float16, "f32": torch.float32, "f64": torch.float64}[dtype]
+    tdt = {"f16": torch.float16, "f32": torch.float32, "f64": torch.float64,
+           "c64": torch.complex64}[dtype]
     g = torch.Generator(device="cuda").manual_seed(1)
     ins = [torch.randn(*s, device="cuda", dtype=tdt, generator=g) for s in shapes[:-1]]
     out = torch.empty(*shapes[-1], device="cuda", dtype=tdt)
@@ -1004,6 +1006,22 @@ def main():
     torch.cuda.empty_cache()
     if args.workload in ("c1", "all"):
         others["c1"] = run_c1(km, args.steps, args.warmup)
+    if args.workload in ("c1", "all"):
+        # the same matmul in the other two dtypes the reference sends to its BLAS
+        # (cublasDgemm / cublasCgemm, gpu_kernel_manager.cc:1543-1558); no configuration
+        # uses them, they are here so that the paths have a number
+        import einsummable_amd as ea
+        n = 2048
+        rows = []
+        for dt, flop in (("f64", 2 * n ** 3), ("c64", 8 * n ** 3)):
+            for spec, inns in (("ij,jk->ik", [[0, 2], [2, 1]]), ("ij,kj->ik", [[0, 2], [1, 2]])):
+                e = ea.Einsummable([n, n, n], inns, 2, "*[hole|%s@0,hole|%s@1]" % (dt, dt), "+")
+                yard = (lambda a, b: torch.matmul(a, b)) if spec == "ij,jk->ik" else \
+                       (lambda a, b: torch.matmul(a, b.t()))
+                rows.append(run_contraction(km, "%s %s 2048^3" % (spec, dt), e,
+                                            [(n, n), (n, n), (n, n)], dt, flop,
+                                            max(args.steps // 5, 3), max(args.warmup // 5, 1), yard))
+        others["f64_c64_matmuls"] = rows
     if args.workload in ("c3", "all"):
         others["c3"] = run_c3(km, args.steps, args.warmup)
     if args.workload in ("c4", "all"):
@@ -1015,6 +1033,7 @@ def main():
     if args.workload == "all":
         others["mfma_f16_register_ceiling"] = run_mfma_peak(km)
         others["read_only_1GiB"] = run_read_ceiling(km, args.steps, args.warmup)
+    if args.workload in ("colred", "all"):
         others["column_reductions"] = run_col_reductions(km, args.steps, args.warmup)
     if args.workload == "all" and not args.no_cpu_baseline:
         others["cpu_baselines"] = cpu_baselines_other_configs()
