@@ -483,12 +483,16 @@ cg_kernel_t gen_elementwise(einsummable_t const& e, int max_vec)
         footprint += e.inn_nelem(k) * dtype_size(e.inn_dtype(k));
     }
     bool const stream_out = out_bytes >= (64ull << 20) && footprint > (288ull << 20);
-    // Such a node reads non-temporally too.  A line that was read normally is still in the
-    // memory-side cache when its result is stored, the store hits it there, and the dirty
-    // line is written back during the NEXT node: the row max behind a 1 GiB in-place scale
-    // read at 5.1 TB/s, behind the same node with streaming loads at 6.2 (C4: row max 0.206
-    // -> 0.173 ms, row sum 0.205 -> 0.168, P.V 0.275 -> 0.215, chain 1.92 -> 1.77 ms).
-    int const nt_mode = env_int("ES_KM_EW_NT", stream_out ? 1 : 4);
+    // With a result beyond the cache's size such a node reads non-temporally too.  A line
+    // that was read normally is still in the memory-side cache when its result is stored, the
+    // store hits it there, and the dirty line is written back during the NEXT node: the row
+    // max behind a 1 GiB in-place scale read at 5.1 TB/s, behind the same node with
+    // streaming loads at 6.2 (C4: row max 0.206 -> 0.173 ms, row sum 0.205 -> 0.168, P.V
+    // 0.275 -> 0.215, chain 1.92 -> 1.77 ms).
+    // A result that itself fits the cache (C2's 128 MiB product, read by the row max next)
+    // is better off with plain loads: row max 22.7 against 25.0 us.
+    bool const stream_in = stream_out && out_bytes >= (256ull << 20);
+    int const nt_mode = env_int("ES_KM_EW_NT", stream_in ? 1 : (stream_out ? 3 : 4));
     int const NT_LD = (nt_mode == 1 || nt_mode == 2) ? 1 : 0;
     int const NT_ST = (nt_mode == 1 || nt_mode == 3) ? 1 : 0;
     uint64_t const n_vec = n_out / uint64_t(V);
