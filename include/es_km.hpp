@@ -176,6 +176,20 @@ public:
                             workspace ? std::get<1>(workspace.value()) : 0));
     }
 
+    // The same call for places that must not allocate (under HIP graph capture, in a serving
+    // loop): the kernel's scratch comes from the library's static device array instead of a
+    // workspace argument (es_km_execute_static_workspace); needs beyond
+    // ES_KM_STATIC_WORKSPACE_BYTES are refused.
+    void execute_static_workspace(einsummable_t const& e, void* stream, void* out,
+                                  std::vector<void const*> inns) const
+    {
+        flat_t f(e);
+        check(es_km_execute_static_workspace(
+            h_, e.join_shape.data(), int(e.join_shape.size()), f.flat.data(), f.offs.data(),
+            int(e.inns.size()), e.out_rank, e.join.c_str(), castable_char(e.castable), stream, out,
+            inns.data(), int(inns.size())));
+    }
+
     void lowerTri_fill(fill_t::lowertri_t const& l, void* stream, void* out) const
     {
         check(es_km_fill_lowertri(h_, int(l.lower.dtype), l.lower.bits(), l.upper.bits(), l.nrow,
@@ -323,8 +337,44 @@ public:
     uint64_t arena_bytes() const { return es_km_graph_arena_bytes(g_); }
     void add_memory_dependencies() { check(es_km_graph_add_memory_dependencies(g_)); }
     void finalize(int n_streams) { check(es_km_graph_finalize(g_, n_streams)); }
+    // optional, before finalize: absorbs whole-range copies into their producers and
+    // single-reader elementwise nodes into their readers; returns how many nodes went
+    int optimize()
+    {
+        int n = 0;
+        check(es_km_graph_optimize(g_, &n));
+        return n;
+    }
     // the whole graph, ordered after and before `stream`; no host synchronisation
     void run(void* stream, void* arena) const { check(es_km_graph_run(g_, stream, arena)); }
+
+    // One node at a time, for a host event loop that keeps the dependencies itself
+    // (gpu_einsummable_t::launch / gpu_touch_t::launch with a callback,
+    // src/engine/gpu/exec_graph.cc:277-335, 354-404): enqueues node `id` on `stream` and,
+    // behind it, a host function that calls callback(user) when the node is done.
+    void launch(int id, void* stream, void* arena, void* workspace, uint64_t workspace_bytes,
+                es_km_callback_t callback, void* user, int first_in_group = -1) const
+    {
+        check(es_km_graph_launch_node(g_, id, stream, arena, workspace, workspace_bytes,
+                                      first_in_group, callback, user));
+    }
+    uint64_t node_workspace(int id) const
+    {
+        uint64_t ws = 0;
+        check(es_km_graph_node_workspace(g_, id, &ws));
+        return ws;
+    }
+    int node_group(int id) const { return es_km_graph_node_group(g_, id); }
+    // dependencies of a node (own and implied), after finalize
+    std::vector<int> node_deps(int id) const
+    {
+        int pos = 0, st = 0, n = 0;
+        check(es_km_graph_node_info(g_, id, &pos, &st, nullptr, 0, &n));
+        std::vector<int> deps(size_t(n), 0);
+        if (n) check(es_km_graph_node_info(g_, id, &pos, &st, deps.data(), n, &n));
+        return deps;
+    }
+    int n_launches() const { return es_km_graph_launches(g_); }
 
 private:
     static void split(std::vector<mem_t> const& m, std::vector<uint64_t>& o,
@@ -348,6 +398,52 @@ private:
     }
     kernel_manager_t& km_;
     es_km_graph_t*    g_;
+};
+
+// The workspace pool of src/engine/gpu/workspace.cc:48-91 (first block that is large enough,
+// else a new allocation) and the stream pool of src/engine/gpu/stream_pool.cc, for callers of
+// exec_graph_t::launch.
+class workspace_pool_t
+{
+public:
+    explicit workspace_pool_t(int device) : p_(es_km_workspace_pool_create(device))
+    {
+        if (!p_) throw std::runtime_error(std::string("workspace_pool_t: ") + es_km_last_error(nullptr));
+    }
+    ~workspace_pool_t() { es_km_workspace_pool_destroy(p_); }
+    workspace_pool_t(workspace_pool_t const&) = delete;
+    workspace_pool_t& operator=(workspace_pool_t const&) = delete;
+    // a block of at least `bytes` (its real size in *got), or nullptr with bytes == 0
+    void* acquire(uint64_t bytes, uint64_t* got = nullptr)
+    {
+        uint64_t g = 0;
+        void*    b = es_km_workspace_pool_acquire(p_, bytes, &g);
+        if (!b && bytes) throw std::runtime_error(std::string("workspace_pool_t: ") + es_km_last_error(nullptr));
+        if (got) *got = g;
+        return b;
+    }
+    void release(void* block) { es_km_workspace_pool_release(p_, block); }
+    int  blocks() const { return es_km_workspace_pool_blocks(p_); }
+
+private:
+    es_km_workspace_pool_t* p_;
+};
+
+class stream_pool_t
+{
+public:
+    stream_pool_t(int device, int n_streams) : p_(es_km_stream_pool_create(device, n_streams))
+    {
+        if (!p_) throw std::runtime_error(std::string("stream_pool_t: ") + es_km_last_error(nullptr));
+    }
+    ~stream_pool_t() { es_km_stream_pool_destroy(p_); }
+    stream_pool_t(stream_pool_t const&) = delete;
+    stream_pool_t& operator=(stream_pool_t const&) = delete;
+    void* try_acquire() { return es_km_stream_pool_try_acquire(p_); }  // nullptr: all in use
+    void  release(void* stream) { es_km_stream_pool_release(p_, stream); }
+
+private:
+    es_km_stream_pool_t* p_;
 };
 
 }  // namespace eskm

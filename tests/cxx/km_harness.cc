@@ -8,7 +8,10 @@
 
 #include <hip/hip_runtime_api.h>
 
+#include <algorithm>
 #include <cmath>
+#include <condition_variable>
+#include <mutex>
 #include <cstdio>
 #include <random>
 
@@ -265,6 +268,152 @@ int main()
             ok = ok && got[n + i] == r && got[2 * n + i] == r && slot[i] == r;
         }
         expect(ok, "memgraph from wire: apply, evict to host storage, load back");
+    }
+
+    {  // a host event loop over the exec nodes, as exec_state_t drives them
+       // (src/engine/exec_state.cc:197-219): every node is launched by itself once all it
+       // depends on has called back; streams and scratch come from the two pools.  The graph:
+       // relu(x) -> copy (a formation) -> exp -> to_f16, and a column sum that needs scratch.
+        uint64_t const n = 64 * 1024, B = n * 4;
+        std::string const relu = "ite_>=[constant{f32|0},hole|f32@0,constant{f32|0},hole|f32@0]";
+        einsummable_t e_relu{{n}, {{0}}, 1, relu, std::nullopt};
+        einsummable_t e_exp{{n}, {{0}}, 1, "exp[hole|f32@0]", std::nullopt};
+        einsummable_t e_half{{n}, {{0}}, 1, "to_f16[hole|f32@0]", std::nullopt};
+        einsummable_t e_col{{256, 256}, {{1, 0}}, 1, "hole|f32@0", castable_t::add};
+        auto x = random_f32(gen, n, -2, 2);
+        auto build_graph = [&](exec_graph_t& g) {
+            int a = g.insert_einsummable(e_relu, {{1 * B, B}, {0, B}});
+            touch_t copy{{{n, n, 0, 0, n}}, std::nullopt, dtype_t::f32};
+            int b = g.insert_touch(copy, -1, {2 * B, B}, {1 * B, B}, {a});
+            g.insert_dummy({1 * B, B}, {b});                       // del of relu's first home
+            int c = g.insert_einsummable(e_exp, {{3 * B, B}, {2 * B, B}}, {b});
+            int d = g.insert_einsummable(e_half, {{4 * B, B / 2}, {3 * B, B}}, {c});
+            g.insert_dummy({3 * B, B}, {d});                       // del of exp's output
+            return g.insert_einsummable(e_col, {{5 * B, 1024}, {2 * B, B}}, {b});
+        };
+        auto run_loop = [&](exec_graph_t& g, device_buffer_t& arena, int N) {
+            struct done_t {
+                std::mutex              m;
+                std::condition_variable cv;
+                std::vector<int>        finished;
+            } done;
+            struct note_t {
+                done_t* d;
+                int     id;
+            };
+            std::vector<note_t> notes;
+            for (int i = 0; i != N; ++i) notes.push_back({&done, i});
+            std::vector<std::vector<int>> deps;
+            std::vector<int>              waiting(N, 0);
+            for (int i = 0; i != N; ++i) {
+                deps.push_back(g.node_deps(i));
+                waiting[size_t(i)] = int(deps.back().size());
+            }
+            workspace_pool_t ws_pool(0);
+            stream_pool_t    st_pool(0, 2);
+            std::vector<void*> held_ws(N, nullptr), held_st(N, nullptr);
+            std::vector<int>   ready;
+            for (int i = 0; i != N; ++i) {
+                if (waiting[size_t(i)] == 0) ready.push_back(i);
+            }
+            int completed = 0;
+            while (completed != N) {
+                // launch what is ready while a stream is free
+                while (!ready.empty()) {
+                    void* st = st_pool.try_acquire();
+                    if (!st) break;
+                    int const id = ready.back();
+                    ready.pop_back();
+                    uint64_t const need = g.node_workspace(id);
+                    uint64_t       got = 0;
+                    held_ws[size_t(id)] = need ? ws_pool.acquire(need, &got) : nullptr;
+                    held_st[size_t(id)] = st;
+                    g.launch(id, st, arena.ptr, held_ws[size_t(id)], got,
+                             [](void* u) {
+                                 note_t* nt = static_cast<note_t*>(u);
+                                 std::lock_guard<std::mutex> lk(nt->d->m);
+                                 nt->d->finished.push_back(nt->id);
+                                 nt->d->cv.notify_one();
+                             },
+                             &notes[size_t(id)]);
+                }
+                std::vector<int> fin;
+                {
+                    std::unique_lock<std::mutex> lk(done.m);
+                    done.cv.wait(lk, [&] { return !done.finished.empty(); });
+                    fin.swap(done.finished);
+                }
+                for (int id : fin) {
+                    ++completed;
+                    st_pool.release(held_st[size_t(id)]);
+                    if (held_ws[size_t(id)]) ws_pool.release(held_ws[size_t(id)]);
+                    for (int v = 0; v != N; ++v) {
+                        if (std::find(deps[size_t(v)].begin(), deps[size_t(v)].end(), id) != deps[size_t(v)].end() &&
+                            --waiting[size_t(v)] == 0) {
+                            ready.push_back(v);
+                        }
+                    }
+                }
+            }
+            HIP_OK(hipDeviceSynchronize());
+            return ws_pool.blocks();
+        };
+        std::vector<float> host(6 * n, 7.0f);
+        std::copy(x.begin(), x.end(), host.begin());
+        device_buffer_t arena1(6 * B), arena2(6 * B);
+        arena1.upload(host.data());
+        arena2.upload(host.data());
+        exec_graph_t g1(km), g2(km);
+        int const col_id = build_graph(g1);
+        build_graph(g2);
+        expect(g2.optimize() == 2, "optimize: the copy and the exp are absorbed");
+        g1.finalize(2);
+        g2.finalize(2);
+        expect(g1.n_launches() == 5 && g2.n_launches() == 3, "launch counts");
+        int const blocks = run_loop(g1, arena1, col_id + 1);
+        expect(blocks == (g1.node_workspace(col_id) ? 1 : 0), "scratch blocks in the pool");
+        g2.run(stream, arena2.ptr);
+        HIP_OK(hipStreamSynchronize(stream));
+        std::vector<float> a1(6 * n), a2(6 * n);
+        arena1.download(a1.data());
+        arena2.download(a2.data());
+        // against the oracle: relu, exp rounded to f16, column sums
+        std::vector<float> r(n), ex(n), col(256);
+        std::vector<uint16_t> hf(n);
+        oracle_run(e_relu, r.data(), {x.data()});
+        oracle_run(e_exp, ex.data(), {r.data()});
+        oracle_run(e_half, hf.data(), {ex.data()});
+        oracle_run(e_col, col.data(), {r.data()});
+        bool ok = std::memcmp(&a1[2 * n], r.data(), B) == 0;
+        uint16_t const* h1 = reinterpret_cast<uint16_t const*>(&a1[4 * n]);
+        double          worst = 0;
+        for (uint64_t i = 0; i != n; ++i) {
+            double a = es_oracle_f16_to_f32(h1[i]), b = es_oracle_f16_to_f32(hf[i]);
+            worst = std::max(worst, std::fabs(a - b) / std::max(std::fabs(b), 1.0));
+        }
+        for (int i = 0; i != 256; ++i) {
+            worst = std::max(worst, std::fabs(double(a1[5 * n + i]) - col[size_t(i)]) / 256.0);
+        }
+        // (one f16 ulp is 2^-10 of the value: exp differs from the oracle's in the last place)
+        expect(ok && worst <= 2e-3, "event loop: results against the oracle");
+        // the optimised burst keeps every range it still writes
+        expect(std::memcmp(&a1[2 * n], &a2[2 * n], B) == 0 &&
+                   std::memcmp(&a1[4 * n], &a2[4 * n], B / 2) == 0 &&
+                   std::memcmp(&a1[5 * n], &a2[5 * n], 1024) == 0,
+               "optimised graph: same bytes in every range still written");
+
+        // the entry point that allocates nothing, against the one with a workspace argument
+        device_buffer_t dx(B), o1(1024), o2(1024);
+        dx.upload(r.data());
+        auto ws = km.build(e_col);
+        device_buffer_t dws(ws.value().value());
+        km(e_col, stream, o1.ptr, {dx.ptr}, std::make_tuple(dws.ptr, ws.value().value()));
+        km.execute_static_workspace(e_col, stream, o2.ptr, {dx.ptr});
+        HIP_OK(hipStreamSynchronize(stream));
+        std::vector<float> c1(256), c2(256);
+        o1.download(c1.data());
+        o2.download(c2.data());
+        expect(std::memcmp(c1.data(), c2.data(), 1024) == 0, "static workspace: same bits");
     }
 
     HIP_OK(hipStreamDestroy(stream));
