@@ -302,44 +302,90 @@ bool absorbable_producer(einsummable_t const& u)
     return true;
 }
 
+// Two row-major shapes of the same element count cut into the coarsest common pieces:
+// `parts_a[i]` / `parts_b[j]` list the pieces (indices into `pieces`) of mode i / j, outermost
+// first.  False when a mode of one shape straddles a boundary of the other unevenly
+// ([6, 4] against [4, 6]).
+bool refine(std::vector<uint64_t> const& a, std::vector<uint64_t> const& b,
+            std::vector<uint64_t>& pieces, std::vector<std::vector<int>>& parts_a,
+            std::vector<std::vector<int>>& parts_b)
+{
+    std::vector<uint64_t>         rev;  // innermost first
+    std::vector<std::vector<int>> pa(a.size()), pb(b.size());
+    int      i = int(a.size()) - 1, j = int(b.size()) - 1;
+    uint64_t ra = i >= 0 ? a[size_t(i)] : 1, rb = j >= 0 ? b[size_t(j)] : 1;
+    while (i >= 0 && j >= 0) {
+        uint64_t const g = std::min(ra, rb);
+        if (ra % g != 0 || rb % g != 0) return false;
+        int const id = int(rev.size());
+        rev.push_back(g);
+        pa[size_t(i)].push_back(id);
+        pb[size_t(j)].push_back(id);
+        ra /= g;
+        rb /= g;
+        if (ra == 1 && --i >= 0) ra = a[size_t(i)];
+        if (rb == 1 && --j >= 0) rb = b[size_t(j)];
+    }
+    // what is left on either side can only be modes of extent one
+    for (; i >= 0; --i) {
+        if (ra != 1) return false;
+        if (i > 0) ra = a[size_t(i - 1)];
+    }
+    for (; j >= 0; --j) {
+        if (rb != 1) return false;
+        if (j > 0) rb = b[size_t(j - 1)];
+    }
+    int const n = int(rev.size());
+    pieces.assign(rev.rbegin(), rev.rend());
+    auto flip = [&](std::vector<std::vector<int>>& p) {
+        for (auto& v : p) {
+            for (int& x : v) x = n - 1 - x;
+            std::reverse(v.begin(), v.end());
+        }
+    };
+    flip(pa);
+    flip(pb);
+    parts_a = pa;
+    parts_b = pb;
+    return true;
+}
+
+std::vector<int> expand(std::vector<int> const& inn, std::vector<std::vector<int>> const& parts)
+{
+    std::vector<int> r;
+    for (int m : inn) r.insert(r.end(), parts[size_t(m)].begin(), parts[size_t(m)].end());
+    return r;
+}
+
 // The einsummable that computes v with u in place of its input k, or nothing when the two
-// do not line up.  v reads input k position by position over its join modes.
+// do not line up.  v reads input k position by position over its join modes; u has no
+// aggregation.  The two may cut the same elements into modes differently ([32, 4194304]
+// against [65536, 2048]): both are rewritten over the common pieces first.
 std::optional<einsummable_t> merged(einsummable_t const& u, einsummable_t const& v, int k)
 {
-    int const Ru = int(u.join_shape.size());
-    int const Rv = int(v.join_shape.size());
     if (u.out_dtype() != v.inn_dtype(k) || u.out_nelem() != v.inn_nelem(k)) return std::nullopt;
     if (u.inns.size() + v.inns.size() - 1 > 6) return std::nullopt;
-    std::vector<std::vector<int>> u_inns = u.inns, v_inns = v.inns;
-    std::vector<uint64_t>         shape = v.join_shape;
-    int                           out_rank = v.out_rank;
-    auto all_iota = [](einsummable_t const& e) {
-        if (e.has_aggregation()) return false;
-        for (auto const& inn : e.inns) {
-            if (!is_iota(inn, int(e.join_shape.size()))) return false;
-        }
-        return true;
-    };
-    auto iota = [](int rank) {
-        std::vector<int> r(size_t(rank), 0);
-        for (int i = 0; i != rank; ++i) r[size_t(i)] = i;
-        return r;
-    };
-    if (u.join_shape == v.join_shape) {
-        // as they are
-    } else if (all_iota(v)) {
-        // v is a map over positions: it takes the shape u gives them
-        shape = u.join_shape;
-        out_rank = Ru;
-        for (auto& inn : v_inns) inn = iota(Ru);
-    } else if (all_iota(u)) {
-        for (auto& inn : u_inns) inn = iota(Rv);
-    } else {
-        return std::nullopt;
+    std::vector<uint64_t>         shape;
+    std::vector<std::vector<int>> pu, pv;
+    if (!refine(u.join_shape, v.join_shape, shape, pu, pv)) return std::nullopt;
+    if (shape.size() > 8) return std::nullopt;
+    int out_rank = 0;
+    for (int m = 0; m != v.out_rank; ++m) out_rank += int(pv[size_t(m)].size());
+    if (out_rank == 0) return std::nullopt;
+    std::vector<std::vector<int>> inns;
+    for (auto const& inn : u.inns) inns.push_back(expand(inn, pu));
+    for (int i = 0; i != int(v.inns.size()); ++i) {
+        if (i != k) inns.push_back(expand(v.inns[size_t(i)], pv));
     }
-    std::vector<std::vector<int>> inns = u_inns;
-    for (int i = 0; i != int(v_inns.size()); ++i) {
-        if (i != k) inns.push_back(v_inns[size_t(i)]);
+    // einsummable_t::make numbers aggregated modes by first appearance: they must already
+    // appear in ascending order, or extents and modes would part ways
+    int next = out_rank;
+    for (auto const& inn : inns) {
+        if (inn.empty()) return std::nullopt;
+        for (int m : inn) {
+            if (m > next) return std::nullopt;
+            if (m == next) ++next;
+        }
     }
     try {
         return einsummable_t::make(shape, inns, out_rank, scalarop_t::compose(v.join, k, u.join),
@@ -349,103 +395,135 @@ std::optional<einsummable_t> merged(einsummable_t const& u, einsummable_t const&
     }
 }
 
+// Smallest element among the output and the inputs: the generated reductions take 16 bytes of
+// it per lane, so it decides how a row's elements are dealt to the lanes, i.e. the order of
+// the sum.
+uint64_t smallest_element(einsummable_t const& e)
+{
+    uint64_t m = dtype_size(e.out_dtype());
+    for (int k = 0; k != int(e.inns.size()); ++k) m = std::min(m, dtype_size(e.inn_dtype(k)));
+    return m;
+}
+
+uint64_t input_bytes(einsummable_t const& e)
+{
+    uint64_t b = 0;
+    for (int k = 0; k != int(e.inns.size()); ++k) b += e.inn_nelem(k) * dtype_size(e.inn_dtype(k));
+    return b;
+}
+
 }  // namespace
 
-bool apply_graph_t::absorb_producer(int v)
+// Tries to make node u's output unnecessary: every node that reads it computes it for itself
+// (or, for a whole-range copy, u writes the copy's output).  True when u became a dummy.
+bool apply_graph_t::absorb_into_readers(int u)
 {
-    node_t& nv = nodes_[size_t(v)];
     int const n = int(nodes_.size());
-    std::vector<int> candidates;  // indices into nv.mems
-    bool const copy = nv.kind == kind_t::touch;
+    node_t&   nu = nodes_[size_t(u)];
+    if (nu.kind != kind_t::einsummable) return false;
+    mem_t const S = nu.mems[0];
+    if (S.size == 0) return false;
+    for (size_t i = 1; i != nu.mems.size(); ++i) {
+        if (overlaps(nu.mems[i], S)) return false;
+    }
+    // who reads S before it is deleted; nobody may rewrite it or, while readers are still to
+    // come, what u reads
+    std::vector<int> readers, slots;
+    bool             deleted = false, clobbered = false;
+    for (int w = u + 1; w < n && !deleted; ++w) {
+        node_t const& nw = nodes_[size_t(w)];
+        if (nw.kind == kind_t::dummy) {
+            deleted = !readers.empty() && covers(nw.mems[0], S) &&
+                      std::binary_search(nw.deps.begin(), nw.deps.end(), readers.back());
+            continue;
+        }
+        bool const writes = nw.kind != kind_t::evict;
+        int        slot = -1, touching = 0;
+        for (size_t i = 1; i < nw.mems.size(); ++i) {
+            if (!overlaps(nw.mems[i], S)) continue;
+            ++touching;
+            if (same_range(nw.mems[i], S)) slot = int(i);
+        }
+        if (touching) {
+            if (touching != 1 || slot < 0 || clobbered) return false;
+            if (writes && overlaps(nw.mems[0], S)) return false;
+            for (size_t i = 1; writes && i != nu.mems.size(); ++i) {
+                if (overlaps(nw.mems[0], nu.mems[i])) return false;  // it would overwrite what it now reads
+            }
+            readers.push_back(w);
+            slots.push_back(slot);
+            continue;
+        }
+        if (!writes) continue;
+        if (overlaps(nw.mems[0], S)) return false;
+        for (size_t i = 1; i != nu.mems.size(); ++i) clobbered = clobbered || overlaps(nw.mems[0], nu.mems[i]);
+    }
+    if (!deleted || readers.empty()) return false;
+
+    // what each reader becomes
+    std::vector<einsummable_t> fused;
+    node_t const&              first = nodes_[size_t(readers[0])];
+    bool const copy = readers.size() == 1 && first.kind == kind_t::touch;
     if (copy) {
-        touch_t const t = nv.touch.simplify();
+        touch_t const t = first.touch.simplify();
         if (t.castable || t.selection.size() != 1) return false;
         touchdim_t const& d = t.selection[0];
         if (d.d_inn != d.size || d.d_out != d.size || d.offset_inn || d.offset_out) return false;
-        if (d.size * dtype_size(t.dtype) != nv.mems[0].size || nv.mems[1].size != nv.mems[0].size) {
+        if (d.size * dtype_size(t.dtype) != first.mems[0].size || first.mems[1].size != first.mems[0].size) {
             return false;
         }
-        for (int w = 0; nv.group >= 0 && w != n; ++w) {
-            if (w != v && nodes_[size_t(w)].kind == kind_t::touch && nodes_[size_t(w)].group == nv.group) {
+        for (int w = 0; first.group >= 0 && w != n; ++w) {
+            if (w != readers[0] && nodes_[size_t(w)].kind == kind_t::touch &&
+                nodes_[size_t(w)].group == first.group) {
                 return false;
             }
         }
-        candidates.push_back(1);
-    } else if (nv.kind == kind_t::einsummable) {
-        einsummable_t const& e = nv.e;
-        if (e.join.has_variables() || (e.has_aggregation() && e.inns.size() != 1)) return false;
-        for (int k = 0; k != int(e.inns.size()); ++k) {
-            if (is_iota(e.inns[size_t(k)], int(e.join_shape.size()))) candidates.push_back(k + 1);
+        fused.push_back(nu.e);
+    } else {
+        if (!absorbable_producer(nu.e)) return false;
+        // every reader repeats u's reads; worth it while that is less than writing S once and
+        // reading it once per reader
+        uint64_t const in_u = input_bytes(nu.e), nr = readers.size();
+        if (nr > 1 && (nr - 1) * in_u >= (nr + 1) * S.size) return false;
+        for (size_t r = 0; r != readers.size(); ++r) {
+            node_t const& nv = nodes_[size_t(readers[r])];
+            if (nv.kind != kind_t::einsummable) return false;
+            einsummable_t const& e = nv.e;
+            int const            k = slots[r] - 1;
+            if (e.join.has_variables() || (e.has_aggregation() && e.inns.size() != 1)) return false;
+            if (!is_iota(e.inns[size_t(k)], int(e.join_shape.size()))) return false;
+            std::optional<einsummable_t> m = merged(nu.e, e, k);
+            if (!m) return false;
+            // A sum (or product) keeps its bits only if its elements are added in the same
+            // order: the same vector width, over the same innermost extent.  min and max do
+            // not care.
+            if (e.has_aggregation() && (e.castable.value() == castable_t::add ||
+                                        e.castable.value() == castable_t::mul)) {
+                if (smallest_element(m.value()) != smallest_element(e) ||
+                    m.value().join_shape.back() != e.join_shape.back()) {
+                    return false;
+                }
+            }
+            if (km_) {
+                try {
+                    if (!km_->build(m.value())) return false;
+                } catch (km_error const&) {
+                    return false;
+                } catch (ir_error const&) {
+                    return false;
+                }
+            }
+            fused.push_back(std::move(m.value()));
         }
     }
-    for (int slot : candidates) {
-        mem_t const S = nv.mems[size_t(slot)];
-        if (S.size == 0) continue;
-        bool clean = true;
-        for (size_t i = 0; i != nv.mems.size(); ++i) {
-            if (int(i) != slot && overlaps(nv.mems[i], S)) clean = false;
-        }
-        if (!clean) continue;
-        // the node that wrote S: the last one before v to write any of it
-        int u = -1;
-        for (int w = v - 1; w >= 0 && u < 0; --w) {
-            node_t const& nw = nodes_[size_t(w)];
-            if (nw.kind == kind_t::dummy || nw.kind == kind_t::evict) continue;
-            if (overlaps(nw.mems[0], S)) u = w;
-        }
-        if (u < 0) continue;
-        node_t& nu = nodes_[size_t(u)];
-        if (nu.kind != kind_t::einsummable || !same_range(nu.mems[0], S)) continue;
-        if (!copy && !absorbable_producer(nu.e)) continue;
-        for (size_t i = 1; i != nu.mems.size(); ++i) {
-            // u reads at v's place now: not what it would write there, not its own old output
-            if (overlaps(nu.mems[i], nv.mems[0]) || overlaps(nu.mems[i], S)) clean = false;
-        }
-        // between the two: nobody else reads S, nobody writes what u reads
-        for (int w = u + 1; w < v && clean; ++w) {
-            node_t const& nw = nodes_[size_t(w)];
-            if (nw.kind == kind_t::dummy) continue;
-            for (size_t i = 1; i < nw.mems.size(); ++i) clean = clean && !overlaps(nw.mems[i], S);
-            if (nw.kind == kind_t::evict) continue;
-            for (size_t i = 1; i != nu.mems.size(); ++i) {
-                clean = clean && !overlaps(nw.mems[0], nu.mems[i]);
-            }
-        }
-        if (!clean) continue;
-        // after v: S is deleted before anybody reads or rewrites it
-        bool deleted = false;
-        for (int w = v + 1; w < n && clean && !deleted; ++w) {
-            node_t const& nw = nodes_[size_t(w)];
-            if (nw.kind == kind_t::dummy) {
-                deleted = covers(nw.mems[0], S) &&
-                          std::binary_search(nw.deps.begin(), nw.deps.end(), v);
-                continue;
-            }
-            for (size_t i = nw.kind == kind_t::evict ? 1 : 0; i < nw.mems.size(); ++i) {
-                clean = clean && !overlaps(nw.mems[i], S);
-            }
-        }
-        if (!clean || !deleted) continue;
 
-        einsummable_t fused = nu.e;
-        if (!copy) {
-            std::optional<einsummable_t> m = merged(nu.e, nv.e, slot - 1);
-            if (!m) continue;
-            fused = std::move(m.value());
-        }
-        if (km_ && !copy) {
-            try {
-                if (!km_->build(fused)) continue;
-            } catch (km_error const&) {
-                continue;
-            } catch (ir_error const&) {
-                continue;
-            }
-        }
+    for (size_t r = 0; r != readers.size(); ++r) {
+        int const v = readers[r];
+        node_t&   nv = nodes_[size_t(v)];
         std::vector<mem_t> mems{nv.mems[0]};
         for (size_t i = 1; i != nu.mems.size(); ++i) mems.push_back(nu.mems[i]);
         for (size_t i = 1; i != nv.mems.size(); ++i) {
-            if (!copy && int(i) != slot) mems.push_back(nv.mems[i]);
+            if (!copy && int(i) != slots[r]) mems.push_back(nv.mems[i]);
         }
         std::vector<int> deps = nv.deps;
         deps.erase(std::remove(deps.begin(), deps.end(), u), deps.end());
@@ -453,30 +531,29 @@ bool apply_graph_t::absorb_producer(int v)
         std::sort(deps.begin(), deps.end());
         deps.erase(std::unique(deps.begin(), deps.end()), deps.end());
         nv.kind = kind_t::einsummable;
-        nv.e = std::move(fused);
+        nv.e = std::move(fused[r]);
         nv.mems = std::move(mems);
         nv.deps = std::move(deps);
         nv.group = -1;
-        nu.kind = kind_t::dummy;
-        nu.mems = {S};
-        // whoever waited for u to be done with its inputs waits for the node that reads them now
+        // whoever waited for u to be done with its inputs waits for the nodes that read them now
         for (int w = v + 1; w < n; ++w) {
             std::vector<int>& d = nodes_[size_t(w)].deps;
             if (std::binary_search(d.begin(), d.end(), u) && !std::binary_search(d.begin(), d.end(), v)) {
                 d.insert(std::upper_bound(d.begin(), d.end(), v), v);
             }
         }
-        return true;
     }
-    return false;
+    nu.kind = kind_t::dummy;
+    nu.mems = {S};
+    return true;
 }
 
 int apply_graph_t::optimize()
 {
     if (finalized_) throw km_error(km_status::invalid, "apply graph: already finalized");
     int absorbed = 0;
-    for (int v = 0; v != int(nodes_.size()); ++v) {
-        while (absorb_producer(v)) ++absorbed;
+    for (int u = 0; u != int(nodes_.size()); ++u) {
+        if (absorb_into_readers(u)) ++absorbed;
     }
     return absorbed;
 }

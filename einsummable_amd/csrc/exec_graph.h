@@ -79,17 +79,20 @@ public:
     void add_memory_dependencies();
 
     // Removes round trips through memory that the node list spells out but the results do not
-    // need, without changing one bit of what stays in memory.  A node v absorbs the node u
-    // that wrote one of its inputs when that range S is written by u alone, read by v alone
-    // and deleted afterwards -- a dummy that covers S and depends on v is read as S's del node
-    // (memgraph.h: del_t) -- and nothing between the two touches what u reads:
-    //  - v a touch that copies S whole (the formation / partialize copy that follows every
-    //    contraction and reduction, taskgraph.cc:3047-3061): u writes v's output itself;
-    //  - v an elementwise einsummable, or a reduction of one input, that takes S position by
-    //    position, and u elementwise: one einsummable whose join is v's with u's put in
-    //    place of the hole (scalarop_t::compose keeps the rounding a store and a load make).
-    // The merged node stands at v's place and u becomes a dummy, so ids, and dependencies on
-    // either, stay valid.  Einsummables the kernel manager cannot build stay as they are.
+    // need, without changing one bit of what stays in memory.  The output S of a node u need
+    // not be stored when u alone writes it, it is deleted after its readers -- a dummy that
+    // covers S and depends on the last of them is read as S's del node (memgraph.h: del_t) --
+    // and nothing before the last reader rewrites what u reads:
+    //  - the one reader is a touch that copies S whole (the formation / partialize copy that
+    //    follows every contraction and reduction, taskgraph.cc:3047-3061): u writes the
+    //    copy's output itself;
+    //  - every reader is an elementwise einsummable, or a reduction of one input, that takes S
+    //    position by position, and u is elementwise: each reader becomes one einsummable
+    //    whose join is its own with u's put in place of the hole (scalarop_t::compose keeps
+    //    the rounding a store and a load make).  With several readers u is computed once
+    //    per reader, which is taken while u's inputs are smaller than the traffic S caused.
+    // A merged node stands at its reader's place and u becomes a dummy, so ids, and
+    // dependencies on either, stay valid.  Einsummables the kernel manager cannot build stay as they are.
     // Before finalize; returns the number of nodes absorbed.  The reference has no such pass
     // at this level: its graphs reach the engine with these nodes in them.
     int optimize();
@@ -166,7 +169,7 @@ private:
     };
 
     int  insert(node_t&& n, std::vector<int> const& deps);
-    bool absorb_producer(int v);
+    bool absorb_into_readers(int u);
     void launch(node_t const& n, hipStream_t stream, char* arena) const;
 
     kernel_manager_t*        km_;

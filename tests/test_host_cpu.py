@@ -230,6 +230,40 @@ def test_exec_graph_optimize_absorbs_copies_and_single_reader_elementwise():
     assert g.launches() == 3                                 # b, f, keep
 
 
+def test_exec_graph_optimize_gives_every_reader_its_own_copy_of_a_cheap_producer():
+    """The softmax pattern: a conversion read by a row reduction and by an elementwise node,
+    the three cut into modes differently."""
+    import einsummable_amd as ea
+
+    E = ea.Einsummable
+    g = ea.ApplyGraph(None)
+    h, s_ = 4, 16
+    n = h * s_ * s_
+    m = lambda slot, nbytes: (slot * 8192, nbytes)
+    add = E([h, s_ * s_], [[0, 1], [1]], 2, "+[hole|f16@0,hole|f16@1]")
+    up = E([n], [[0]], 1, "to_f32[hole|f16@0]")
+    rmax = E([h * s_, s_], [[0, 1]], 1, "hole|f32@0", "^")
+    sub = E([h * s_, s_], [[0, 1], [0]], 2, "+[hole|f32@0,*[constant{f32|-1},hole|f32@1]]")
+    a = g.add_einsummable(add, [m(2, 2 * n), m(0, 2 * n), m(1, 2 * s_ * s_)])
+    b = g.add_einsummable(up, [m(3, 4 * n), m(2, 2 * n)])
+    g.add_dummy(m(2, 2 * n), [b])
+    c = g.add_einsummable(rmax, [m(4, 4 * h * s_), m(3, 4 * n)])
+    d = g.add_einsummable(sub, [m(5, 4 * n), m(3, 4 * n), m(4, 4 * h * s_)])
+    g.add_dummy(m(3, 4 * n), [c, d])
+    g.add_memory_dependencies()
+    assert g.optimize() == 2
+    assert g.describe(a).startswith("dummy") and g.describe(b).startswith("dummy")
+    inner = "to_f32[to_f32[to_f16[+[hole|f16@0,hole|f16@1]]]]"
+    # both readers over the common pieces [4, 16, 16]: the reduction keeps its two output modes
+    assert g.describe(c) == "einsummable 32768:256 0:2048 8192:512 | [4,16,16]^ 0.1.2.,1.2.->2 | " + inner
+    assert g.describe(d) == "einsummable 40960:4096 0:2048 8192:512 32768:256 | [4,16,16]: " + \
+        "0.1.2.,1.2.,0.1.->3 | +[" + inner + ",*[constant{f32|-1},hole|f32@2]]"
+    g.finalize(1)
+    assert g.launches() == 2
+    # the second reader waits for the first one's result, and both for what the producers waited for
+    assert c in g.node_info(d)[2]
+
+
 def test_exec_graph_optimize_leaves_what_it_cannot_prove():
     import einsummable_amd as ea
 
@@ -254,9 +288,21 @@ def test_exec_graph_optimize_leaves_what_it_cannot_prove():
     g.add_memory_dependencies()
     assert g.optimize() == 0
 
-    # the range is read again before it is deleted
+    # one of two readers cannot take the producer in (it transposes): the range stays
     g = ea.ApplyGraph(None)
+    tr = E([32, 32], [[1, 0]], 2, "hole|f32@0")
     a = g.add_einsummable(exp, [m(1), m(0)])
+    b = g.add_einsummable(sq, [m(2), m(1)])
+    c = g.add_einsummable(tr, [m(3), m(1)])
+    g.add_dummy(m(1), [b, c])
+    g.add_memory_dependencies()
+    assert g.optimize() == 0
+
+    # two readers, but the producer reads more than its result saves: three inputs of the
+    # result's size read twice against one write and two reads
+    g = ea.ApplyGraph(None)
+    fma = E([1024], [[0], [0], [0]], 1, "+[*[hole|f32@0,hole|f32@1],hole|f32@2]")
+    a = g.add_einsummable(fma, [m(1), m(0), m(5), m(6)])
     b = g.add_einsummable(sq, [m(2), m(1)])
     c = g.add_einsummable(sq, [m(3), m(1)])
     g.add_dummy(m(1), [b, c])
