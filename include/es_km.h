@@ -219,15 +219,17 @@ int es_km_graph_add_memory_dependencies(es_km_graph_t* g);
 /* Optional, before finalize: removes round trips through memory that change no stored bit.
  * A touch that copies a whole range which one einsummable wrote and nobody else reads (the
  * formation copy behind every contraction and reduction, src/einsummable/taskgraph.cc:
- * 3047-3061) is dropped and the einsummable writes the copy's output; an elementwise
- * einsummable, or a reduction of one input, whose input was written by an elementwise
- * einsummable and is read by nobody else becomes one einsummable with both joins, the inner
- * value rounded as the store between them rounded it.  Both need the range's del node
- * (memgraph.h: del_t) in the graph, as a dummy that covers the range and depends on the
- * reader: without it the range counts as a result and stays.  Node ids stay valid: the
- * absorbed node becomes a dummy.  *n_absorbed (may be null) receives how many were absorbed.
- * No counterpart in the reference, whose engine launches the nodes as the memgraph lists
- * them. */
+ * 3047-3061) is dropped and the einsummable writes the copy's output.  An elementwise
+ * einsummable whose output is read only by elementwise einsummables (or reductions of one
+ * input) that take it position by position is computed by each of those readers instead: a
+ * reader becomes one einsummable with both joins, the inner value rounded as the store
+ * between them rounded it.  With several readers that is taken while the producer's inputs are
+ * smaller than the traffic its output caused; a sum is only merged when its order of addition
+ * stays what it was.  Both need the range's del node (memgraph.h: del_t) in the graph, as a
+ * dummy that covers the range and depends on its last reader: without it the range counts as
+ * a result and stays.  Node ids stay valid: an absorbed node becomes a dummy.  *n_absorbed
+ * (may be null) receives how many were absorbed.  No counterpart in the reference, whose
+ * engine launches the nodes as the memgraph lists them. */
 int es_km_graph_optimize(es_km_graph_t* g, int* n_absorbed);
 
 /* Builds every einsummable (an unsupported one is an error here), places the nodes on
