@@ -74,7 +74,7 @@ struct tile_option_t {
 };
 
 void choose_tile(dtype_t dt, uint64_t M, uint64_t N, uint64_t K, uint64_t batch, bool dma_ok,
-                 int& bm, int& bn)
+                 bool big_ok, int& bm, int& bn)
 {
     bm = 128;
     bn = 128;
@@ -113,6 +113,7 @@ void choose_tile(dtype_t dt, uint64_t M, uint64_t N, uint64_t K, uint64_t batch,
     double best = 0;
     uint64_t const nk = K * dtype_size(dt) / 64;
     for (tile_option_t const& o : options) {
+        if (o.bm == 256 && o.bn == 256 && !big_ok) continue;
         uint64_t tiles = ((M + o.bm - 1) / o.bm) * ((N + o.bn - 1) / o.bn) * batch;
         // at most 128 tiles and a long reduction: plan_contraction will cut k into splits
         // (same rule as there), which costs a pass over the fp32 partial tiles.  In units of
@@ -305,7 +306,13 @@ std::shared_ptr<plan_t> plan_contraction(einsummable_t const& e, int)
     // large tiles exist in the direct-to-LDS kernel (both operands on a vector path) and, for
     // A along k, in the register-staged one
     if (dma_ok || (a.a_mode == 0 && a.b_mode != 2)) {
-        choose_tile(dt, M, N, K, Bt, dma_ok, p->bm, p->bn);
+        // The f16 256 x 256 tile is taken where the eight-wavefront kernel can run it (K in
+        // whole 128-byte slices): the four-wavefront instance of that tile needs more registers
+        // than a wave has and spills.
+        const char* waves = std::getenv("ES_KM_GEMM_WAVES");
+        bool const  big_ok = dt != dtype_t::f16 || !dma_ok ||
+                            (K % 64 == 0 && !(waves && waves[0] == '4'));
+        choose_tile(dt, M, N, K, Bt, dma_ok, big_ok, p->bm, p->bn);
     }
     a.tiles_m = uint32_t((M + p->bm - 1) / p->bm);
     a.tiles_n = uint32_t((N + p->bn - 1) / p->bn);
@@ -399,7 +406,7 @@ std::shared_ptr<plan_t> plan_contraction(einsummable_t const& e, int)
         }
     }
     a.wave8 = 0;
-    if (dt == dtype_t::f16 && p->planned_dma && a.a_mode == 0 && a.b_mode == 0 && !a.shortk &&
+    if (dt == dtype_t::f16 && p->planned_dma && a.a_mode <= 1 && a.b_mode <= 1 && !a.shortk &&
         !a.wide_slices && (p->bm == 256 || p->bn == 256) &&
         gemm::gemm_dma_wide_eligible<_Float16>(a, p->bm == 256 && p->bn == 256 ? 2u : 3u)) {
         const char* env = std::getenv("ES_KM_GEMM_WAVES");  // tuning and tests: 4 keeps the old kernel

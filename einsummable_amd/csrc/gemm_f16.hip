@@ -56,20 +56,35 @@ void launch_gemm_f16(int bm, int bn, gemm_args_t const& a, hipStream_t stream)
         // that one covers the other's waits.  Measured against the four-wavefront kernel on
         // 64-byte slices: 8192^3 1.13 -> 1.21 PFLOP/s, 4096^3 1.04 -> 1.14, 2048 x 4096 x
         // 4096 0.80 -> 1.00, 2048 x 11008 x 4096 0.86 -> 1.01 (results bit-identical).
-        if (a.wave8 && a.a_mode == 0 && a.b_mode == 0) {
-            if (bm == 256 && bn == 256 && gemm_dma_wide_eligible<T>(a, 2)) {
-                launch_gemm_dma_kernel_mode<T, 256, 256, 2, 0, 0, 128, 2, 4>(a, stream);
+        if (a.wave8 && a.a_mode <= 1 && a.b_mode <= 1) {
+            // (each operand along k or along its own m / n mode)
+            auto modes = [&](auto launch00, auto launch01, auto launch10, auto launch11) {
+                if (a.a_mode == 0) {
+                    a.b_mode == 0 ? launch00() : launch01();
+                } else {
+                    a.b_mode == 0 ? launch10() : launch11();
+                }
                 if (a.splits > 1) launch_gemm_fold<T>(a, stream);
+            };
+            if (bm == 256 && bn == 256 && gemm_dma_wide_eligible<T>(a, 2)) {
+                modes([&] { launch_gemm_dma_kernel_mode<T, 256, 256, 2, 0, 0, 128, 2, 4>(a, stream); },
+                      [&] { launch_gemm_dma_kernel_mode<T, 256, 256, 2, 0, 1, 128, 2, 4>(a, stream); },
+                      [&] { launch_gemm_dma_kernel_mode<T, 256, 256, 2, 1, 0, 128, 2, 4>(a, stream); },
+                      [&] { launch_gemm_dma_kernel_mode<T, 256, 256, 2, 1, 1, 128, 2, 4>(a, stream); });
                 return;
             }
             if (bm == 256 && bn == 128 && gemm_dma_wide_eligible<T>(a, 3)) {
-                launch_gemm_dma_kernel_mode<T, 256, 128, 3, 0, 0, 128, 4, 2>(a, stream);
-                if (a.splits > 1) launch_gemm_fold<T>(a, stream);
+                modes([&] { launch_gemm_dma_kernel_mode<T, 256, 128, 3, 0, 0, 128, 4, 2>(a, stream); },
+                      [&] { launch_gemm_dma_kernel_mode<T, 256, 128, 3, 0, 1, 128, 4, 2>(a, stream); },
+                      [&] { launch_gemm_dma_kernel_mode<T, 256, 128, 3, 1, 0, 128, 4, 2>(a, stream); },
+                      [&] { launch_gemm_dma_kernel_mode<T, 256, 128, 3, 1, 1, 128, 4, 2>(a, stream); });
                 return;
             }
             if (bm == 128 && bn == 256 && gemm_dma_wide_eligible<T>(a, 3)) {
-                launch_gemm_dma_kernel_mode<T, 128, 256, 3, 0, 0, 128, 2, 4>(a, stream);
-                if (a.splits > 1) launch_gemm_fold<T>(a, stream);
+                modes([&] { launch_gemm_dma_kernel_mode<T, 128, 256, 3, 0, 0, 128, 2, 4>(a, stream); },
+                      [&] { launch_gemm_dma_kernel_mode<T, 128, 256, 3, 0, 1, 128, 2, 4>(a, stream); },
+                      [&] { launch_gemm_dma_kernel_mode<T, 128, 256, 3, 1, 0, 128, 2, 4>(a, stream); },
+                      [&] { launch_gemm_dma_kernel_mode<T, 128, 256, 3, 1, 1, 128, 2, 4>(a, stream); });
                 return;
             }
         }

@@ -251,7 +251,12 @@ def test_big_tile_kernels(km, monkeypatch, case, tile):
 
 
 EIGHT_WAVE_CASES = [
-    # both operands along k, K a whole number of 128-byte slices: the eight-wavefront kernels
+    # K a whole number of 128-byte slices: the eight-wavefront kernels, each operand along k
+    # or along its own mode
+    ("ij,jk->ik", dict(i=520, j=448, k=264)),                    # B along n
+    ("ji,kj->ik", dict(i=264, j=448, k=520)),                    # A along m
+    ("ji,jk->ik", dict(i=272, j=192, k=264)),                    # both
+    ("bij,bjk->bik", dict(b=2, i=264, j=256, k=136)),
     ("ij,kj->ik", dict(i=512, j=512, k=512)),                    # full tiles
     ("ij,kj->ik", dict(i=264, j=448, k=520)),                    # ragged m and n, seven slices
     ("ij,kj->ik", dict(i=40, j=192, k=24)),                      # one partial tile, three slices
