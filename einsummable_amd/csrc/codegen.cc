@@ -1075,10 +1075,15 @@ std::vector<char> compile_hip_source(std::string const& source, std::string cons
         throw km_error(km_status::device, "hiprtcCreateProgram failed");
     }
     std::string arch_opt = "--offload-arch=" + arch;
-    // packed-fp32 instruction selection is switched off for all device code of this library
+    // packed-fp32 instruction selection is switched off for all device code of this library.
+    // No contraction of a product and a sum into a fused multiply-add: every node of a join
+    // rounds by itself, as the reference's interpreter does, and -- what matters when the
+    // exec graph merges two einsummables into one kernel -- the same expression gives the same
+    // bits in whatever kernel it ends up (left to the compiler, 1.7 * x + y became an FMA in
+    // a kernel of its own and a product and a sum inside a larger join).
     const char* opts[] = {arch_opt.c_str(), "-O3",      "-std=c++17",       "-Xclang",
-                          "-target-feature", "-Xclang", "-packed-fp32-ops"};
-    int         n_opts = 7;
+                          "-target-feature", "-Xclang", "-packed-fp32-ops", "-ffp-contract=off"};
+    int         n_opts = 8;
     hiprtcResult rc = hiprtcCompileProgram(prog, n_opts, opts);
     if (rc != HIPRTC_SUCCESS) {
         size_t n = 0;
@@ -1110,7 +1115,7 @@ namespace
 // by default it is $XDG_CACHE_HOME/es_km or $HOME/.cache/es_km.  Files are written under a
 // temporary name and renamed, so concurrent processes never see half a file.
 
-constexpr char COMPILE_OPTIONS[] = "gfx950 -O3 -std=c++17 -packed-fp32-ops";
+constexpr char COMPILE_OPTIONS[] = "gfx950 -O3 -std=c++17 -packed-fp32-ops -ffp-contract=off";
 
 std::string cache_dir()
 {

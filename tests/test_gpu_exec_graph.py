@@ -350,6 +350,104 @@ def test_optimized_layer_keeps_every_stored_bit(km, shape, n_streams):
         assert torch.equal(a, b), name
 
 
+def random_ssa_graph(r, n_nodes):
+    """Every node writes a slot of its own: elementwise nodes whose joins invite a fused
+    multiply-add across a merge, conversions through f16, broadcasts of a row statistic, row
+    maxima and sums, whole-range copies.  Returns (nodes, slot sizes, input slots)."""
+    R, C = 64, 96
+    n = R * C
+    bounded = "*[hole|f32@0,power{-1}[+[constant{f32|1},*[hole|f32@0,hole|f32@0]]]]"   # x / (1 + x^2)
+    full = [("f32", n)] * 3          # slots 0..2 are inputs
+    kinds = ["f32"] * 3
+    nodes = []
+    def pick(kind):
+        c = [i for i, k in enumerate(kinds) if k == kind]
+        return int(c[r.randint(0, len(c))]) if c else None
+    for _ in range(n_nodes):
+        op = r.choice(["bounded", "axpy", "mul", "half", "unhalf", "rowmax", "rowsum", "bcast", "copy",
+                       "scale"], p=[0.15, 0.15, 0.1, 0.1, 0.1, 0.08, 0.08, 0.1, 0.07, 0.07])
+        out = len(kinds)
+        a, b = pick("f32"), pick("f32")
+        if op == "bounded":
+            nodes.append((E([n], [[0]], 1, bounded), out, [a])); kinds.append("f32")
+        elif op == "scale":
+            nodes.append((E([R, C], [[0, 1]], 2, "*[constant{f32|0.75},hole|f32@0]"), out, [a])); kinds.append("f32")
+        elif op == "axpy":
+            nodes.append((E([n], [[0], [0]], 1, "+[*[constant{f32|1.7},hole|f32@0],hole|f32@1]"), out, [a, b]))
+            kinds.append("f32")
+        elif op == "mul":
+            nodes.append((E([R, C], [[0, 1], [0, 1]], 2, "*[hole|f32@0,hole|f32@1]"), out, [a, b])); kinds.append("f32")
+        elif op == "half":
+            nodes.append((E([n], [[0]], 1, "to_f16[hole|f32@0]"), out, [a])); kinds.append("f16")
+        elif op == "unhalf":
+            h = pick("f16")
+            if h is None:
+                continue
+            nodes.append((E([n], [[0]], 1, "to_f32[hole|f16@0]"), out, [h])); kinds.append("f32")
+        elif op in ("rowmax", "rowsum"):
+            nodes.append((E([R, C], [[0, 1]], 1, "hole|f32@0", "^" if op == "rowmax" else "+"), out, [a]))
+            kinds.append("row")
+        elif op == "bcast":
+            row = pick("row")
+            if row is None:
+                continue
+            nodes.append((E([R, C], [[0, 1], [0]], 2, "+[hole|f32@0,*[constant{f32|-0.01},hole|f32@1]]"), out,
+                          [a, row]))
+            kinds.append("f32")
+        else:
+            nodes.append((ea.Touch([(n, n, 0, 0, n)], None, ea.F32), out, [a])); kinds.append("f32")
+    size = {"f32": 4 * n, "f16": 2 * n, "row": 4 * R}
+    return nodes, [size[k] for k in kinds], 3
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_optimized_random_graphs_keep_every_stored_bit(km, seed):
+    import torch
+
+    r = rng(300 + seed)
+    nodes, sizes, n_inputs = random_ssa_graph(r, 40)
+    offs = np.concatenate([[0], np.cumsum([(s + 255) // 256 * 256 for s in sizes])]).astype(np.int64)
+    mem = lambda k: (int(offs[k]), sizes[k])
+    init = normal(r, int(offs[-1]) // 4, np.float32)
+    arenas, graphs, ids = [], [], []
+    for optimize in (False, True):
+        g = ea.ApplyGraph(km)
+        my = []
+        last_reader = {}
+        for what, out, inns in nodes:
+            if isinstance(what, ea.Touch):
+                i = g.add_touch(what, -1, [mem(out), mem(inns[0])])
+            else:
+                i = g.add_einsummable(what, [mem(out)] + [mem(k) for k in inns])
+            my.append(i)
+            for k in inns:
+                last_reader[k] = i
+        # del nodes for most of what is read at all; the rest counts as results
+        rr = rng(400 + seed)
+        for k, i in sorted(last_reader.items()):
+            if k >= n_inputs and rr.uniform() < 0.85:
+                g.add_dummy(mem(k), [i])
+        g.add_memory_dependencies()
+        absorbed = g.optimize() if optimize else 0
+        g.finalize(2)
+        arena = torch.from_numpy(init.copy()).cuda()
+        g.run(stream_handle(), arena.data_ptr())
+        torch.cuda.synchronize()
+        arenas.append(arena.cpu().numpy().view(np.uint8))
+        graphs.append(g)
+        ids.append(my)
+    assert absorbed > 0
+    assert graphs[1].launches() == graphs[0].launches() - absorbed
+    kept = 0
+    for (what, out, inns), i in zip(nodes, ids[1]):
+        if graphs[1].describe(i).startswith("dummy"):
+            continue
+        lo, nb = mem(out)
+        assert np.array_equal(arenas[0][lo:lo + nb], arenas[1][lo:lo + nb]), (seed, i, graphs[1].describe(i))
+        kept += 1
+    assert kept > 0
+
+
 @pytest.mark.parametrize("n_streams", [
     1,
     pytest.param(4, marks=pytest.mark.skip(
