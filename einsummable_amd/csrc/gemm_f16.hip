@@ -9,34 +9,45 @@ namespace gemm
 {
 
 __global__ __launch_bounds__(256) void gemm_warm_kernel(chunk_t const* p, uint64_t n_chunks,
+                                                        chunk_t const* q, uint64_t n_chunks_q,
                                                         uint32_t* sink)
 {
-    // 16 bytes per lane, four grid strides per thread; what is read is folded into a word
-    // that is stored only to a sink nobody passes, which keeps the loads alive
+    // 16 bytes per lane, four grid strides per thread, first over p, then over q; what is read
+    // is folded into a word that is stored only to a sink nobody passes, which keeps the loads
+    // alive
     uint64_t const stride = uint64_t(gridDim.x) * 256;
+    uint64_t const total = n_chunks + n_chunks_q;
     uint64_t       i = uint64_t(blockIdx.x) * 256 + threadIdx.x;
     uint32_t       acc = 0;
 #pragma unroll
     for (int r = 0; r != 4; ++r, i += stride) {
-        if (i < n_chunks) {
-            chunk_t const v = p[i];
+        if (i < total) {
+            chunk_t const v = i < n_chunks ? p[i] : q[i - n_chunks];
             acc ^= v[0] ^ v[1] ^ v[2] ^ v[3];
         }
     }
     if (sink && acc == 0x9e3779b9u) *sink = acc;
 }
 
-void gemm_warm_operands(void const* p, uint64_t bytes, hipStream_t stream)
+// Reads both operands (either may be empty) into the memory-side cache with one launch.
+void gemm_warm_operands(void const* p, uint64_t bytes_p, void const* q, uint64_t bytes_q,
+                        hipStream_t stream)
 {
     // the part before the first and after the last whole 16 bytes is left out: it shares its
     // lines with chunks that are read
-    uint64_t const addr = reinterpret_cast<uint64_t>(p);
-    uint64_t const first = (addr + 15) & ~uint64_t(15);
-    if (bytes < 64 || first - addr >= bytes) return;
-    uint64_t const n_chunks = (bytes - (first - addr)) / 16;
-    uint64_t const blocks = (n_chunks + 1023) / 1024;
-    hipLaunchKernelGGL(gemm_warm_kernel, dim3(unsigned(blocks)), dim3(256), 0, stream,
-                       reinterpret_cast<chunk_t const*>(first), n_chunks,
+    auto whole = [](void const* x, uint64_t bytes, chunk_t const*& first, uint64_t& n) {
+        uint64_t const addr = reinterpret_cast<uint64_t>(x);
+        uint64_t const lo = (addr + 15) & ~uint64_t(15);
+        first = reinterpret_cast<chunk_t const*>(lo);
+        n = (bytes < 64 || lo - addr >= bytes) ? 0 : (bytes - (lo - addr)) / 16;
+    };
+    chunk_t const *fp, *fq;
+    uint64_t       np, nq;
+    whole(p, bytes_p, fp, np);
+    whole(q, bytes_q, fq, nq);
+    if (np + nq == 0) return;
+    uint64_t const blocks = (np + nq + 1023) / 1024;
+    hipLaunchKernelGGL(gemm_warm_kernel, dim3(unsigned(blocks)), dim3(256), 0, stream, fp, np, fq, nq,
                        static_cast<uint32_t*>(nullptr));
 }
 
@@ -46,8 +57,9 @@ void launch_gemm_f16(int bm, int bn, gemm_args_t const& a, hipStream_t stream)
 {
     using T = _Float16;
     if (a.tiles_m == 0) return;
-    if (a.warm_a_bytes) gemm_warm_operands(a.A, a.warm_a_bytes, stream);
-    if (a.warm_b_bytes) gemm_warm_operands(a.B, a.warm_b_bytes, stream);
+    if (a.warm_a_bytes || a.warm_b_bytes) {
+        gemm_warm_operands(a.A, a.warm_a_bytes, a.B, a.warm_b_bytes, stream);
+    }
     if (gemm_dma_eligible<T>(a)) {
         if (a.shortk && gemm_shortk_eligible(a)) return launch_gemm_shortk(a, stream);
         // Compute-bound products with both operands along k: slices of 128 bytes per row

@@ -912,7 +912,8 @@ double probe_mfma_f16(void const* operands, void* scratch, int blocks, int iters
 // reads that have to go to HBM in the middle of that write stream cost far more than their
 // size suggests (attention scores, 128 MiB of operands against 1 GiB of output: 0.35 ms
 // with cold operands, 0.21 ms with warm ones plus 0.03 ms for warming them).
-void gemm_warm_operands(void const* p, uint64_t bytes, hipStream_t stream);
+void gemm_warm_operands(void const* p, uint64_t bytes_p, void const* q, uint64_t bytes_q,
+                        hipStream_t stream);
 
 // The fp16 kernel for reductions of exactly 128 elements (gemm_shortk_kernel.h)
 bool gemm_shortk_eligible(gemm_args_t const& a);
