@@ -264,6 +264,51 @@ def test_exec_graph_optimize_gives_every_reader_its_own_copy_of_a_cheap_producer
     assert c in g.node_info(d)[2]
 
 
+def test_exec_graph_optimize_brings_modes_to_their_common_pieces_or_declines():
+    import einsummable_amd as ea
+
+    E = ea.Einsummable
+    m = lambda slot, nbytes=4096: (slot * 8192, nbytes)
+
+    def pair(u, v, v_inputs):
+        g = ea.ApplyGraph(None)
+        a = g.add_einsummable(u, [m(1, 96), m(0, 96)])
+        b = g.add_einsummable(v, [m(2, 96)] + v_inputs)
+        g.add_dummy(m(1, 96), [b])
+        g.add_memory_dependencies()
+        return g, g.optimize(), b
+
+    # [6, 4] against [4, 6]: a mode of one straddles a boundary of the other unevenly
+    u = E([6, 4], [[0, 1]], 2, "exp[hole|f32@0]")
+    v = E([4, 6], [[0, 1], [1]], 2, "*[hole|f32@0,hole|f32@1]")
+    g, n, b = pair(u, v, [m(1, 96), m(3, 24)])
+    assert n == 0
+
+    # [2, 12] and [4, 6] meet in [2, 2, 6]; the broadcast input keeps its one mode
+    u = E([2, 12], [[0, 1]], 2, "exp[hole|f32@0]")
+    g, n, b = pair(u, v, [m(1, 96), m(3, 24)])
+    assert n == 1
+    assert g.describe(b).endswith("| [2,2,6]: 0.1.2.,2.->3 | *[to_f32[exp[hole|f32@0]],hole|f32@1]")
+
+    # modes of extent one on either side
+    u = E([1, 24, 1], [[0, 1, 2]], 3, "exp[hole|f32@0]")
+    v = E([24], [[0]], 1, "*[constant{f32|2},hole|f32@0]")
+    g, n, b = pair(u, v, [m(1, 96)])
+    assert n == 1, g.describe(b)
+
+    # a row sum keeps its innermost extent and its element size, or stays as it is
+    u = E([4, 6], [[0, 1]], 2, "exp[hole|f32@0]")
+    rsum = E([4, 6], [[0, 1]], 1, "hole|f32@0", "+")
+    g, n, b = pair(u, rsum, [m(1, 96)])
+    assert n == 1 and "[4,6]+ 0.1.->1 | to_f32[exp[hole|f32@0]]" in g.describe(b)
+    up = E([24], [[0]], 1, "to_f32[hole|f16@0]")
+    g, n, b = pair(up, rsum, [m(1, 96)])
+    assert n == 0                                   # 2-byte elements would be dealt to the lanes differently
+    rmax = E([4, 6], [[0, 1]], 1, "hole|f32@0", "^")
+    g, n, b = pair(up, rmax, [m(1, 96)])
+    assert n == 1                                   # a maximum does not care
+
+
 def test_exec_graph_optimize_leaves_what_it_cannot_prove():
     import einsummable_amd as ea
 
