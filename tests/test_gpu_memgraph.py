@@ -73,10 +73,12 @@ def test_every_node_kind_runs(km, n_streams):
     assert np.array_equal(got[~touched], init[~touched])
 
 
-def layer_memgraph(graph, ranges):
+def layer_memgraph(graph, ranges, with_dels=False):
     """The decoder layer's node list as a memgraph: an inputmem per buffer nobody writes,
     an alloc per buffer somebody writes, one apply / constant per node, and the edges the
-    memory ranges imply (the memgraph carries edges, not ranges, for ordering)."""
+    memory ranges imply (the memgraph carries edges, not ranges, for ordering).  `with_dels`:
+    a del node, behind all its readers, for every buffer that is neither an input nor the
+    layer's output (memgraph.h: del_t)."""
     def overlap(x, y):
         return x[0] < y[0] + y[1] and y[0] < x[0] + x[1]
 
@@ -119,6 +121,11 @@ def layer_memgraph(graph, ranges):
                                start=n["start"]))
         history.append((len(nodes), out, inns))
         nodes.append(m)
+    if with_dels:
+        for name, (off, size) in ranges.items():
+            readers = {i for i, _, rs in history if any(overlap((off, size), x) for x in rs)}
+            if name in written and name != graph.output and readers:
+                nodes.append(node("del", readers, loc=0, offset=off, size=size))
     return dict(num_compute_locs=1, num_storage_locs=0, nodes=nodes)
 
 
@@ -149,6 +156,36 @@ def test_llama_layer_replayed_from_wire_equals_node_by_node_launches(km, n_strea
     torch.cuda.synchronize()
     host = arena.cpu().numpy()
     for name, (o, nb) in ranges.items():
+        assert np.array_equal(seq.get(name, np.uint8), host[o:o + nb]), name
+
+
+def test_llama_layer_from_wire_optimized_keeps_the_result(km):
+    """The del nodes of a serialized memgraph are what the optimisation pass needs: the layer
+    loaded from the wire, optimised, gives the bytes of the node-by-node run in its output."""
+    import torch
+
+    lg = LayerGraph(dim=256, n_heads=4, ffn=688, seq=128)
+    vals = make_inputs(lg, 6)
+    seq = DeviceRunner(km, lg)
+    ranges, off = {}, 0
+    for name, nbytes in lg.buffers.items():
+        ranges[name] = (off, nbytes)
+        off += (nbytes + 255) // 256 * 256
+    g = ea.ApplyGraph(km)
+    g.load_memgraph(mp.to_wire(layer_memgraph(lg, ranges, with_dels=True)))
+    assert g.optimize() == 27          # as when the runner adds the del nodes itself
+    g.finalize(2)
+    arena = torch.zeros(g.arena_bytes(), dtype=torch.uint8, device="cuda")
+    for k, v in vals.items():
+        seq.set_input(k, v)
+        o, nb = ranges[k]
+        arena[o:o + nb] = torch.from_numpy(np.ascontiguousarray(v).view(np.uint8).reshape(-1)).cuda()
+    seq.run()
+    g.run(stream_handle(), arena.data_ptr())
+    torch.cuda.synchronize()
+    host = arena.cpu().numpy()
+    for name in (lg.output, "values.f", "sm.to_f16", "gate"):
+        o, nb = ranges[name]
         assert np.array_equal(seq.get(name, np.uint8), host[o:o + nb]), name
 
 
