@@ -536,7 +536,9 @@ bool apply_graph_t::absorb_into_readers(int u)
         nv.deps = std::move(deps);
         nv.group = -1;
         // whoever waited for u to be done with its inputs waits for the nodes that read them now
+        // (the other readers only shared u with this one)
         for (int w = v + 1; w < n; ++w) {
+            if (std::find(readers.begin(), readers.end(), w) != readers.end()) continue;
             std::vector<int>& d = nodes_[size_t(w)].deps;
             if (std::binary_search(d.begin(), d.end(), u) && !std::binary_search(d.begin(), d.end(), v)) {
                 d.insert(std::upper_bound(d.begin(), d.end(), v), v);
