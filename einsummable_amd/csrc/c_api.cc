@@ -477,6 +477,7 @@ es_km_graph_t* es_km_graph_create(es_km_t* h)
 
 void es_km_graph_destroy(es_km_graph_t* g) { delete g; }
 
+extern "C++" {
 namespace
 {
 std::vector<es::mem_t> make_mems(const uint64_t* offsets, const uint64_t* sizes, int n)
@@ -492,6 +493,7 @@ std::vector<int> make_deps(const int* deps, int n)
     return std::vector<int>(deps, deps + n);
 }
 }  // namespace
+}  // extern "C++"
 
 int es_km_graph_add_einsummable(es_km_graph_t* g, const uint64_t* join_shape, int join_rank,
                                 const int* inns_flat, const int* inns_offsets, int n_inns,
