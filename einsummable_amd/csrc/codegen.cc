@@ -187,8 +187,9 @@ __device__ __forceinline__ double keep_apart(double v)
     return v;
 }
 __device__ __forceinline__ c64 keep_apart(c64 v) { return c64{keep_apart(v.re), keep_apart(v.im)}; }
+// (at most 16 bytes of alignment: a wider vector moves as 16-byte pieces)
 template <typename T, int N>
-struct __attribute__((aligned(sizeof(T) * N))) vec_t { T v[N]; };
+struct __attribute__((aligned(sizeof(T) * N < 16 ? sizeof(T) * N : 16))) vec_t { T v[N]; };
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 struct u32x8 { u32x4 lo, hi; };
 // vector load / store; NT != 0 marks the access non-temporal (streamed once, no reuse)
@@ -608,6 +609,19 @@ cg_kernel_t gen_elementwise(einsummable_t const& e, int max_vec)
     return std::move(g.k);
 }
 
+}  // namespace
+
+// Elements of a row that one lane takes per step of a row reduction.  It fixes how a row is
+// dealt to the lanes, i.e. the order of a sum: the same for 2- and 4-byte elements (16 bytes
+// of the former, two 16-byte pieces of the latter), so that a reduction keeps its order when
+// its input arrives in another of those types.
+int row_reduction_lane_elems(int smallest_elem_bytes)
+{
+    return smallest_elem_bytes <= 4 ? 8 : std::max(1, 16 / smallest_elem_bytes);
+}
+
+namespace
+{
 // --------------------------------------------------------------- reduce, aggregated modes
 // innermost: a team of TEAM lanes (one wavefront, or a 256-thread workgroup for long rows)
 // owns one output element, strides over the flattened aggregated index space in V-element
@@ -630,7 +644,7 @@ cg_kernel_t gen_reduce_row(einsummable_t const& e, int max_vec)
     uint64_t nA = 1;
     for (int m = O; m != R; ++m) nA *= L.shape[m];
     uint64_t const n_out = e.out_nelem();
-    int const vcap = std::min(max_vec, 16 / min_elem_size(e));
+    int const vcap = std::min(max_vec, row_reduction_lane_elems(min_elem_size(e)));
     int const V = pow2_divisor(L.shape[R - 1], vcap);
     uint64_t const nvecA = nA / uint64_t(V);
     int const TEAM = env_int("ES_KM_RED_TEAM", (nvecA >= 512) ? 256 : 64) == 256 ? 256 : 64;
@@ -843,7 +857,7 @@ cg_kernel_t gen_reduce_row(einsummable_t const& e, int max_vec)
     g.k.out_inn_align.push_back(int(dtype_size(od)));
     for (int k = 0; k != L.NI; ++k) {
         bool wide = acc[k] == access_t::vec && !row_const[k];
-        g.k.out_inn_align.push_back((wide ? V : 1) * int(dtype_size(e.inn_dtype(k))));
+        g.k.out_inn_align.push_back(std::min(16, (wide ? V : 1) * int(dtype_size(e.inn_dtype(k)))));
     }
     return std::move(g.k);
 }
@@ -1058,12 +1072,17 @@ cg_kernel_t generate_kernel(einsummable_t const& e, int max_vec)
         (e.castable.value() == castable_t::min || e.castable.value() == castable_t::max)) {
         throw ir_error("generate_kernel: min/max aggregation of complex values");
     }
+    return is_row_reduction(e) ? gen_reduce_row(e, max_vec) : gen_reduce_col(e, max_vec);
+}
+
+bool is_row_reduction(einsummable_t const& e)
+{
+    if (!e.has_aggregation()) return false;
     int const R = int(e.join_shape.size());
-    bool      row = false;
     for (int k = 0; k != int(e.inns.size()); ++k) {
-        row = row || (!e.inns[k].empty() && e.inns[k].back() == R - 1);
+        if (!e.inns[k].empty() && e.inns[k].back() == R - 1) return true;
     }
-    return row ? gen_reduce_row(e, max_vec) : gen_reduce_col(e, max_vec);
+    return false;
 }
 
 std::vector<char> compile_hip_source(std::string const& source, std::string const& name,

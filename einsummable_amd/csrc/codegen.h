@@ -42,6 +42,14 @@ struct cg_kernel_t {
 // the scalar variant used when a buffer is not 16-byte aligned).
 cg_kernel_t generate_kernel(einsummable_t const& e, int max_vec = 16);
 
+// Elements of a row per lane and step in the generated row reductions, by the smallest element
+// among output and inputs: two reductions that agree in it (and in the row's length) add a
+// row's elements in the same order.
+int row_reduction_lane_elems(int smallest_elem_bytes);
+
+// Whether generate_kernel makes a row reduction of e (some input holds the innermost mode).
+bool is_row_reduction(einsummable_t const& e);
+
 // Compile `source` for `arch` (e.g. "gfx950"); returns the code object.  Throws km_error.
 std::vector<char> compile_hip_source(std::string const& source, std::string const& name,
                                      std::string const& arch);

@@ -1,5 +1,7 @@
 #include "exec_graph.h"
 
+#include "codegen.h"
+
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -495,11 +497,16 @@ bool apply_graph_t::absorb_into_readers(int u)
             std::optional<einsummable_t> m = merged(nu.e, e, k);
             if (!m) return false;
             // A sum (or product) keeps its bits only if its elements are added in the same
-            // order: the same vector width, over the same innermost extent.  min and max do
-            // not care.
+            // order: dealt to the lanes in the same way (row reductions deal 2- and 4-byte
+            // elements alike), over the same innermost extent.  min and max do not care.
             if (e.has_aggregation() && (e.castable.value() == castable_t::add ||
                                         e.castable.value() == castable_t::mul)) {
-                if (smallest_element(m.value()) != smallest_element(e) ||
+                bool const row = is_row_reduction(e);
+                bool const same_deal =
+                    row ? row_reduction_lane_elems(int(smallest_element(m.value()))) ==
+                              row_reduction_lane_elems(int(smallest_element(e)))
+                        : smallest_element(m.value()) == smallest_element(e);
+                if (row != is_row_reduction(m.value()) || !same_deal ||
                     m.value().join_shape.back() != e.join_shape.back()) {
                     return false;
                 }

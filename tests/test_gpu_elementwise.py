@@ -295,7 +295,7 @@ SPLIT_ROW_REDUCTIONS = [
     # a handful of very long rows: each row is cut into slices that run side by side
     (E([3, 131072], [[0, 1]], 1, "hole|f16@0", "+"), False),
     (E([1, 262144], [[0, 1]], 1, "hole|f32@0", "^"), True),
-    (E([5, 70000], [[0, 1]], 1, "hole|f32@0", "+"), False),                      # ragged last slice
+    (E([5, 140000], [[0, 1]], 1, "hole|f32@0", "+"), False),                     # ragged last slice
     (E([2, 64, 2048], [[0, 1, 2]], 1, "hole|f16@0", "v"), True),                 # two aggregated modes
     (E([2, 131072], [[0, 1], [0]], 1, "exp[+[hole|f16@0,*[constant{f16|-1},hole|f16@1]]]", "+"),
      False),                                                                      # ab,a->a

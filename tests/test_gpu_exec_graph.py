@@ -328,12 +328,13 @@ def test_optimized_layer_keeps_every_stored_bit(km, shape, n_streams):
     vals = make_inputs(g, 11)
     plain = ArenaRunner(km, g, n_streams)
     fused = ArenaRunner(km, g, n_streams, optimize=True)
-    # 13 formation copies and 14 elementwise nodes: in each of the two norms to_f32 (taken in
-    # by the square and by x * rstd), mean_eps, x_rstd and to_f16; scores+mask, to_f32 (taken
-    # in by the row max and by x - max), x - max, the division; silu; the first residual
-    # (taken in by the second norm and by the second residual).  The squares and exp stay:
-    # the sums behind them would add in another order over 2-byte than over 4-byte inputs.
-    assert fused.absorbed == 13 + 14, fused.absorbed
+    # 13 formation copies and 17 elementwise nodes: in each of the two norms to_f32 (taken in
+    # by the square and by x * rstd), the square (taken in by the row sum, which deals a row
+    # of 2-byte elements to the lanes as it deals one of 4-byte elements), mean_eps, x_rstd
+    # and to_f16; scores+mask, to_f32 (taken in by the row max and by x - max), x - max, exp
+    # (taken in by the row sum and by the division), the division; silu; the first residual
+    # (taken in by the second norm and by the second residual).
+    assert fused.absorbed == 13 + 17, fused.absorbed
     assert fused.graph.launches() == plain.graph.launches() - fused.absorbed
     for k, v in vals.items():
         plain.set_input(k, v)
@@ -342,8 +343,8 @@ def test_optimized_layer_keeps_every_stored_bit(km, shape, n_streams):
     fused.run()
     torch.cuda.synchronize()
     kept = surviving_buffers(fused)
-    assert g.output in kept and "sm.to_f16" in kept and "values.f" in kept and "sm.exp" in kept
-    for gone in ("scores", "sm.to_f32", "sm.sub", "sm.div", "silu", "residual1"):
+    assert g.output in kept and "sm.to_f16" in kept and "values.f" in kept and "sm.rowsum.f" in kept
+    for gone in ("scores", "sm.to_f32", "sm.sub", "sm.exp", "sm.div", "an.square", "silu", "residual1"):
         assert gone not in kept, gone
     for name in sorted(kept):
         a, b = plain.view(name), fused.view(name)

@@ -303,10 +303,22 @@ def test_exec_graph_optimize_brings_modes_to_their_common_pieces_or_declines():
     assert n == 1 and "[4,6]+ 0.1.->1 | to_f32[exp[hole|f32@0]]" in g.describe(b)
     up = E([24], [[0]], 1, "to_f32[hole|f16@0]")
     g, n, b = pair(up, rsum, [m(1, 96)])
-    assert n == 0                                   # 2-byte elements would be dealt to the lanes differently
-    rmax = E([4, 6], [[0, 1]], 1, "hole|f32@0", "^")
-    g, n, b = pair(up, rmax, [m(1, 96)])
+    assert n == 1                                   # rows of 2- and 4-byte elements are dealt to the lanes alike
+    assert "[4,6]+ 0.1.->1 | to_f32[to_f32[hole|f16@0]]" in g.describe(b)
+    down = E([24], [[0]], 1, "to_f32[hole|f64@0]")
+    g, n, b = pair(down, rsum, [m(1, 96)])
+    assert n == 1                                   # 8-byte input, 4-byte output: the smallest element stays 4
+    rsum64 = E([4, 3], [[0, 1]], 1, "hole|f64@0", "+")
+    up64 = E([12], [[0]], 1, "to_f64[hole|f32@0]")
+    g, n, b = pair(up64, rsum64, [m(1, 96)])
+    assert n == 0                                   # 8-byte rows read as 4-byte ones would change the order
+    rmax64 = E([4, 3], [[0, 1]], 1, "hole|f64@0", "^")
+    g, n, b = pair(up64, rmax64, [m(1, 96)])
     assert n == 1                                   # a maximum does not care
+    # a column sum walks each column in one thread: element sizes must agree as before
+    csum = E([6, 4], [[1, 0]], 1, "hole|f32@0", "+")
+    g, n, b = pair(up, csum, [m(1, 96)])
+    assert n == 0
 
 
 def test_exec_graph_optimize_leaves_what_it_cannot_prove():
