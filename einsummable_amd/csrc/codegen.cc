@@ -421,6 +421,15 @@ bool fits32(einsummable_t const& e)
     return true;
 }
 
+bool is_pow2(uint64_t v) { return v != 0 && (v & (v - 1)) == 0; }
+
+int log2_of(uint64_t v)
+{
+    int n = 0;
+    while ((1ull << n) < v) ++n;
+    return n;
+}
+
 int min_elem_size(einsummable_t const& e)
 {
     int m = int(dtype_size(e.out_dtype()));
@@ -456,8 +465,10 @@ cg_kernel_t gen_elementwise(einsummable_t const& e, int max_vec)
     // accesses 32 bytes apart, so every instruction touches half of each line: a 2^27-element
     // f16 -> f32 conversion ran at 3.1 TB/s that way and runs at 5.0 TB/s this way, the
     // reverse went from 4.4 to 5.0.
+    // (An input without the innermost mode is one scalar per vector and has no say in this.)
     int widest = int(dtype_size(e.out_dtype()));
     for (int k = 0; k != int(e.inns.size()); ++k) {
+        if (acc[k] == access_t::bcast) continue;
         widest = std::max(widest, int(dtype_size(e.inn_dtype(k))));
     }
     int const vcap = std::min(max_vec, 16 / widest);
@@ -500,7 +511,8 @@ cg_kernel_t gen_elementwise(einsummable_t const& e, int max_vec)
     g.k.vec = V;
 
     int p_nvec = g.param(n_vec);
-    int p_vpr = g.param(all_straight ? n_vec : inner / uint64_t(V));
+    uint64_t const vpr = all_straight ? n_vec : inner / uint64_t(V);
+    int p_vpr = g.param(vpr);
     std::vector<int> p_shape(R);
     for (int m = 0; m != R; ++m) p_shape[m] = g.param(L.shape[m]);
     std::vector<std::vector<int>> p_str(L.NI, std::vector<int>(R, -1));
@@ -509,6 +521,15 @@ cg_kernel_t gen_elementwise(einsummable_t const& e, int max_vec)
         for (int m = 0; m != R; ++m) {
             if (L.stride[k][m]) p_str[k][m] = g.param(L.stride[k][m]);
         }
+    }
+    // Every thread takes its vector's index apart.  A division by a run-time value is some
+    // twenty vector instructions, two of them as many as the arithmetic of eight elements of
+    // a softmax; by a power of two (the shift is a parameter, so all such shapes share the
+    // code) it is two.
+    int p_vpr_sh = (!all_straight && is_pow2(vpr)) ? g.param(uint64_t(log2_of(vpr))) : -1;
+    std::vector<int> p_shape_sh(R, -1);
+    for (int m = 1; m + 1 < R; ++m) {
+        if (!all_straight && is_pow2(L.shape[m])) p_shape_sh[m] = g.param(uint64_t(log2_of(L.shape[m])));
     }
 
     g.header();
@@ -531,13 +552,21 @@ cg_kernel_t gen_elementwise(einsummable_t const& e, int max_vec)
     s << "        live[u] = vid[u] < n_vec;\n";
     s << "        if (live[u]) {\n";
     if (!all_straight) {
+        // name = rem mod divisor; rem = rem / divisor
+        auto split = [&](std::string const& name, int p_div, int p_sh, const char* scale) {
+            if (p_sh >= 0) {
+                s << "            const idx_t " << name << " = (rem & (" << g.P(p_div) << " - 1))"
+                  << scale << ";\n";
+                s << "            rem >>= " << g.P(p_sh) << ";\n";
+            } else {
+                s << "            const idx_t " << name << " = (rem % " << g.P(p_div) << ")" << scale
+                  << ";\n";
+                s << "            rem /= " << g.P(p_div) << ";\n";
+            }
+        };
         s << "            idx_t rem = vid[u];\n";
-        s << "            const idx_t c = (rem % " << g.P(p_vpr) << ") * V;\n";
-        s << "            rem /= " << g.P(p_vpr) << ";\n";
-        for (int m = R - 2; m >= 1; --m) {
-            s << "            const idx_t d" << m << " = rem % " << g.P(p_shape[m]) << ";\n";
-            s << "            rem /= " << g.P(p_shape[m]) << ";\n";
-        }
+        split("c", p_vpr, p_vpr_sh, " * V");
+        for (int m = R - 2; m >= 1; --m) split("d" + std::to_string(m), p_shape[m], p_shape_sh[m], "");
         if (R >= 2) s << "            const idx_t d0 = rem;\n";
     }
     for (int k = 0; k != L.NI; ++k) {
@@ -552,7 +581,10 @@ cg_kernel_t gen_elementwise(einsummable_t const& e, int max_vec)
             if (p_str[k][m] >= 0) off += " + d" + std::to_string(m) + " * " + g.P(p_str[k][m]);
         }
         if (acc[k] == access_t::vec) {
-            s << "            r" << k << "[u] = ldv<" << NT_LD << ">(reinterpret_cast<const vec_t<" << T
+            // an input that lacks an outer mode is read again for every index of that mode:
+            // it is not streamed, whatever the node's size
+            int const nt = e.inn_nelem(k) == n_out ? NT_LD : 0;
+            s << "            r" << k << "[u] = ldv<" << nt << ">(reinterpret_cast<const vec_t<" << T
               << ", V>*>(a.in" << k << " + (" << off << " + c)));\n";
         } else if (acc[k] == access_t::bcast) {
             s << "            s" << k << "[u] = a.in" << k << "[" << off << "];\n";

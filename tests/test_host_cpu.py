@@ -116,9 +116,14 @@ def test_generated_kernels_compile_for_gfx950(e):
 
 
 def test_generated_source_is_deterministic_and_keyed_on_structure_not_shape():
-    a = ea.codegen_source(E([64, 256], [[0, 1], [0]], 2, GOLDEN["make"]["exp_sub|f16"]))
-    b = ea.codegen_source(E([640, 2560], [[0, 1], [0]], 2, GOLDEN["make"]["exp_sub|f16"]))
-    assert a == b  # extents travel as kernel arguments: one compile serves every shape
+    src = lambda shape: ea.codegen_source(E(shape, [[0, 1], [0]], 2, GOLDEN["make"]["exp_sub|f16"]))
+    # extents travel as kernel arguments: one compile serves every shape ...
+    assert src([640, 2560]) == src([300, 5120])
+    # ... of its kind: rows of a power-of-two number of vectors are taken apart with shifts
+    # (the shift is an argument too), the others with divisions
+    assert src([64, 256]) == src([640, 2048])
+    assert src([64, 256]) != src([640, 2560])
+    assert ">>=" in src([64, 256]) and ">>=" not in src([640, 2560])
 
 
 def test_aggregated_modes_are_numbered_by_first_appearance():
