@@ -1084,10 +1084,11 @@ cg_kernel_t gen_reduce_col(einsummable_t const& e, int max_vec)
     g.k.source = s.str();
     g.k.grid = std::max<uint64_t>(1, (n_vec + 255) / 256);
     g.k.block = 256;
-    g.k.out_inn_align.push_back(V * int(dtype_size(od)));
+    // (a vector wider than 16 bytes moves as 16-byte pieces: vec_t asks for no more)
+    g.k.out_inn_align.push_back(std::min(16, V * int(dtype_size(od))));
     for (int k = 0; k != L.NI; ++k) {
         bool wide = acc[k] == access_t::vec;
-        g.k.out_inn_align.push_back((wide ? V : 1) * int(dtype_size(e.inn_dtype(k))));
+        g.k.out_inn_align.push_back(std::min(16, (wide ? V : 1) * int(dtype_size(e.inn_dtype(k)))));
     }
     return std::move(g.k);
 }

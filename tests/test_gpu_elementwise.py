@@ -355,3 +355,60 @@ def test_large_transposed_input_is_staged_by_default(km):
     with pytest.raises(ea.KmError) as ei:
         km(e, stream_handle(), d.data_ptr(), [d.data_ptr(), d.data_ptr()])
     assert ei.value.code == -3
+
+
+# ------------------------------------------------------------------ buffers off the vector grid
+
+def run_at_offsets(km, e, xs, shift):
+    """Every buffer starts `shift` bytes behind a 256-byte boundary of one byte arena (the
+    engine hands out arena offsets aligned to 16 bytes only, memgraph.cc:58-62)."""
+    import torch
+
+    from helpers import stream_handle
+
+    od, dts = oracle.scalarop_info(e.join)
+    ws = km.build(e)
+    assert ws is not None
+    sizes = [x.nbytes for x in xs] + [e.out_nelem() * np.dtype(NP[od]).itemsize, max(ws, 1)]
+    offs, off = [], 0
+    for nb in sizes:
+        offs.append(off + shift)
+        off += (nb + shift + 255) // 256 * 256 + 256
+    arena = torch.zeros(off, dtype=torch.uint8, device="cuda")
+    for x, o in zip(xs, offs):
+        arena[o:o + x.nbytes] = torch.from_numpy(np.ascontiguousarray(x).view(np.uint8).reshape(-1)).cuda()
+    base = arena.data_ptr()
+    assert base % 256 == 0
+    km(e, stream_handle(), base + offs[len(xs)], [base + o for o in offs[:len(xs)]],
+       (base + offs[-1], ws) if ws else None)
+    torch.cuda.synchronize()
+    o = offs[len(xs)]
+    return arena[o:o + sizes[len(xs)]].cpu().numpy().view(NP[od])
+
+
+OFF_GRID = [
+    E([96, 512], [[0, 1]], 2, "to_f32[hole|f16@0]"),                                   # 8 f16 in, 32 bytes out
+    E([96, 512], [[0, 1], [0]], 2, "to_f16[*[hole|f32@0,hole|f32@1]]"),               # f32 row statistic
+    E([40, 2048], [[0, 1]], 1, "hole|f32@0", "+"),                                     # 32 bytes per lane and step
+    E([40, 2048], [[0, 1], [1]], 1, "to_f32[+[hole|f16@0,hole|f16@1]]", "+"),
+    E([3, 131072], [[0, 1]], 1, "hole|f32@0", "+"),                                    # slices and fold
+    E([512, 96], [[1, 0]], 1, "to_f32[hole|f16@0]", "+"),                              # column sum, f32 out
+    E([4, 64, 128], [[0, 1, 2], [1, 2], [0, 1]], 3, "exp[+[to_f32[+[hole|f16@0,hole|f16@1]],*[constant{f32|-1},hole|f32@2]]]"),
+]
+
+
+@pytest.mark.parametrize("case", range(len(OFF_GRID)))
+def test_generated_kernels_at_buffers_off_the_vector_grid(km, case):
+    """At 16 bytes behind a 256-byte boundary the vector kernels still apply (a 32-byte vector
+    moves as two 16-byte pieces) and a reduction adds in the same order as at the boundary;
+    at one element's size behind it the scalar variant runs: every result against the oracle."""
+    e = OFF_GRID[case]
+    od, dts = oracle.scalarop_info(e.join)
+    xs = inputs_for(e, rng(140 + case), 0.5)
+    want = oracle_einsummable(e, xs, oracle.WIDE)
+    at0 = run_at_offsets(km, e, xs, 0)
+    at16 = run_at_offsets(km, e, xs, 16)
+    assert_close(at0, want, od, what="on the grid")
+    assert_bits_equal(at16, at0, "16 bytes off: same kernel, same bits")
+    smallest = min([np.dtype(NP[d]).itemsize for d in dts] + [np.dtype(NP[od]).itemsize])
+    assert_close(run_at_offsets(km, e, xs, smallest), want, od, what="one element off")
