@@ -588,16 +588,47 @@ void apply_graph_t::finalize(int n_streams)
     // still the last node of its stream (the most recent such dependency): that needs no
     // wait at all.  Otherwise it takes the stream whose last node is oldest, and independent
     // branches spread over the pool.
+    // A node that moves 4 MiB or more fills the device by itself: beside another one it gains
+    // nothing, while every change of stream costs an event and a wait (some microseconds
+    // each; the LLaMA-7B layer's 28 launches took 1.58 ms spread over four streams and 1.44
+    // on one).  Such nodes all go to the first stream, in launch order; the pool is for the
+    // small ones.
+    auto wide = [](node_t const& x) {
+        if (x.kind == kind_t::dummy) return false;
+        uint64_t bytes = 0;
+        for (mem_t const& m : x.mems) bytes += m.size;
+        return bytes >= (4ull << 20);
+    };
     std::vector<int> last(size_t(n_streams), -1);
     std::vector<std::vector<int>> synced(size_t(n_streams), std::vector<int>(size_t(n_streams), -1));
     order_.resize(size_t(n));
     n_waits_ = 0;
+    // A dummy launches nothing: it takes no place on a stream and nobody waits for it; who
+    // depends on it depends on what it depends on.
+    std::vector<std::vector<int>> real_deps{size_t(n)};
     for (int v = 0; v != n; ++v) {
         node_t& nv = nodes_[v];
         nv.position = v;
         order_[size_t(v)] = v;
-        int best = -1;
+        std::vector<int>& deps = real_deps[size_t(v)];
         for (int d : nv.deps) {
+            if (nodes_[d].kind == kind_t::dummy) {
+                deps.insert(deps.end(), real_deps[size_t(d)].begin(), real_deps[size_t(d)].end());
+            } else {
+                deps.push_back(d);
+            }
+        }
+        std::sort(deps.begin(), deps.end(), [](int x, int y) { return x > y; });
+        deps.erase(std::unique(deps.begin(), deps.end()), deps.end());
+        nv.waits.clear();
+        if (nv.kind == kind_t::dummy) {
+            nv.stream = 0;
+            continue;
+        }
+        bool const first_stream = wide(nv);
+        int        best = first_stream ? 0 : -1;
+        for (int d : deps) {
+            if (first_stream) break;
             int s = nodes_[d].stream;
             if (last[size_t(s)] == d && (best < 0 || d > last[size_t(best)])) best = s;
         }
@@ -610,10 +641,7 @@ void apply_graph_t::finalize(int n_streams)
         nv.stream = best;
         last[size_t(best)] = v;
         // waits: a stream runs in order, so waiting for a node covers everything its stream
-        // launched before it
-        nv.waits.clear();
-        std::vector<int> deps = nv.deps;
-        std::sort(deps.begin(), deps.end(), [](int x, int y) { return x > y; });
+        // launched before it (deps: latest first)
         for (int d : deps) {
             int sd = nodes_[d].stream;
             if (sd == best) continue;
@@ -623,6 +651,16 @@ void apply_graph_t::finalize(int n_streams)
             nodes_[d].record = true;
             ++n_waits_;
         }
+    }
+
+    // A pool stream is forked off the caller's stream only if it holds a node, and joined at
+    // the end only if its last node is not already waited for by a node of the first stream:
+    // each fork and join is an event and a wait that the first stream pays for.
+    stream_used_.assign(size_t(n_streams), 0);
+    stream_joins_.assign(size_t(n_streams), 0);
+    for (int s = 1; s != n_streams; ++s) {
+        stream_used_[size_t(s)] = last[size_t(s)] >= 0;
+        stream_joins_[size_t(s)] = last[size_t(s)] >= 0 && synced[0][size_t(s)] < last[size_t(s)];
     }
 
     // Runs of grouped touches.  The reference's engine launches the touches of a group one
@@ -828,8 +866,11 @@ void apply_graph_t::run(hipStream_t main, void* arena_) const
                            "apply graph: a run on more than one stream cannot be captured into "
                            "a HIP graph; finalize the graph on one stream for that");
         }
-        check(hipEventRecord(fork_, main), "hipEventRecord");
+        bool forked = false;
         for (size_t s = 1; s != ns; ++s) {
+            if (!stream_used_[s]) continue;
+            if (!forked) check(hipEventRecord(fork_, main), "hipEventRecord");
+            forked = true;
             check(hipStreamWaitEvent(streams_[s], fork_, 0), "hipStreamWaitEvent");
         }
     }
@@ -868,6 +909,7 @@ void apply_graph_t::run(hipStream_t main, void* arena_) const
         }
     }
     for (size_t s = 1; s != ns; ++s) {
+        if (!stream_joins_[s]) continue;
         check(hipEventRecord(joins_[s - 1], streams_[s]), "hipEventRecord");
         check(hipStreamWaitEvent(main, joins_[s - 1], 0), "hipStreamWaitEvent");
     }

@@ -192,6 +192,9 @@ private:
     slot_t const* slot(int storage_id) const;
     hipEvent_t               fork_ = nullptr;
     std::vector<hipEvent_t>  joins_;
+    // per stream: holds a node at all; its last node is not yet waited for by a node of the
+    // first stream (only then run() ends with a join of that stream)
+    std::vector<char>        stream_used_, stream_joins_;
     int                      n_waits_ = 0;
     bool                     finalized_ = false;
 };
