@@ -192,6 +192,34 @@ def test_exec_graph_memory_dependencies_and_stream_placement():
     assert g.cross_stream_waits() >= 2
 
 
+def test_exec_graph_placement_keeps_large_nodes_together_and_looks_through_dummies():
+    import einsummable_amd as ea
+
+    E = ea.Einsummable
+    small = E([1024], [[0]], 1, "hole|f32@0")                       # 4 KiB in, 4 KiB out
+    large = E([1 << 20], [[0]], 1, "hole|f32@0")                    # 4 MiB in, 4 MiB out
+    S, L = 4096, 4 << 20
+    g = ea.ApplyGraph(None)
+    a = g.add_einsummable(large, [(0 * L, L), (1 * L, L)])
+    b = g.add_einsummable(large, [(2 * L, L), (3 * L, L)])          # independent of a
+    base = 4 * L
+    c = g.add_einsummable(small, [(base + 0 * S, S), (base + 1 * S, S)])
+    d = g.add_einsummable(small, [(base + 2 * S, S), (base + 3 * S, S)])
+    gone = g.add_dummy((base + 1 * S, S), [c])                      # c's input is released
+    e = g.add_einsummable(small, [(base + 4 * S, S), (base + 5 * S, S)], [gone])   # listed behind the dummy only
+    f = g.add_einsummable(large, [(1 * L, L), (0 * L, L)])          # reads a's output
+    g.add_memory_dependencies()
+    g.finalize(4)
+    stream = lambda i: g.node_info(i)[1]
+    # nodes that fill the device go to the first stream, whatever they depend on
+    assert stream(a) == stream(b) == stream(f) == 0
+    # small independent nodes spread over the pool
+    assert stream(c) != 0 and stream(d) != 0 and stream(c) != stream(d)
+    # e depends on the dummy, i.e. on c, which is still the last node of its stream: no wait
+    assert g.node_info(e)[2] == [gone] and stream(e) == stream(c)
+    assert g.cross_stream_waits() == 0
+
+
 def test_exec_graph_optimize_absorbs_copies_and_single_reader_elementwise():
     import einsummable_amd as ea
 
