@@ -750,9 +750,9 @@ def run_c5(km, steps, warmup):
         par = ArenaRunner(km, g, ns, optimize=optimize)
         for name, t in state.items():
             par.view(name).copy_(t)
-        for _ in range(max(warmup, 2)):
-            par.run()
-        torch.cuda.synchronize()
+        # (building a runner leaves the device idle for a while: warm() runs until the clocks
+        # have settled again, or a variant is charged for the one built before it)
+        warm(par.run, max(warmup, 2))
         t0 = time.perf_counter()
         for _ in range(steps):
             par.run()
