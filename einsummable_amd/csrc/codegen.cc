@@ -481,7 +481,32 @@ cg_kernel_t gen_elementwise(einsummable_t const& e, int max_vec)
     } else {
         V = pow2_divisor(inner, vcap);
     }
-    int const U = env_int("ES_KM_EW_UNROLL", 1);
+    int U = env_int("ES_KM_EW_UNROLL", 1);
+    // A large permutation that keeps the innermost mode moves rows: the workgroup's 256
+    // consecutive output vectors are whole rows that lie next to each other in the output,
+    // while in the input each stands alone (C3a: 256-byte rows, 8 KiB apart).  When the mode
+    // that follows the innermost one in the INPUT has an even extent, a thread takes the same
+    // vector of two neighbours along it: the reads then come in runs of two rows as well
+    // (abcd->acbd over 32 x 2048 x 32 x 128 f16, stand-alone: 0.77 -> 0.80 of HBM; more
+    // than two neighbours per thread gain no more).
+    int      pair_mode = -1;
+    uint64_t pair_inner = 0;  // output vectors per index of that mode
+    int const pair_rule = env_int("ES_KM_EW_PAIR", 1);  // tuning and tests: 0 never, 2 at any size
+    if (U == 1 && !all_straight && L.NI == 1 && acc[0] == access_t::vec && R >= 3 &&
+        (pair_rule == 2 || (pair_rule == 1 && n_out * dtype_size(e.out_dtype()) >= (32ull << 20)))) {
+        int next = -1;
+        for (int m = 0; m + 1 < R; ++m) {
+            if (L.stride[0][m] == 0) continue;
+            if (next < 0 || L.stride[0][m] < L.stride[0][next]) next = m;
+        }
+        if (next >= 0 && next != R - 2 && L.shape[next] % 2 == 0) {
+            pair_mode = next;
+            g.k.row_pairs = true;
+            pair_inner = inner / uint64_t(V);
+            for (int m = next + 1; m + 1 < R; ++m) pair_inner *= L.shape[m];
+            U = 2;
+        }
+    }
     // Outputs far larger than the last-level cache are written non-temporally: they would
     // only evict inputs that later nodes still read (measured on 8192^2 f16: +20% on the
     // producing kernel).  ES_KM_EW_NT: 1 loads and stores, 2 loads only, 3 stores only, 4 none.
@@ -526,6 +551,8 @@ cg_kernel_t gen_elementwise(einsummable_t const& e, int max_vec)
     // twenty vector instructions, two of them as many as the arithmetic of eight elements of
     // a softmax; by a power of two (the shift is a parameter, so all such shapes share the
     // code) it is two.
+    int p_pair = pair_mode >= 0 ? g.param(pair_inner) : -1;
+    int p_pair_sh = (pair_mode >= 0 && is_pow2(pair_inner)) ? g.param(uint64_t(log2_of(pair_inner))) : -1;
     int p_vpr_sh = (!all_straight && is_pow2(vpr)) ? g.param(uint64_t(log2_of(vpr))) : -1;
     std::vector<int> p_shape_sh(R, -1);
     for (int m = 1; m + 1 < R; ++m) {
@@ -547,9 +574,24 @@ cg_kernel_t gen_elementwise(einsummable_t const& e, int max_vec)
         }
     }
     s << "    idx_t vid[U];\n    bool live[U];\n";
+    if (pair_mode >= 0) {
+        // work item w stands for the vectors (.., 2 q, ..) and (.., 2 q + 1, ..) of the paired
+        // mode: with t = w / inner (all outer indices and q), the first is w + t * inner
+        s << "    const idx_t w = ((idx_t)blockIdx.y * gridDim.x + blockIdx.x) * 256 + threadIdx.x;\n";
+        if (p_pair_sh >= 0) {
+            s << "    const idx_t wt = w >> " << g.P(p_pair_sh) << ";\n";
+        } else {
+            s << "    const idx_t wt = w / " << g.P(p_pair) << ";\n";
+        }
+    }
     s << "#pragma unroll\n    for (int u = 0; u != U; ++u) {\n";
-    s << "        vid[u] = (((idx_t)blockIdx.y * gridDim.x + blockIdx.x) * U + u) * 256 + threadIdx.x;\n";
-    s << "        live[u] = vid[u] < n_vec;\n";
+    if (pair_mode >= 0) {
+        s << "        vid[u] = w + (wt + (idx_t)u) * " << g.P(p_pair) << ";\n";
+        s << "        live[u] = w < n_vec / 2;\n";
+    } else {
+        s << "        vid[u] = (((idx_t)blockIdx.y * gridDim.x + blockIdx.x) * U + u) * 256 + threadIdx.x;\n";
+        s << "        live[u] = vid[u] < n_vec;\n";
+    }
     s << "        if (live[u]) {\n";
     if (!all_straight) {
         // name = rem mod divisor; rem = rem / divisor
@@ -1464,6 +1506,7 @@ std::shared_ptr<plan_t> plan_codegen(einsummable_t const& e, int device)
             break;
     }
     p->description += " vec=" + std::to_string(p->wide.k.vec);
+    if (p->wide.k.row_pairs) p->description += " row_pairs";
     if (p->wide.k.splits > 1) p->description += " splits=" + std::to_string(p->wide.k.splits);
     p->workspace_bytes = std::max(p->wide.k.ws_bytes, p->narrow.k.ws_bytes);
     return p;

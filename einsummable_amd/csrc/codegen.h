@@ -25,6 +25,7 @@ struct cg_kernel_t {
     int         n_inns = 0;
     bool        idx64 = false;
     int         vec = 1;                 // elements per vector access
+    bool        row_pairs = false;       // elementwise: a thread moves two neighbouring input rows
     unsigned    block = 256;
     uint64_t    grid = 0;
     std::vector<uint64_t> params;        // written after the pointers as idx_t values

@@ -139,3 +139,31 @@ def test_long_tiles_forced_on_small_ragged_transposes(monkeypatch, dt, npdt, til
         assert ("xcd_runs" in d) == (order != 0) and ("out_first" in d) == (order == 2), d
         want = np.ascontiguousarray(np.transpose(x, perm)).reshape(-1)
         assert_bits_equal(got, want, "permute %s %s" % (shape, perm))
+
+
+@pytest.mark.parametrize("dt,npdt", [("f16", np.float16), ("f32", np.float32), ("c64", np.complex64)])
+def test_row_permutes_in_pairs_of_input_neighbours(monkeypatch, dt, npdt):
+    """A permutation that keeps the innermost mode is a copy of rows; for large ones a thread
+    moves the same vector of two rows that are neighbours in the input.  Forced here at small
+    sizes: inner extents that are and are not powers of two (shift and division), a last
+    workgroup that is not full, and shapes whose mode next to the innermost one in the input
+    has an odd extent, which keep the plain mapping."""
+    monkeypatch.setenv("ES_KM_EW_PAIR", "2")
+    km = ea.KernelManager(0)
+    r = rng(57)
+    v = 16 // np.dtype(npdt).itemsize
+    cases = [((3, 64, 4, 8 * v), (0, 2, 1, 3), True),       # abcd->acbd, inner count a power of two
+             ((2, 6, 10, 3 * v), (0, 2, 1, 3), True),       # 6 x 3 vectors under the pair: division
+             ((5, 7, 2, v), (2, 0, 1, 3), True),            # the paired mode is outermost in the output
+             ((4, 3, 6, 5 * v), (1, 2, 0, 3), True),
+             ((3, 8, 5, 4 * v), (0, 2, 1, 3), False),       # 5 rows next to each other: odd
+             ((6, 4, 2 * v), (1, 0, 2), True),
+             ((2, 3, 4, 2 * v), (1, 0, 2, 3), False)]       # c and d merge; next to them in the input: 3 rows
+    for shape, perm, paired in cases:
+        x = normal(r, int(np.prod(shape)), npdt).reshape(shape)
+        e = permute_einsummable(shape, perm, dt)
+        got = run_einsummable(km, e, [x])
+        d = km.describe(e)
+        assert d.startswith("elementwise") and ("row_pairs" in d) == paired, (shape, perm, d)
+        want = np.ascontiguousarray(np.transpose(x, perm)).reshape(-1)
+        assert_bits_equal(got, want, "permute %s %s" % (shape, perm))
