@@ -33,9 +33,9 @@ HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E
 PEAK_TFLOPS = {"f16": 2500.0, "f32": 157.3, "f64": 78.6, "c64": 157.3}
 
 # HBM bytes per launch of the dominant kernel (C2 node (i)) from two rocprofv3 --pmc runs:
-# FETCH_SIZE 131084.8 KiB x 1.9999 + WRITE_SIZE 131074.1 KiB x 1.0000, the factors being what
+# FETCH_SIZE 131084.4 KiB x 1.9999 + WRITE_SIZE 131075.3 KiB x 1.0000, the factors being what
 # the same counters read for a 512 MiB copy of known size.
-DOMINANT_KERNEL_TRAFFIC_BYTES = 402662083
+DOMINANT_KERNEL_TRAFFIC_BYTES = 402662523
 
 RELU_MUL = "*[ite_>=[constant{f16|0},hole|f16@0,constant{f16|0},hole|f16@0],hole|f16@1]"
 EXP_SUB = "exp[+[hole|f16@0,*[constant{f16|-1},hole|f16@1]]]"
