@@ -744,6 +744,15 @@ int es_km_graph_add_dummy(es_km_graph_t* g, uint64_t offset, uint64_t size, cons
     });
 }
 
+int es_km_graph_add_placeholder(es_km_graph_t* g, uint64_t offset, uint64_t size, const int* deps,
+                                int n_deps)
+{
+    return guarded(g ? g->owner : nullptr, [&]() -> int {
+        if (!g) throw es::ir_error("null graph");
+        return g->graph->add_dummy(es::mem_t{offset, size}, make_deps(deps, n_deps), false);
+    });
+}
+
 int es_km_graph_add_evict(es_km_graph_t* g, uint64_t offset, uint64_t size, int storage_id,
                           const int* deps, int n_deps)
 {

@@ -146,11 +146,12 @@ int apply_graph_t::add_copy(mem_t dst, mem_t src, std::vector<int> const& deps)
     return insert(std::move(n), deps);
 }
 
-int apply_graph_t::add_dummy(mem_t range, std::vector<int> const& deps)
+int apply_graph_t::add_dummy(mem_t range, std::vector<int> const& deps, bool is_del)
 {
     node_t n;
     n.kind = kind_t::dummy;
     n.mems = {range};
+    n.is_del = is_del && range.size != 0;
     return insert(std::move(n), deps);
 }
 
@@ -435,7 +436,7 @@ bool apply_graph_t::absorb_into_readers(int u)
     for (int w = u + 1; w < n && !deleted; ++w) {
         node_t const& nw = nodes_[size_t(w)];
         if (nw.kind == kind_t::dummy) {
-            deleted = !readers.empty() && covers(nw.mems[0], S) &&
+            deleted = nw.is_del && !readers.empty() && covers(nw.mems[0], S) &&
                       std::binary_search(nw.deps.begin(), nw.deps.end(), readers.back());
             continue;
         }
@@ -524,6 +525,22 @@ bool apply_graph_t::absorb_into_readers(int u)
         }
     }
 
+    // Who waits for u: u itself and every dummy that, through dummies, depends on it (the
+    // del of one of u's inputs stands right behind u, before the readers).  A node that
+    // depends on any of them was promised that u is done with its inputs; those are now read
+    // by the readers.
+    std::vector<char> waits_for_u(size_t(n), 0);
+    waits_for_u[size_t(u)] = 1;
+    for (int w = u + 1; w < n; ++w) {
+        node_t const& nw = nodes_[size_t(w)];
+        if (nw.kind != kind_t::dummy) continue;
+        for (int d : nw.deps) {
+            if (waits_for_u[size_t(d)]) {
+                waits_for_u[size_t(w)] = 1;
+                break;
+            }
+        }
+    }
     for (size_t r = 0; r != readers.size(); ++r) {
         int const v = readers[r];
         node_t&   nv = nodes_[size_t(v)];
@@ -547,13 +564,16 @@ bool apply_graph_t::absorb_into_readers(int u)
         for (int w = v + 1; w < n; ++w) {
             if (std::find(readers.begin(), readers.end(), w) != readers.end()) continue;
             std::vector<int>& d = nodes_[size_t(w)].deps;
-            if (std::binary_search(d.begin(), d.end(), u) && !std::binary_search(d.begin(), d.end(), v)) {
+            bool const promised = std::any_of(d.begin(), d.end(),
+                                              [&](int x) { return waits_for_u[size_t(x)] != 0; });
+            if (promised && !std::binary_search(d.begin(), d.end(), v)) {
                 d.insert(std::upper_bound(d.begin(), d.end(), v), v);
             }
         }
     }
     nu.kind = kind_t::dummy;
     nu.mems = {S};
+    nu.is_del = false;
     return true;
 }
 

@@ -60,7 +60,10 @@ public:
     // of inputmem / inputsto / partialize / alloc / del nodes and of nodes that live on
     // another device (gpu/exec_graph.cc:94-97).  `range` is kept for inspection only and
     // takes no part in add_memory_dependencies.
-    int add_dummy(mem_t range, std::vector<int> const& deps);
+    // `is_del`: the dummy stands for the deletion of `range` (what a caller's own dels and the
+    // memgraph's del nodes are); the other ranged dummies (inputmem, alloc, partialize) only
+    // name a range and never let optimize() drop what is stored there
+    int add_dummy(mem_t range, std::vector<int> const& deps, bool is_del = true);
     // Host storage (gpu_evict_t / gpu_load_t, gpu/exec_graph.cc:466-577; the reference's
     // storage is host memory too, src/engine/gpu/storage_manager.h).  evict copies an arena
     // range into the storage slot `storage_id`, load copies the slot back.  Slots are pinned
@@ -154,6 +157,7 @@ private:
         uint64_t           bits0 = 0, bits1 = 0, n0 = 0, n1 = 0;
         int64_t            start = 0;
         int                storage_id = -1;
+        bool               is_del = false;  // dummies: the range is deleted here
         std::vector<mem_t> mems;
         std::vector<int>   deps;
         std::vector<int>   waits;  // dependencies on other streams, reduced

@@ -557,8 +557,10 @@ void memgraph_t::populate(apply_graph_t& g, int loc,
             case mg_kind::inputmem:
             case mg_kind::partialize:
             case mg_kind::alloc:
+                g.add_dummy(range, n.inns, false);
+                break;
             case mg_kind::del:
-                g.add_dummy(range, n.inns);
+                g.add_dummy(range, n.inns, true);
                 break;
             case mg_kind::inputsto:
                 break;

@@ -55,6 +55,7 @@ EXPORTS = [
     "es_km_stream_pool_try_acquire",
     "es_km_stream_pool_release",
     "es_km_graph_add_dummy",
+    "es_km_graph_add_placeholder",
     "es_km_graph_add_evict",
     "es_km_graph_add_load",
     "es_km_graph_declare_storage",
@@ -220,6 +221,7 @@ def load_library():
     lib.es_km_stream_pool_try_acquire.argtypes = [V]
     lib.es_km_stream_pool_release.argtypes = [V, V]
     lib.es_km_graph_add_dummy.argtypes = [V, U64, U64, V, I]
+    lib.es_km_graph_add_placeholder.argtypes = [V, U64, U64, V, I]
     lib.es_km_graph_add_evict.argtypes = [V, U64, U64, I, V, I]
     lib.es_km_graph_add_load.argtypes = [V, I, U64, U64, V, I]
     lib.es_km_graph_declare_storage.argtypes = [V, I, U64]
@@ -653,10 +655,12 @@ class ApplyGraph:
             self._g, int(i), stream, arena, ws_ptr, ws_size, int(first_in_group),
             ctypes.cast(callback, ctypes.c_void_p) if callback is not None else None, user))
 
-    def add_dummy(self, mem=(0, 0), deps=None):
+    def add_dummy(self, mem=(0, 0), deps=None, is_del=True):
+        """A node that launches nothing.  With a range it stands for the range's del, unless
+        is_del is False (a placeholder: the range of an input or an alloc)."""
         d, nd = self._deps(deps)
-        return self._check(self._lib.es_km_graph_add_dummy(self._g, int(mem[0]), int(mem[1]),
-                                                           d, nd))
+        f = self._lib.es_km_graph_add_dummy if is_del else self._lib.es_km_graph_add_placeholder
+        return self._check(f(self._g, int(mem[0]), int(mem[1]), d, nd))
 
     def add_evict(self, mem, storage_id, deps=None):
         d, nd = self._deps(deps)

@@ -304,6 +304,13 @@ int   es_km_stream_pool_release(es_km_stream_pool_t* p, void* stream);
  * The range is kept for inspection and takes no part in add_memory_dependencies. */
 int es_km_graph_add_dummy(es_km_graph_t* g, uint64_t offset, uint64_t size, const int* deps,
                           int n_deps);
+/* add_dummy with a non-empty range is how a caller spells a del (memgraph.h: del_t): it is
+ * what lets es_km_graph_optimize drop the range.  add_placeholder names a range without
+ * deleting it -- what the memgraph loader makes of inputmem / alloc / partialize nodes, whose
+ * ranges hold or will hold data (gpu/exec_graph.cc:94-97 makes dummy_t of all of them alike;
+ * only this library's optimize() needs to tell them apart). */
+int es_km_graph_add_placeholder(es_km_graph_t* g, uint64_t offset, uint64_t size, const int* deps,
+                                int n_deps);
 
 /* Host storage: gpu_evict_t::launch / gpu_load_t::launch, src/engine/gpu/exec_graph.cc:482-577
  * (memgraph_t::evict_t / load_t, src/einsummable/memgraph.h:306-325).  evict copies an arena

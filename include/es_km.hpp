@@ -295,11 +295,13 @@ public:
         return id(es_km_graph_add_copy(g_, dst.offset, src.offset, dst.size, inns.data(),
                                        int(inns.size())));
     }
-    // dummy_t: launches nothing, only orders (inputmem / partialize / alloc / del nodes)
-    int insert_dummy(mem_t range = {0, 0}, std::vector<int> const& inns = {})
+    // dummy_t: launches nothing, only orders (inputmem / partialize / alloc / del nodes).
+    // With a range it stands for the range's del unless is_del is false (the range of an
+    // input or an alloc: optimize() never drops what is stored there).
+    int insert_dummy(mem_t range = {0, 0}, std::vector<int> const& inns = {}, bool is_del = true)
     {
-        return id(es_km_graph_add_dummy(g_, range.offset, range.size, inns.data(),
-                                        int(inns.size())));
+        auto const add = is_del ? es_km_graph_add_dummy : es_km_graph_add_placeholder;
+        return id(add(g_, range.offset, range.size, inns.data(), int(inns.size())));
     }
     // gpu_evict_t / gpu_load_t: arena range <-> host storage slot
     int insert_evict(mem_t src, int storage_id, std::vector<int> const& inns = {})

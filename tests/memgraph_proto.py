@@ -254,3 +254,140 @@ def describe(mg):
                          _list(n["inns"]),
                          ",".join("%d:%d" % (o, s) for o, s in mems), tail))
     return "\n".join(lines) + "\n"
+
+
+def layer_node(n, deps, out, inns):
+    """One node of einsummable_amd.llama_layer.LayerGraph (einsummable, touch or the mask's
+    lowertri fill) as a memgraph node dict over the given ranges."""
+    import numpy as np
+
+    import einsummable_amd as ea
+
+    if n["kind"] == "einsummable":
+        e = n["e"]
+        return node("apply", deps, loc=0, mems=[out] + inns, group=-1,
+                    einsummable=dict(join_shape=e.join_shape, inns=e.inns, out_rank=e.out_rank,
+                                     join=e.join, castable=e.castable or ""))
+    if n["kind"] == "touch":
+        t = n["t"]
+        return node("apply", deps, loc=0, mems=[out] + inns, group=-1,
+                    touch=dict(selection=t.selection, castable=t.castable or "",
+                               dtype=["f16", "f32", "f64", "c64"][t.dtype]))
+    assert n["dtype"] == ea.F16 and n["lower"] == 0.0 and n["upper"] == -np.inf
+    # written as the reference's to_proto writes it; its reader exchanges the two (the mask
+    # is square here, so the exchange does not show)
+    assert n["nrow"] == n["ncol"]
+    return node("constant", deps, loc=0, offset=out[0],
+                fill=dict(lower="f16|0", upper="f16|NINF", nrow=n["nrow"], ncol=n["ncol"],
+                          start=n["start"]))
+
+
+def layer_memgraph_reusing(graph, align=256):
+    """The decoder layer as the reference's memgraph compiler lays it out: an inputmem per
+    layer input; every other buffer is allocated right before its first writer, deleted right
+    behind its last user (the del depends on every user) and its range handed to later allocs
+    (first fit), which depend on the dels that freed what they cover.  Apply nodes depend on
+    the producers of what they read and on the alloc of what they write -- nothing is derived
+    from the ranges.  Returns (memgraph dict, {input name: range}, output range, arena bytes)."""
+    def names_in(n):
+        if n["kind"] == "einsummable":
+            return list(n["inns"])
+        return [n["inn"]] if n["kind"] == "touch" else []
+
+    written = {n["out"] for n in graph.nodes}
+    last_use = {}
+    for i, n in enumerate(graph.nodes):
+        for b in names_in(n) + [n["out"]]:
+            last_use[b] = i
+    nodes, where, top = [], {}, 0
+    users = {}        # buffer -> ids of the nodes that read or wrote it
+    producer = {}     # buffer -> id of the inputmem / last writer
+    input_ranges = {}
+    for name, nbytes in graph.buffers.items():
+        if name in written:
+            continue
+        where[name] = (top, nbytes)
+        input_ranges[name] = where[name]
+        producer[name] = len(nodes)
+        nodes.append(node("inputmem", loc=0, offset=top, size=nbytes))
+        top += (nbytes + align - 1) // align * align
+    free = []         # (offset, size, id of the del that freed it)
+    for i, n in enumerate(graph.nodes):
+        out = n["out"]
+        deps = set()
+        if out not in where:
+            nbytes = graph.buffers[out]
+            need = (nbytes + align - 1) // align * align
+            hit = next((f for f in free if f[1] >= need), None)
+            if hit is None:
+                off, freed_by = top, []
+                top += need
+            else:
+                free.remove(hit)
+                off, freed_by = hit[0], [hit[2]]
+                if hit[1] > need:
+                    free.append((hit[0] + need, hit[1] - need, hit[2]))
+                    free.sort()
+            where[out] = (off, nbytes)
+            deps.add(len(nodes))
+            nodes.append(node("alloc", freed_by, loc=0, offset=off, size=nbytes))
+        else:
+            deps.update(users.get(out, ()))
+        ins = names_in(n)
+        for b in ins:
+            deps.add(producer[b])
+        me = len(nodes)
+        nodes.append(layer_node(n, deps, where[out], [where[b] for b in ins]))
+        producer[out] = me
+        for b in ins + [out]:
+            users.setdefault(b, set()).add(me)
+        for b in dict.fromkeys(ins + [out]):
+            if last_use[b] == i and b in written and b != graph.output:
+                off, nbytes = where[b]
+                d = len(nodes)
+                nodes.append(node("del", users[b], loc=0, offset=off, size=nbytes))
+                free.append((off, (nbytes + align - 1) // align * align, d))
+                free.sort()
+    mg = dict(num_compute_locs=1, num_storage_locs=0, nodes=nodes)
+    return mg, input_ranges, where[graph.output], top
+
+
+def unordered_conflicts(g):
+    """Pairs (i, j), i < j, of launching nodes of an einsummable_amd.ApplyGraph where j writes
+    what i reads or writes, or reads what i writes, without depending on i (through any
+    chain of dependencies)."""
+    n = g.num_nodes()
+    kinds, mems, deps = [], [], []
+    for i in range(n):
+        k, m = g.node_mems(i)
+        kinds.append(k)
+        mems.append(m)
+        deps.append(g.node_info(i)[2])
+    reach = []
+    for i in range(n):
+        r = set()
+        for d in deps[i]:
+            r.add(d)
+            r |= reach[d]
+        reach.append(r)
+
+    def overlap(x, y):
+        return x[1] and y[1] and x[0] < y[0] + y[1] and y[0] < x[0] + x[1]
+
+    def split(i):
+        if kinds[i] == "dummy":
+            return [], []
+        if kinds[i] == "evict":
+            return [], mems[i]
+        return mems[i][:1], mems[i][1:]
+
+    bad = []
+    for j in range(n):
+        wj, rj = split(j)
+        for i in range(j):
+            wi, ri = split(i)
+            clash = any(overlap(a, b) for a in wj for b in wi + ri) or \
+                any(overlap(a, b) for a in rj for b in wi)
+            if clash and i not in reach[j]:
+                bad.append((i, j))
+    return bad

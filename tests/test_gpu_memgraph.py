@@ -101,24 +101,7 @@ def layer_memgraph(graph, ranges, with_dels=False):
         for i, o, rs in history:
             if overlap(o, out) or any(overlap(o, x) for x in inns) or any(overlap(out, x) for x in rs):
                 deps.add(i)
-        if n["kind"] == "einsummable":
-            e = n["e"]
-            m = node("apply", deps, loc=0, mems=[out] + inns, group=-1,
-                     einsummable=dict(join_shape=e.join_shape, inns=e.inns, out_rank=e.out_rank,
-                                      join=e.join, castable=e.castable or ""))
-        elif n["kind"] == "touch":
-            t = n["t"]
-            m = node("apply", deps, loc=0, mems=[out] + inns, group=-1,
-                     touch=dict(selection=t.selection, castable=t.castable or "",
-                                dtype=["f16", "f32", "f64", "c64"][t.dtype]))
-        else:
-            assert n["dtype"] == ea.F16 and n["lower"] == 0.0 and n["upper"] == -np.inf
-            # written as the reference's to_proto writes it; its reader exchanges the two
-            # (the mask is square here, so the exchange does not show)
-            assert n["nrow"] == n["ncol"]
-            m = node("constant", deps, loc=0, offset=out[0],
-                     fill=dict(lower="f16|0", upper="f16|NINF", nrow=n["nrow"], ncol=n["ncol"],
-                               start=n["start"]))
+        m = mp.layer_node(n, deps, out, inns)
         history.append((len(nodes), out, inns))
         nodes.append(m)
     if with_dels:
@@ -199,3 +182,33 @@ def test_storage_slot_errors(km):
         g.storage_read(4, 8)
     with pytest.raises(ea.KmError, match="too small"):
         g.storage_write(3, b"\0" * 65)
+
+
+@pytest.mark.parametrize("n_streams", [1, 4])
+def test_llama_layer_with_reused_ranges_optimized(km, n_streams):
+    """The reference's layout: dels right behind the last user, freed ranges handed to later
+    allocs, ordering carried by the memgraph's edges alone.  Optimised and spread over
+    streams, the layer's output holds the bytes of the node-by-node run."""
+    import torch
+
+    lg = LayerGraph(dim=256, n_heads=4, ffn=688, seq=128)
+    vals = make_inputs(lg, 7)
+    seq = DeviceRunner(km, lg)
+    mg, input_ranges, out_range, top = mp.layer_memgraph_reusing(lg)
+    assert top < sum((b + 255) // 256 * 256 for b in lg.buffers.values())   # ranges were reused
+    g = ea.ApplyGraph(km)
+    g.load_memgraph(mp.to_wire(mg))
+    assert g.optimize() > 10           # fewer than with private ranges: a reused range is often still read
+    assert mp.unordered_conflicts(g) == []
+    g.finalize(n_streams)
+    arena = torch.zeros(max(g.arena_bytes(), top), dtype=torch.uint8, device="cuda")
+    for k, v in vals.items():
+        seq.set_input(k, v)
+        o, nb = input_ranges[k]
+        arena[o:o + nb] = torch.from_numpy(np.ascontiguousarray(v).view(np.uint8).reshape(-1)).cuda()
+    seq.run()
+    for _ in range(3):
+        g.run(stream_handle(), arena.data_ptr())
+    torch.cuda.synchronize()
+    o, nb = out_range
+    assert np.array_equal(seq.get(lg.output, np.uint8), arena[o:o + nb].cpu().numpy())

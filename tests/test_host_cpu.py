@@ -458,3 +458,74 @@ def test_assert_close_does_not_accept_a_finite_value_for_an_infinite_one():
                       ([1.0, np.nan], [1.0, 3.0])):
         with pytest.raises(AssertionError):
             assert_close(np.array(got), np.array(want), ea.F32, what="must fail")
+
+
+def test_exec_graph_optimize_keeps_write_after_read_through_dels():
+    """The reference's memgraphs put each del right behind its last user and let a later node
+    reuse the range, waiting only for that del.  When the user is absorbed into its reader,
+    the reader reads the range instead, and the node that reuses it must wait for the reader."""
+    import einsummable_amd as ea
+
+    E = ea.Einsummable
+    exp = E([1024], [[0]], 1, "exp[hole|f32@0]")
+    sq = E([1024], [[0]], 1, "power{2}[hole|f32@0]")
+    m = lambda slot: (slot * 4096, 4096)
+    X, S, T, Y = 0, 1, 2, 3
+
+    g = ea.ApplyGraph(None)
+    n0 = g.add_einsummable(exp, [m(S), m(X)])          # exp X -> S
+    n1 = g.add_dummy(m(X), [n0])                       # del X, right behind its only user
+    n2 = g.add_einsummable(sq, [m(T), m(S)], [n0])     # sq S -> T
+    n3 = g.add_dummy(m(S), [n2])                       # del S
+    n4 = g.add_einsummable(exp, [m(X), m(Y)], [n1])    # writes X's range, waits for its del only
+    assert g.optimize() == 1
+    assert g.describe(n0).startswith("dummy")
+    assert g.describe(n2).startswith("einsummable %d:4096 %d:4096 |" % (T * 4096, X * 4096))
+    # the writer of X now waits for the node that reads X
+    assert n2 in g.node_info(n4)[2]
+    g.finalize(2)
+    s2, s4 = g.node_info(n2)[1], g.node_info(n4)[1]
+    assert s2 == s4 or g.cross_stream_waits() >= 1
+
+    # the same through two dummies in a row, and with the del behind the reader
+    g = ea.ApplyGraph(None)
+    n0 = g.add_einsummable(exp, [m(S), m(X)])
+    n1 = g.add_dummy((0, 0), [n0])
+    n2 = g.add_dummy(m(X), [n1])
+    n3 = g.add_einsummable(sq, [m(T), m(S)], [n0])
+    n4 = g.add_dummy(m(S), [n3])
+    n5 = g.add_dummy(m(X), [n0])                       # a del of X listed behind the reader
+    n6 = g.add_einsummable(exp, [m(X), m(Y)], [n2])
+    n7 = g.add_einsummable(exp, [m(X), m(Y)], [n5, n6])
+    assert g.optimize() == 1
+    assert n3 in g.node_info(n6)[2]
+    assert n3 in g.node_info(n5)[2]
+
+    # a ranged dummy that is not a del (an alloc of the memgraph) deletes nothing
+    wire_like = ea.ApplyGraph(None)
+    a = wire_like.add_einsummable(exp, [m(S), m(X)])
+    b = wire_like.add_einsummable(sq, [m(T), m(S)], [a])
+    wire_like.add_dummy(m(S), [b], is_del=False)
+    assert wire_like.optimize() == 0
+
+
+def test_exec_graph_optimize_on_the_reference_memgraph_layout():
+    """A decoder layer laid out as the reference's memgraph compiler does (dels right behind
+    the last user, ranges reused, ordering by edges only), loaded from the wire: before and
+    after optimize() every pair of nodes that meet in memory is ordered by the dependencies."""
+    import einsummable_amd as ea
+    import memgraph_proto as mp
+    from einsummable_amd.llama_layer import LayerGraph
+
+    lg = LayerGraph(dim=64, n_heads=2, ffn=176, seq=32)
+    mg, input_ranges, out_range, top = mp.layer_memgraph_reusing(lg)
+    kinds = [n["kind"] for n in mg["nodes"]]
+    # the layout under test: dels stand between the applies, and allocs wait for dels
+    assert kinds.index("del") < len(kinds) - 20
+    assert any(n["kind"] == "alloc" and n["inns"] for n in mg["nodes"])
+    g = ea.ApplyGraph(None)
+    g.load_memgraph(mp.to_wire(mg))
+    assert mp.unordered_conflicts(g) == []
+    assert g.optimize() > 10           # fewer than with private ranges: a reused range is often still read
+    assert mp.unordered_conflicts(g) == []
+    g.finalize(4)
