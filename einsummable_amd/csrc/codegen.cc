@@ -1506,6 +1506,7 @@ std::shared_ptr<plan_t> plan_codegen(einsummable_t const& e, int device)
             break;
     }
     p->description += " vec=" + std::to_string(p->wide.k.vec);
+    if (p->wide.k.idx64) p->description += " idx64";
     if (p->wide.k.row_pairs) p->description += " row_pairs";
     if (p->wide.k.splits > 1) p->description += " splits=" + std::to_string(p->wide.k.splits);
     p->workspace_bytes = std::max(p->wide.k.ws_bytes, p->narrow.k.ws_bytes);

@@ -21,6 +21,7 @@
 // fp16 inputs accumulate in fp32 (v_mfma_f32_32x32x16_f16), fp32 uses v_mfma_f32_32x32x2_f32,
 // f64 uses v_mfma_f64_16x16x4_f64.
 #include "gemm_dma_kernel.h"
+#include "gemm_pc_kernel.h"
 #include "gemm_kernel.h"
 #include "kernel_manager.h"
 
@@ -406,11 +407,33 @@ std::shared_ptr<plan_t> plan_contraction(einsummable_t const& e, int)
         }
     }
     a.wave8 = 0;
+    a.persistent = 0;
+    a.workgroups = 0;
     if (dt == dtype_t::f16 && p->planned_dma && a.a_mode <= 1 && a.b_mode <= 1 && !a.shortk &&
         !a.wide_slices && (p->bm == 256 || p->bn == 256) &&
         gemm::gemm_dma_wide_eligible<_Float16>(a, p->bm == 256 && p->bn == 256 ? 2u : 3u)) {
         const char* env = std::getenv("ES_KM_GEMM_WAVES");  // tuning and tests: 4 keeps the old kernel
         a.wave8 = !(env && env[0] == '4');
+        // Both operands along k, whole tiles' worth of work for every compute unit: the
+        // persistent kernels (ES_KM_GEMM_WAVES=8 keeps the eight-wavefront kernel: tests)
+        a.persistent = 0;
+        bool const along_k = a.a_mode == 0 && a.b_mode == 0 && a.splits <= 1;
+        if (a.wave8 && along_k && !(env && env[0] == '8')) {
+            if (p->bm == 256 && p->bn == 256 && gemm::w4::gemm_w4_eligible<2>(a)) {
+                a.persistent = 1;
+            } else if (p->bm != p->bn && gemm::pc::gemm_pc_eligible(a)) {
+                a.persistent = 2;
+            }
+        }
+        if (a.persistent) {
+            int dev = 0, cus = 0;
+            if (hipGetDevice(&dev) != hipSuccess ||
+                hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+                cus <= 0) {
+                a.persistent = 0;
+            }
+            a.workgroups = uint32_t(cus);
+        }
     }
     static const char* mode_name[] = {"k", "mn", "elem"};
     p->description = std::string("contraction_mfma_") + dtype_name(dt) + " tile=" +
@@ -423,7 +446,11 @@ std::shared_ptr<plan_t> plan_contraction(einsummable_t const& e, int)
                      (a.splits > 1 ? " split_k=" + std::to_string(a.splits) : "") +
                      (a.shortk ? " resident_a" : "") + (a.warm_a_bytes ? " warm_operands" : "") +
                      (a.wide_slices ? " slices=128B" : "") +
-                     (a.wave8 ? " slices=128B waves=8" : "") + (alpha != 1.0 ? " scaled" : "");
+                     (a.persistent == 1   ? " slices=128B waves=4 persistent"
+                      : a.persistent == 2 ? " slices=128B waves=4+4 persistent"
+                      : a.wave8           ? " slices=128B waves=8"
+                                          : "") +
+                     (alpha != 1.0 ? " scaled" : "");
     return p;
 }
 

@@ -68,7 +68,7 @@ __device__ __forceinline__ void wait_loads_and_lds()
 // stand-alone walk of the same pattern), eight rows per load instruction instead of sixteen,
 // and four k-steps per slice instead of two.
 template <typename T, int BM, int BN, int NS, int AMODE, int BMODE, int RB = DMA_ROW, int WGM = 2,
-          int WGN = 2, bool PIN = false>
+          int WGN = 2>
 __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dma_kernel(gemm_args_t a)
 {
     using tr = traits_t<T>;
@@ -455,12 +455,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dma_kernel(gemm_args_t a)
 #pragma unroll
             for (int q = 0; q != MMAS; ++q) {
                 int const p = q % PAIRS;
-                if constexpr (PIN) {
-                    tr::mma_pinned(acc[p / TN][p % TN], fb[s & 1][p % TN], fa[s & 1][p / TN]);
-                } else {
-                    tr::mma_sub(acc[p / TN][p % TN], fb[s & 1][p % TN], fa[s & 1][p / TN],
-                                q / PAIRS);
-                }
+                tr::mma_sub(acc[p / TN][p % TN], fb[s & 1][p % TN], fa[s & 1][p / TN], q / PAIRS);
 #pragma unroll
                 for (int r = q * R0; r != (q + 1) * R0; ++r) {
                     if (r < READS) read_frag(cur, s + 1, r, fa[(s + 1) & 1], fb[(s + 1) & 1]);
@@ -479,11 +474,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dma_kernel(gemm_args_t a)
 #pragma unroll
         for (int q = 0; q != MMAS; ++q) {
             int const p = q % PAIRS;
-            if constexpr (PIN) {
-                tr::mma_pinned(acc[p / TN][p % TN], fb[1][p % TN], fa[1][p / TN]);
-            } else {
-                tr::mma_sub(acc[p / TN][p % TN], fb[1][p % TN], fa[1][p / TN], q / PAIRS);
-            }
+            tr::mma_sub(acc[p / TN][p % TN], fb[1][p % TN], fa[1][p / TN], q / PAIRS);
             if (YOUNGER >= 0) {
                 if (q == 0) {
                     // this wave's part of slice kt+1 has landed and its reads of this stage
@@ -520,7 +511,6 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dma_kernel(gemm_args_t a)
         tail(tail, integral_constant<int, 0>{});
     }
 
-    if constexpr (PIN) settle_accumulators();
     // Epilogue: each wave turns MI rows of its tile through a private LDS strip so that the
     // global stores are 16 bytes per lane and whole row segments per wavefront.
     if (a.splits > 1) {
@@ -619,7 +609,7 @@ bool gemm_dma_wide_eligible(gemm_args_t const& a, uint32_t stages)
 }
 
 template <typename T, int BM, int BN, int NS, int AMODE, int BMODE, int RB = DMA_ROW, int WGM = 2,
-          int WGN = 2, bool PIN = false>
+          int WGN = 2>
 void launch_gemm_dma_kernel_mode(gemm_args_t const& a, hipStream_t stream)
 {
     static_assert(NS >= 2 && NS <= 4, "eligibility guarantees four slices");
@@ -627,13 +617,13 @@ void launch_gemm_dma_kernel_mode(gemm_args_t const& a, hipStream_t stream)
     static bool const raised = [] {
         (void)hipFuncSetAttribute(
             reinterpret_cast<const void*>(
-                &gemm_dma_kernel<T, BM, BN, NS, AMODE, BMODE, RB, WGM, WGN, PIN>),
+                &gemm_dma_kernel<T, BM, BN, NS, AMODE, BMODE, RB, WGM, WGN>),
             hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         return true;
     }();
     (void)raised;
     dim3 grid(a.tiles_m * a.tiles_n, a.batch, a.splits > 1 ? a.splits : 1);
-    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, NS, AMODE, BMODE, RB, WGM, WGN, PIN>), grid,
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, NS, AMODE, BMODE, RB, WGM, WGN>), grid,
                        dim3(64 * WGM * WGN), lds, stream, a);
 }
 

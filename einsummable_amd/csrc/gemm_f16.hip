@@ -1,6 +1,7 @@
 // fp16-in / fp32-accumulate instantiations of the MFMA GEMM kernel.
 #include "gemm_dma_kernel.h"
 #include "gemm_kernel.h"
+#include "gemm_pc_kernel.h"
 #include "gemm_shortk_kernel.h"
 
 namespace es
@@ -68,6 +69,16 @@ void launch_gemm_f16(int bm, int bn, gemm_args_t const& a, hipStream_t stream)
         // that one covers the other's waits.  Measured against the four-wavefront kernel on
         // 64-byte slices: 8192^3 1.13 -> 1.21 PFLOP/s, 4096^3 1.04 -> 1.14, 2048 x 4096 x
         // 4096 0.80 -> 1.00, 2048 x 11008 x 4096 0.86 -> 1.01 (results bit-identical).
+        // Both operands along k and the buffers as aligned as at build time: the persistent
+        // kernels (four wavefronts with the accumulators in named registers on 256 x 256,
+        // multiplying and loading wavefronts on the rectangular tiles)
+        if (a.persistent == 1 && bm == 256 && bn == 256 && w4::gemm_w4_eligible<2>(a)) {
+            return w4::launch_gemm_w4<256, 256, 2>(a, a.workgroups, stream);
+        }
+        if (a.persistent == 2 && pc::gemm_pc_eligible(a)) {
+            if (bm == 128 && bn == 256) return pc::launch_gemm_pc<128, 256>(a, a.workgroups, stream);
+            if (bm == 256 && bn == 128) return pc::launch_gemm_pc<256, 128>(a, a.workgroups, stream);
+        }
         if (a.wave8 && a.a_mode <= 1 && a.b_mode <= 1) {
             // (each operand along k or along its own m / n mode)
             auto modes = [&](auto launch00, auto launch01, auto launch10, auto launch11) {

@@ -64,6 +64,12 @@ struct gemm_args_t {
     // f16, both operands along k, compute bound: eight wavefronts per workgroup on slices of
     // 128 bytes (launch_gemm_f16)
     int         wave8;
+    // 0, or which of the persistent kernels runs it (f16, both operands along k, compute
+    // bound): 1 four wavefronts on 256 x 256 (gemm_w4_kernel), 2 four multiplying and four
+    // loading wavefronts on 128 x 256 / 256 x 128 (gemm_pc_kernel); `workgroups`: how many
+    // of them walk the tiles (the device's compute units)
+    int         persistent;
+    uint32_t    workgroups;
     // every sum is multiplied by this before it is rounded to the output type (1 for a plain
     // product); split-K partial tiles stay unscaled, the fold applies it
     double      alpha;
@@ -175,30 +181,8 @@ struct traits_t<_Float16> {
     {
         mma(acc, row, col);
     }
-    // The same instruction with the accumulator pinned to the accumulation registers.  A
-    // wave that owns 128 x 128 of C holds 256 accumulators, all of a[0:255]; left to itself
-    // the register allocator keeps some of them in v registers and moves them to and fro
-    // around every matrix instruction (five moves per instruction) and spills.  The compiler
-    // does not see the instruction: callers keep dependent instructions apart themselves
-    // (the main loops go round all accumulator tiles between two uses of one; see
-    // settle_accumulators for the reads that follow).
-    __device__ static __forceinline__ void mma_pinned(acc_t& acc, chunk_t const& row,
-                                                      chunk_t const& col)
-    {
-        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0"
-                     : "+a"(acc)
-                     : "v"(row), "v"(col));
-    }
 };
 
-// After the last pinned matrix instruction and before anything else reads an accumulator:
-// an 8-pass instruction needs 11 idle issue slots before its result may be read by another
-// unit, and the compiler, which inserts them for its own matrix instructions, does not know
-// that the assembly statements were any.
-__device__ __forceinline__ void settle_accumulators()
-{
-    asm volatile("s_nop 15\n\ts_nop 7" : : : "memory");
-}
 
 template <>
 struct traits_t<float> {

@@ -270,12 +270,16 @@ EIGHT_WAVE_CASES = [
 @pytest.mark.parametrize("case", range(len(EIGHT_WAVE_CASES)))
 def test_eight_wavefront_kernels_match_the_four_wavefront_ones_bitwise(km, monkeypatch, case, tile):
     # same products summed in the same order: the bits must agree on random data, and both
-    # must agree with the oracle
+    # must agree with the oracle.  The default plan is a third kernel where both operands lie
+    # along k (persistent workgroups, accumulators in named registers): the same bits again.
     spec, sizes = EIGHT_WAVE_CASES[case]
     e = contraction(spec, sizes, "f16")
     monkeypatch.setenv("ES_KM_GEMM_TILE", tile)
+    default = ea.KernelManager(0)
+    default.build(e)  # the planner reads its tuning variables when it plans
+    monkeypatch.setenv("ES_KM_GEMM_WAVES", "8")
     eight = ea.KernelManager(0)
-    eight.build(e)  # the planner reads its tuning variables when it plans
+    eight.build(e)
     monkeypatch.setenv("ES_KM_GEMM_WAVES", "4")
     four = ea.KernelManager(0)
     four.build(e)
@@ -283,10 +287,67 @@ def test_eight_wavefront_kernels_match_the_four_wavefront_ones_bitwise(km, monke
     xs = [uniform(r, int(np.prod(e.inn_shape(k))), np.float16) for k in range(2)]
     a = run_einsummable(eight, e, xs)
     b = run_einsummable(four, e, xs)
+    c = run_einsummable(default, e, xs)
     assert "waves=8" in eight.describe(e), eight.describe(e)
-    assert "waves=8" not in four.describe(e) and "tile=" + tile in four.describe(e), four.describe(e)
+    assert "waves=" not in four.describe(e) and "tile=" + tile in four.describe(e), four.describe(e)
+    d = default.describe(e)
+    along_k = " A=k B=k " in d and "split_k" not in d
+    assert ("persistent" in d) == along_k, d
+    if along_k:
+        assert ("waves=4 persistent" if tile == "256x256" else "waves=4+4 persistent") in d, d
     np.testing.assert_array_equal(a.view(np.uint16), b.view(np.uint16))
+    np.testing.assert_array_equal(a.view(np.uint16), c.view(np.uint16))
     assert_close(a, oracle_einsummable(e, xs, oracle.WIDE), ea.F16, what=eight.describe(e))
+
+
+PERSISTENT_CASES = [
+    # several tiles per workgroup, ragged edges (the output's inner extent in whole 16-byte
+    # vectors: the wide epilogue), K not a multiple of the stage count
+    ("ij,kj->ik", dict(i=2300, j=448, k=4504), "256x256"),
+    ("ij,kj->ik", dict(i=2300, j=448, k=4504), "128x256"),
+    ("ij,kj->ik", dict(i=4500, j=320, k=2296), "256x128"),
+    # a batch of products walked across its entries; two k modes stepped by the slice walker
+    ("bij,bkj->bik", dict(b=40, i=520, j=192, k=776), "128x256"),
+    ("bij,bkj->bik", dict(b=9, i=1030, j=256, k=1288), "256x256"),
+    ("adbe,cde->abc", dict(a=2, d=4, b=1100, e=64, c=2056), "128x256"),
+    ("adbe,cde->abc", dict(a=1, d=3, b=2100, e=128, c=2056), "256x256"),
+    # the scale applied to the fp32 sums in the epilogue
+    ("ij,kj->ik", dict(i=1500, j=512, k=3000), "256x128"),
+]
+
+
+@pytest.mark.parametrize("case", range(len(PERSISTENT_CASES)))
+def test_persistent_kernels_walk_many_tiles(km, monkeypatch, case):
+    """More tiles than compute units: every workgroup of the persistent kernels computes
+    several tiles, with the next tile's first slices loaded under the current one's last.
+    Bitwise equal to the eight-wavefront kernel (same order of summation) and within the
+    f16 tolerance of the oracle."""
+    spec, sizes, tile = PERSISTENT_CASES[case]
+    scaled = case == len(PERSISTENT_CASES) - 1
+    e = contraction(spec, sizes, "f16")
+    if scaled:
+        e = ea.Einsummable(e.join_shape, e.inns, e.out_rank,
+                           "*[constant{f16|0.0883789},*[hole|f16@0,hole|f16@1]]", "+")
+    monkeypatch.setenv("ES_KM_GEMM_TILE", tile)
+    pers = ea.KernelManager(0)
+    pers.build(e)
+    monkeypatch.setenv("ES_KM_GEMM_WAVES", "8")
+    eight = ea.KernelManager(0)
+    eight.build(e)
+    assert "persistent" in pers.describe(e) and "tile=" + tile in pers.describe(e), pers.describe(e)
+    assert "waves=8" in eight.describe(e), eight.describe(e)
+    r = rng(300 + case)
+    xs = [uniform(r, int(np.prod(e.inn_shape(k))), np.float16) for k in range(2)]
+    a = run_einsummable(pers, e, xs)
+    b = run_einsummable(eight, e, xs)
+    np.testing.assert_array_equal(a.view(np.uint16), b.view(np.uint16))
+    # the oracle on a sample of rows (the whole product would take it minutes)
+    if not scaled and spec == "ij,kj->ik":
+        i, j, k = sizes["i"], sizes["j"], sizes["k"]
+        rows = np.array([0, 1, 127, 128, 255, 256, i // 2, i - 2, i - 1])
+        sub = contraction(spec, dict(i=len(rows), j=j, k=k), "f16")
+        want = oracle_einsummable(sub, [xs[0].reshape(i, j)[rows].reshape(-1), xs[1]], oracle.WIDE)
+        assert_close(a.reshape(i, k)[rows].reshape(-1), want, ea.F16, what=pers.describe(e))
 
 
 def test_big_tile_matches_small_tile_bitwise_on_exact_data(km, monkeypatch):
