@@ -927,44 +927,53 @@ import json, sys, time
 sys.path.insert(0, %r)
 import torch
 import einsummable_amd as ea
-from einsummable_amd.llama_layer import LayerGraph
+from einsummable_amd.llama_layer import ArenaRunner, LayerGraph
+mode = %r
 torch.cuda.init()
 km = ea.KernelManager(0)
 g = LayerGraph()
+n = len([1 for node in g.nodes if node["kind"] == "einsummable"])
 t0 = time.perf_counter()
-n = 0
-for node in g.nodes:
-    if node["kind"] == "einsummable":
-        km.build(node["e"])
-        n += 1
+if mode == "graph":
+    # the exec graph builds its distinct einsummables together (es_km_graph_finalize)
+    ArenaRunner(km, g, n_streams=1)
+else:
+    for node in g.nodes:
+        if node["kind"] == "einsummable":
+            km.build(node["e"])
 print(json.dumps({"ms": (time.perf_counter() - t0) * 1e3, "einsummables": n}))
 """
 
 
 def run_build_latency():
-    """Time of kernel_manager_t::build over the einsummables of the LLaMA-7B layer (runtime
-    compilation of the generated kernels is most of it), in a fresh process with an empty
-    code-object cache and again in a second process that finds the cache filled."""
+    """Time to build the einsummables of the LLaMA-7B layer (runtime compilation of the
+    generated kernels is most of it): through the exec graph, which builds a graph's
+    distinct einsummables on several threads, in a fresh process with an empty code-object
+    cache and again in a second process that finds the cache filled; and one build() call
+    after the other (the reference's call pattern) in a third process with an empty cache."""
     import shutil
     import subprocess
     import tempfile
 
     root = os.path.dirname(os.path.abspath(__file__))
-    cache = tempfile.mkdtemp(prefix="es_km_cache_")
     out = {}
+    runs = [("first_process_empty_cache", "graph", 0), ("second_process_cache_on_disk", "graph", 0),
+            ("one_build_call_after_the_other_empty_cache", "serial", 1)]
+    caches = [tempfile.mkdtemp(prefix="es_km_cache_") for _ in range(2)]
     try:
-        env = dict(os.environ, ES_KM_CACHE_DIR=cache)
-        for label in ("first_process_empty_cache", "second_process_cache_on_disk"):
-            p = subprocess.run([sys.executable, "-c", BUILD_PROBE % root], env=env,
+        for label, mode, which in runs:
+            env = dict(os.environ, ES_KM_CACHE_DIR=caches[which])
+            p = subprocess.run([sys.executable, "-c", BUILD_PROBE % (root, mode)], env=env,
                                capture_output=True, text=True, timeout=600)
             if p.returncode != 0:
                 out[label] = {"error": p.stderr[-300:]}
                 continue
             r = json.loads(p.stdout.strip().splitlines()[-1])
             out[label] = {"build_ms": round(r["ms"], 1), "einsummables": r["einsummables"]}
-        out["code_objects_cached"] = len([f for f in os.listdir(cache) if f.endswith(".co")])
+        out["code_objects_cached"] = len([f for f in os.listdir(caches[0]) if f.endswith(".co")])
     finally:
-        shutil.rmtree(cache, ignore_errors=True)
+        for c in caches:
+            shutil.rmtree(c, ignore_errors=True)
     return out
 
 

@@ -27,4 +27,5 @@ from .km import (  # noqa: F401
     memgraph_describe,
     merge_adjacent_dims,
     scalarop_roundtrip,
+    scalarop_simplify,
 )

@@ -394,6 +394,23 @@ int es_km_scalarop_roundtrip(const char* text, char* out, size_t cap, int* out_d
     });
 }
 
+int es_km_scalarop_simplify(const char* text, const char* const* var_names,
+                            const double* var_values, int n_vars, char* out, size_t cap)
+{
+    return guarded(nullptr, [&]() -> int {
+        if (!text || !out || cap == 0) throw es::ir_error("simplify: null argument");
+        if (n_vars < 0 || (n_vars > 0 && (!var_names || !var_values))) {
+            throw es::ir_error("simplify: bad variable list");
+        }
+        std::vector<std::pair<std::string, double>> vars;
+        for (int i = 0; i != n_vars; ++i) vars.emplace_back(var_names[i], var_values[i]);
+        std::string const s = es::scalarop_t::parse(text).replace_variables(vars).simplify().str();
+        if (s.size() + 1 > cap) throw es::ir_error("simplify: buffer too small");
+        std::memcpy(out, s.c_str(), s.size() + 1);
+        return ES_KM_OK;
+    });
+}
+
 int es_km_merge_adjacent_dims(const uint64_t* join_shape, int join_rank, const int* inns_flat,
                               const int* inns_offsets, int n_inns, int out_rank,
                               const char* join_text, char castable, uint64_t* new_join_shape,

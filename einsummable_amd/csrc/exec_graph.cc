@@ -595,9 +595,13 @@ void apply_graph_t::finalize(int n_streams)
     }
     int const n = int(nodes_.size());
     if (km_) {
+        // the graph's distinct einsummables are built together, on several threads
+        std::vector<einsummable_t> es;
         for (node_t const& nd : nodes_) {
-            if (nd.kind != kind_t::einsummable) continue;
-            if (!km_->build(nd.e)) {
+            if (nd.kind == kind_t::einsummable) es.push_back(nd.e);
+        }
+        for (std::optional<uint64_t> const& ws : km_->build_many(es)) {
+            if (!ws) {
                 throw km_error(km_status::invalid, "apply graph: no kernel for an einsummable "
                                                    "(build returned unsupported)");
             }

@@ -253,14 +253,14 @@ __global__ __launch_bounds__(256) void gemm_w4_kernel(gemm_args_t a, uint32_t to
         }
         rewind_k();
     };
-    // load q of the loader's slice into stage ST: A rows for q < NLA, B rows after that
-    auto issue = [&](auto st_tag, auto q_tag) ES_INLINE {
-        constexpr int q = decltype(q_tag)::value, ST = decltype(st_tag)::value;
-        // this wave's first slot of the stage plus the instruction's own slot: a constant
+    // load q of the loader's slice into the stage whose first slot of this wave is `slot`: A
+    // rows for q < NLA, B rows after that; the instruction's own slot is a constant
+    auto issue = [&](uint32_t slot, auto q_tag) ES_INLINE {
+        constexpr int q = decltype(q_tag)::value;
         if constexpr (q < NLA) {
-            load_lds<ST * STAGE + NW * q * 1024>(A_ld, voa[q], lds_wave);
+            load_lds<NW * q * 1024>(A_ld, voa[q], slot);
         } else {
-            load_lds<ST * STAGE + A_BYTES + NW * (q - NLA) * 1024>(B_ld, vob[q - NLA], lds_wave);
+            load_lds<A_BYTES + NW * (q - NLA) * 1024>(B_ld, vob[q - NLA], slot);
         }
     };
     // on to the next slice of the loader's tile
@@ -312,10 +312,9 @@ __global__ __launch_bounds__(256) void gemm_w4_kernel(gemm_args_t a, uint32_t to
     int const fb_base = A_BYTES + wn * WN * RB;
     chunk_t   fa[2][TM], fb[2][TN];
     // read order: what the first matrix instructions of a step need comes first
-    auto read_frag = [&](auto st_tag, auto s_tag, auto q_tag, chunk_t(&xa)[TM],
+    auto read_frag = [&](char const* stage, auto s_tag, auto q_tag, chunk_t(&xa)[TM],
                          chunk_t(&xb)[TN]) ES_INLINE {
         constexpr int s = decltype(s_tag)::value, q = decltype(q_tag)::value;
-        char const*   stage = lds + decltype(st_tag)::value * STAGE;
         if constexpr (q == 0) {
             xa[0] = *reinterpret_cast<chunk_t const*>(stage + fa_base + f_off[s]);
         } else if constexpr (q <= TN) {
@@ -331,37 +330,40 @@ __global__ __launch_bounds__(256) void gemm_w4_kernel(gemm_args_t a, uint32_t to
     // ---- prologue: slices 0 .. NS-2 whole and part 0 of slice NS-1 in flight
     seek_tile(L_ld);
     static_for<NS - 1>([&](auto st_tag) ES_INLINE {
-        static_for<LOADS>([&](auto q_tag) ES_INLINE { issue(st_tag, q_tag); });
+        static_for<LOADS>([&](auto q_tag) ES_INLINE {
+            issue(lds_wave + decltype(st_tag)::value * STAGE, q_tag);
+        });
         next_slice();  // nk >= NS: still inside the first tile
     });
     static_for<LOADS / PARTS>([&](auto q_tag) ES_INLINE {
-        issue(integral_constant<int, NS - 1>{}, q_tag);
+        issue(lds_wave + (NS - 1) * STAGE, q_tag);
     });
     wait_vm_lgkm<(NS - 2) * LOADS + LOADS / PARTS>();
     __builtin_amdgcn_s_barrier();
     static_for<READS>([&](auto q_tag) ES_INLINE {
-        read_frag(integral_constant<int, 0>{}, integral_constant<int, 0>{}, q_tag, fa[0], fb[0]);
+        read_frag(lds, integral_constant<int, 0>{}, q_tag, fa[0], fb[0]);
     });
 
-    // One slice, computed from stage ST, in two halves with the loader's step between them.
-    // k-steps 0 .. 2: the other parts of the loader's slice go to the stage before ST.
-    auto head = [&](auto st_tag) ES_INLINE {
-        constexpr int ST = decltype(st_tag)::value;
-        using ld_stage = integral_constant<int, (ST + NS - 1) % NS>;
+    // One slice, computed from stage st, in two halves with the loader's step between them.
+    // k-steps 0 .. 2: the other parts of the loader's slice go to the stage before st.
+    uint32_t st = 0;  // stage of the slice being computed
+    auto head = [&]() ES_INLINE {
+        char const*    cur = lds + st * STAGE;
+        uint32_t const ld_slot = lds_wave + (st == 0 ? NS - 1 : st - 1) * STAGE;
         static_for<STEPS - 1>([&](auto s_tag) ES_INLINE {
             constexpr int s = decltype(s_tag)::value;
             static_for<NT>([&](auto q_tag) ES_INLINE {
                 constexpr int q = decltype(q_tag)::value;
                 mma<q>(fb[s & 1][q % TN], fa[s & 1][q / TN]);
                 if constexpr (q < READS) {
-                    read_frag(st_tag, integral_constant<int, s + 1>{}, q_tag, fa[(s + 1) & 1],
+                    read_frag(cur, integral_constant<int, s + 1>{}, q_tag, fa[(s + 1) & 1],
                               fb[(s + 1) & 1]);
                 }
                 if constexpr (s + 1 < PARTS) {
                     // part s + 1 of the loader's slice, spread over the step
                     constexpr int lo = (s + 1) * LOADS / PARTS, n = LOADS / PARTS;
                     static_for<(q + 1) * n / NT - q * n / NT>([&](auto r_tag) ES_INLINE {
-                        issue(ld_stage{},
+                        issue(ld_slot,
                               integral_constant<int, lo + q * n / NT + decltype(r_tag)::value>{});
                     });
                 }
@@ -372,10 +374,11 @@ __global__ __launch_bounds__(256) void gemm_w4_kernel(gemm_args_t a, uint32_t to
     // The last k-step: the next slice has landed, this stage is free and takes part 0 of the
     // loader's new slice -- unless this is the tile's LAST slice: then the freed stage is the
     // epilogue's first.
-    auto tail = [&](auto st_tag, auto last_tag) ES_INLINE {
-        constexpr int  ST = decltype(st_tag)::value;
+    auto tail = [&](auto last_tag) ES_INLINE {
         constexpr bool LAST = decltype(last_tag)::value;
-        using next_stage = integral_constant<int, (ST + 1) % NS>;
+        uint32_t const nx = st + 1 == NS ? 0 : st + 1;
+        char const*    nxt = lds + nx * STAGE;
+        uint32_t const ld_slot = lds_wave + st * STAGE;
         static_for<NT>([&](auto q_tag) ES_INLINE {
             constexpr int q = decltype(q_tag)::value;
             mma<q>(fb[1][q % TN], fa[1][q / TN]);
@@ -386,26 +389,29 @@ __global__ __launch_bounds__(256) void gemm_w4_kernel(gemm_args_t a, uint32_t to
                 __builtin_amdgcn_s_barrier();
             } else {
                 if constexpr (q - 1 < READS) {
-                    read_frag(next_stage{}, integral_constant<int, 0>{},
-                              integral_constant<int, q - 1>{}, fa[0], fb[0]);
+                    read_frag(nxt, integral_constant<int, 0>{}, integral_constant<int, q - 1>{},
+                              fa[0], fb[0]);
                 }
                 if constexpr (!LAST) {
                     constexpr int n = LOADS / PARTS;
                     static_for<q * n / (NT - 1) - (q - 1) * n / (NT - 1)>([&](auto r_tag) ES_INLINE {
-                        issue(st_tag, integral_constant<int, (q - 1) * n / (NT - 1) +
-                                                                 decltype(r_tag)::value>{});
+                        issue(ld_slot, integral_constant<int, (q - 1) * n / (NT - 1) +
+                                                                  decltype(r_tag)::value>{});
                     });
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
         });
+        st = nx;
     };
 
     // ---- epilogue of one tile: each wave turns 32 rows of its part through an LDS strip in
     // the stage that has just been freed, so that the global stores are 16 bytes per lane
-    // and whole row segments; the accumulators are cleared on the way
+    // and whole row segments; the accumulators are cleared on the way.  All chunks of a band
+    // are read back before the first store, so the LDS latency is paid once per band.
     constexpr int STRIP_PITCH = WN * int(sizeof(T)) + 16;
     constexpr int CPR = WN * int(sizeof(T)) / 16;
+    constexpr int CPL = MI * CPR / 64;  // chunks per lane per band
     static_assert(NW * MI * STRIP_PITCH <= STAGE, "");
     float const alpha = float(a.alpha);
     auto epilogue = [&](uint32_t L, uint32_t freed_stage) ES_INLINE {
@@ -426,6 +432,16 @@ __global__ __launch_bounds__(256) void gemm_w4_kernel(gemm_args_t a, uint32_t to
         T* const    C = static_cast<T*>(a.C) + boc;
         char* const strip = lds + freed_stage * STAGE + wave * (MI * STRIP_PITCH);
         typedef T   quad_t __attribute__((ext_vector_type(4)));
+        // this lane's chunks of a band: rows lane / CPR + c * (64 / CPR), 16 bytes at
+        // (lane % CPR) * 8 elements
+        uint32_t const m0 = t.tm * BM + wm * WM + uint32_t(lane / CPR);
+        uint32_t const n0 = t.tn * BN + wn * WN + uint32_t(lane % CPR) * VL;
+        // C with one mode per side and unit stride along n: a row is a multiple of the
+        // leading dimension away (32-bit byte offsets from the tile's first row: a.lin)
+        bool const     lin = a.lin != 0;
+        uint32_t const ldc_bytes = uint32_t(a.gm.sy[0]) * uint32_t(sizeof(T));
+        char* const    c_lin = reinterpret_cast<char*>(C) + int64_t(t.tm * BM + wm * WM) * a.gm.sy[0] * int64_t(sizeof(T));
+        uint32_t const v_lin = uint32_t(lane / CPR) * ldc_bytes + n0 * uint32_t(sizeof(T));
         settle();
         static_for<TM>([&](auto i_tag) ES_INLINE {
             constexpr int i = decltype(i_tag)::value;
@@ -451,26 +467,35 @@ __global__ __launch_bounds__(256) void gemm_w4_kernel(gemm_args_t a, uint32_t to
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            chunk_t v[CPL];
 #pragma unroll
-            for (int c = 0; c != MI * CPR / 64; ++c) {
-                int      idx = c * 64 + lane;
-                int      r = idx / CPR, ch = idx % CPR;
-                uint32_t m = t.tm * BM + wm * WM + i * MI + uint32_t(r);
-                uint32_t n = t.tn * BN + wn * WN + uint32_t(ch) * VL;
-                chunk_t  v = *reinterpret_cast<chunk_t const*>(strip + r * STRIP_PITCH + ch * 16);
+            for (int c = 0; c != CPL; ++c) {
+                int const idx = c * 64 + lane;
+                v[c] = *reinterpret_cast<chunk_t const*>(strip + (idx / CPR) * STRIP_PITCH +
+                                                         (idx % CPR) * 16);
+            }
+#pragma unroll
+            for (int c = 0; c != CPL; ++c) {
+                uint32_t const m = m0 + uint32_t(i * MI + c * (64 / CPR));
 #ifdef ES_W4_ABL_NO_STORE
-                if (m < a.M && n < a.N && v[0] == 0x12345678u) {
+                if (m < a.M && n0 < a.N && v[c][0] == 0x12345678u) {
 #else
-                if (m < a.M && n < a.N) {
+                if (m < a.M && n0 < a.N) {
 #endif
-                    int64_t mo_a, mo_c, no_b, no_c;
-                    group_offsets(a.gm, m, mo_a, mo_c);
-                    group_offsets(a.gn, n, no_b, no_c);
-                    chunk_t* const dst = reinterpret_cast<chunk_t*>(C + mo_c + no_c);
-                    if (a.c_stream) {
-                        store_16_streaming(dst, v);
+                    chunk_t* dst;
+                    if (lin) {
+                        dst = reinterpret_cast<chunk_t*>(
+                            c_lin + (v_lin + uint32_t(i * MI + c * (64 / CPR)) * ldc_bytes));
                     } else {
-                        *dst = v;
+                        int64_t mo_a, mo_c, no_b, no_c;
+                        group_offsets(a.gm, m, mo_a, mo_c);
+                        group_offsets(a.gn, n0, no_b, no_c);
+                        dst = reinterpret_cast<chunk_t*>(C + mo_c + no_c);
+                    }
+                    if (a.c_stream) {
+                        store_16_streaming(dst, v[c]);
+                    } else {
+                        *dst = v[c];
                     }
                 }
             }
@@ -483,34 +508,21 @@ __global__ __launch_bounds__(256) void gemm_w4_kernel(gemm_args_t a, uint32_t to
     // ---- the walk over this workgroup's tiles.  The loader is NS - 1 slices ahead of the
     // slice being computed and steps once per slice; in the tile's slice nk - NS it steps
     // into the next tile.
-    uint32_t st_c = 0;  // stage of the slice being computed
-    auto on_stage = [&](auto&& f) ES_INLINE {
-        if constexpr (NS == 2) {
-            if (st_c == 0) f(integral_constant<int, 0>{});
-            else f(integral_constant<int, 1>{});
-        } else {
-            if (st_c == 0) f(integral_constant<int, 0>{});
-            else if (st_c == 1) f(integral_constant<int, 1>{});
-            else f(integral_constant<int, 2>{});
-        }
-    };
     uint32_t const my_tiles = (total_tiles - blockIdx.x + G - 1) / G;
     for (uint32_t it = 0; it != my_tiles; ++it) {
 #ifdef ES_W4_STAMP
         uint64_t const stamp0 = __builtin_amdgcn_s_memtime();
 #endif
         for (uint32_t kt = 0; kt + 1 < nk; ++kt) {
-            on_stage([&](auto st_tag) ES_INLINE { head(st_tag); });
+            head();
             if (kt + NS == nk) next_tile();
             else next_slice();
-            on_stage([&](auto st_tag) ES_INLINE { tail(st_tag, std::false_type{}); });
-            st_c = st_c + 1 == NS ? 0 : st_c + 1;
+            tail(std::false_type{});
         }
-        on_stage([&](auto st_tag) ES_INLINE { head(st_tag); });
+        head();
         next_slice();
-        on_stage([&](auto st_tag) ES_INLINE { tail(st_tag, std::true_type{}); });
-        uint32_t const freed = st_c;
-        st_c = st_c + 1 == NS ? 0 : st_c + 1;
+        uint32_t const freed = st;
+        tail(std::true_type{});
 #ifdef ES_W4_STAMP
         uint64_t const stamp1 = __builtin_amdgcn_s_memtime();
 #endif
@@ -521,27 +533,18 @@ __global__ __launch_bounds__(256) void gemm_w4_kernel(gemm_args_t a, uint32_t to
         // every wave is done with its strip: the stage can take part 0 of its next slice
         asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");
         __builtin_amdgcn_s_barrier();
-        auto part0 = [&](auto st_tag) ES_INLINE {
-            static_for<LOADS / PARTS>([&](auto q_tag) ES_INLINE { issue(st_tag, q_tag); });
-        };
-        if constexpr (NS == 2) {
-            if (freed == 0) part0(integral_constant<int, 0>{});
-            else part0(integral_constant<int, 1>{});
-        } else {
-            if (freed == 0) part0(integral_constant<int, 0>{});
-            else if (freed == 1) part0(integral_constant<int, 1>{});
-            else part0(integral_constant<int, 2>{});
-        }
+        static_for<LOADS / PARTS>([&](auto q_tag) ES_INLINE {
+            issue(lds_wave + freed * STAGE, q_tag);
+        });
 #ifdef ES_W4_STAMP
         {
-            uint64_t const stamp3 = __builtin_amdgcn_s_memtime();
             asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");
             if (tid == 0 && it < 8) {
                 uint64_t* dst = reinterpret_cast<uint64_t*>(a.ws) + (size_t(blockIdx.x) * 8 + it) * 4;
                 dst[0] = stamp0;
                 dst[1] = stamp1;
                 dst[2] = stamp2;
-                dst[3] = stamp3;
+                dst[3] = stamp0;
             }
         }
 #endif

@@ -2,6 +2,7 @@
 
 #include <algorithm>
 #include <cmath>
+#include <complex>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -441,6 +442,239 @@ scalarop_t scalarop_t::replace_variables(
 {
     scalarop_t ret = *this;
     replace_in(ret.root, values);
+    return ret;
+}
+
+namespace
+{
+// node_t's operator== in the reference compares the printed texts (scalarop.cc:2648-2651): two
+// constants that print alike are equal, and a NaN equals a NaN
+bool same_node(node_t const& a, node_t const& b)
+{
+    std::string x, y;
+    print_node(x, a);
+    print_node(y, b);
+    return x == y;
+}
+
+int max_hole(node_t const& n)
+{
+    if (n.kind == op_kind::hole) return n.arg;
+    int r = -1;
+    for (node_t const& c : n.children) r = std::max(r, max_hole(c));
+    return r;
+}
+
+bool has_hole(node_t const& n) { return max_hole(n) >= 0; }
+
+struct value_t {
+    double re = 0.0, im = 0.0;  // held in the node's dtype (f16 / f32 values are exact in double)
+};
+
+// op_t::eval (scalarop.cc:554-780) on constants: every operation in its dtype
+value_t eval_constant(node_t const& n)
+{
+    if (n.kind == op_kind::constant) return value_t{n.re, n.im};
+    std::vector<value_t> x;
+    for (node_t const& c : n.children) x.push_back(eval_constant(c));
+    dtype_t const in = n.children.empty() ? n.dtype : n.children[0].dtype;
+    auto          rnd = [&](dtype_t d, double v) { return round_to_dtype(d, v); };
+    switch (n.kind) {
+        case op_kind::add:
+            if (in == dtype_t::c64) {
+                return value_t{double(float(x[0].re) + float(x[1].re)),
+                               double(float(x[0].im) + float(x[1].im))};
+            }
+            // the sum of two f16 or two f32 values is exact in double: one rounding
+            return value_t{rnd(in, x[0].re + x[1].re), 0.0};
+        case op_kind::mul:
+            if (in == dtype_t::c64) {
+                std::complex<float> const r = std::complex<float>(float(x[0].re), float(x[0].im)) *
+                                              std::complex<float>(float(x[1].re), float(x[1].im));
+                return value_t{double(r.real()), double(r.imag())};
+            }
+            if (in == dtype_t::f32) return value_t{double(float(x[0].re) * float(x[1].re)), 0.0};
+            return value_t{rnd(in, x[0].re * x[1].re), 0.0};
+        case op_kind::exp:
+            if (in == dtype_t::f32) return value_t{double(std::exp(float(x[0].re))), 0.0};
+            return value_t{rnd(in, std::exp(x[0].re)), 0.0};
+        case op_kind::log:
+            if (in == dtype_t::f32) return value_t{double(std::log(float(x[0].re))), 0.0};
+            return value_t{rnd(in, std::log(x[0].re)), 0.0};
+        case op_kind::power:
+            if (in == dtype_t::f32) {
+                return value_t{double(std::pow(float(x[0].re), float(n.power))), 0.0};
+            }
+            if (in == dtype_t::f16) {
+                return value_t{rnd(in, std::pow(x[0].re, rnd(dtype_t::f16, n.power))), 0.0};
+            }
+            return value_t{std::pow(x[0].re, n.power), 0.0};
+        case op_kind::ite: {
+            bool c = false;
+            switch (n.compare) {
+                case compare_t::lt: c = x[0].re < x[1].re; break;
+                case compare_t::gt: c = x[0].re > x[1].re; break;
+                case compare_t::eq: c = x[0].re == x[1].re; break;
+                case compare_t::le: c = x[0].re <= x[1].re; break;
+                case compare_t::ge: c = x[0].re >= x[1].re; break;
+            }
+            return c ? x[2] : x[3];
+        }
+        case op_kind::convert:
+            return value_t{rnd(n.dtype, x[0].re), 0.0};
+        case op_kind::conj:
+            return value_t{x[0].re, -x[0].im};
+        case op_kind::real:
+            return value_t{x[0].re, 0.0};
+        case op_kind::imag:
+            return value_t{x[0].im, 0.0};
+        case op_kind::cplex:
+            return value_t{x[0].re, x[1].re};
+        default:
+            throw ir_error("simplify: cannot evaluate a hole or a variable");
+    }
+}
+
+// "constant{" + write_with_ss(value) + "}" read back (scalarop.cc:1258-1260): the value
+// passes through six significant digits
+node_t constant_through_text(dtype_t dt, value_t v)
+{
+    node_t c;
+    c.kind = op_kind::constant;
+    c.dtype = dt;
+    c.re = v.re;
+    c.im = v.im;
+    std::string text;
+    print_node(text, c);
+    cursor_t cur{text};
+    return parse_node(cur, 0);
+}
+
+node_t make_const(dtype_t dt, double re, double im = 0.0)
+{
+    node_t c;
+    c.kind = op_kind::constant;
+    c.dtype = dt;
+    c.re = re;
+    c.im = im;
+    return c;
+}
+
+bool is_const(node_t const& n, double re, double im = 0.0)
+{
+    return n.kind == op_kind::constant && n.re == re && n.im == im;
+}
+
+compare_t compare_flip(compare_t c)
+{
+    switch (c) {
+        case compare_t::lt: return compare_t::ge;
+        case compare_t::gt: return compare_t::le;
+        case compare_t::eq: return compare_t::eq;
+        case compare_t::le: return compare_t::gt;
+        default: return compare_t::lt;
+    }
+}
+
+node_t simplify_node(node_t const& n);
+
+node_t simplify_once(node_t const& n)
+{
+    if (n.kind == op_kind::hole || n.kind == op_kind::constant || n.kind == op_kind::variable) {
+        return n;
+    }
+    if (!has_hole(n) && !node_has_variable(n)) {
+        return constant_through_text(n.dtype, eval_constant(n));
+    }
+    node_t self = n;
+    for (node_t& c : self.children) c = simplify_node(c);
+    std::vector<node_t>& ch = self.children;
+
+    // normalize_order: the operand with the smaller highest hole comes first (a constant has
+    // none: -1); equal highest holes are left as they stand
+    auto unordered = [](node_t const& l, node_t const& r) { return max_hole(r) < max_hole(l); };
+    if (n.kind == op_kind::add || n.kind == op_kind::mul) {
+        if (unordered(ch[0], ch[1])) {
+            std::swap(ch[0], ch[1]);
+            return self;
+        }
+    } else if (n.kind == op_kind::ite) {
+        bool const fix_co = unordered(ch[0], ch[1]);
+        bool const fix_tt = unordered(ch[2], ch[3]);
+        if (fix_co) {
+            self.compare = compare_flip(self.compare);
+            std::swap(ch[0], ch[1]);
+        }
+        if (fix_tt) std::swap(ch[2], ch[3]);
+        if (fix_co || fix_tt) return self;
+    }
+
+    dtype_t const dt = n.dtype;
+    bool const    cx = dt == dtype_t::c64;
+    if (n.kind == op_kind::add) {
+        if (is_const(ch[0], 0.0)) return ch[1];
+        if (is_const(ch[1], 0.0)) return ch[0];
+        if (!cx) {
+            for (int i = 0; i != 2; ++i) {
+                if (ch[i].kind == op_kind::constant && std::isinf(ch[i].re)) return ch[i];
+            }
+        }
+    }
+    if (n.kind == op_kind::mul) {
+        if (is_const(ch[0], 0.0) || is_const(ch[1], 0.0)) return make_const(dt, 0.0);
+        auto fold_pair = [&]() -> std::optional<node_t> {
+            // c0 * (c1 * hole)
+            if (ch[0].kind == op_kind::constant && ch[1].kind == op_kind::mul &&
+                ch[1].children[0].kind == op_kind::constant &&
+                ch[1].children[1].kind == op_kind::hole) {
+                node_t prod;
+                prod.kind = op_kind::mul;
+                prod.dtype = ch[0].dtype;
+                prod.children = {ch[0], ch[1].children[0]};
+                value_t const v = eval_constant(prod);
+                node_t        r;
+                r.kind = op_kind::mul;
+                r.dtype = ch[0].dtype;
+                r.children = {make_const(ch[0].dtype, v.re, v.im), ch[1].children[1]};
+                return r;
+            }
+            return std::nullopt;
+        };
+        if (auto r = fold_pair()) return r.value();
+        if (is_const(ch[0], 1.0)) return ch[1];
+        if (is_const(ch[1], 1.0)) return ch[0];
+    }
+    if (n.kind == op_kind::power) {
+        if (n.power == 0.0) return make_const(dt, 1.0);
+        if (n.power == 1.0) return ch[0];
+    }
+    if (n.kind == op_kind::ite) {
+        if (same_node(ch[0], ch[1]) && self.compare == compare_t::eq) return ch[2];
+        if (same_node(ch[2], ch[3])) return ch[2];
+    }
+    if (n.kind == op_kind::conj && ch[0].kind == op_kind::conj) return ch[0].children[0];
+    return self;
+}
+
+node_t simplify_node(node_t const& n)
+{
+    node_t r0 = simplify_once(n);
+    if (same_node(r0, n)) return r0;
+    for (int guard = 0; guard != 1000; ++guard) {
+        node_t r1 = simplify_once(r0);
+        if (same_node(r0, r1)) return r1;
+        r0 = std::move(r1);
+    }
+    throw ir_error("simplify: no fixed point");
+}
+}  // namespace
+
+scalarop_t scalarop_t::simplify() const
+{
+    scalarop_t ret;
+    ret.root = simplify_node(root);
+    // a hole that folded away keeps its dtype: the einsummable still has that input
+    ret.hole_dtypes = hole_dtypes;
     return ret;
 }
 

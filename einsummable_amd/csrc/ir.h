@@ -83,6 +83,17 @@ struct scalarop_t {
     // einsummable.cc:221-233).  Variables not named stay.
     scalarop_t replace_variables(std::vector<std::pair<std::string, double>> const& values) const;
 
+    // The reference's canonical form (node_t::simplify, scalarop.cc:1233-1416, which every
+    // scalarop_t constructor applies, :1942-1948): a subtree without holes and variables
+    // becomes one constant -- evaluated in its dtype, printed with six significant digits and
+    // read back, as the reference does -- commutative operands and comparisons are ordered by
+    // the highest hole they use (normalize_order, :1442-1493, with its habit of turning
+    // ite_>[x,c,x,c] into ite_<=[c,x,c,x]), and 0 + x, 0 * x, 1 * x, c0 * (c1 * hole),
+    // x ^ 0, x ^ 1, ite with equal arms and conj(conj(x)) fold.  Repeated until nothing
+    // changes.  Texts the reference wrote are fixed points; what is not is a join whose
+    // variables have just been replaced by constants.
+    scalarop_t simplify() const;
+
     // `outer` with hole k replaced by the whole of `inner`, whose value passes through a
     // conversion to inner's own output dtype first (what a store by one kernel and a load by
     // the next do to it: a rounding for f16, nothing for the other dtypes, where the node

@@ -1,5 +1,9 @@
 #include "kernel_manager.h"
 
+#include <atomic>
+#include <exception>
+#include <thread>
+
 #include "launch.h"
 #include "static_workspace.h"
 
@@ -142,15 +146,76 @@ std::optional<uint64_t> kernel_manager_t::build(einsummable_t const& e_)
     auto          it = plans_.find(key);
     if (it != plans_.end()) return it->second->workspace_bytes;
 
+    std::shared_ptr<plan_t> p = make_plan(e);
+    if (!p) return std::nullopt;
+    plans_.emplace(key, p);
+    return p->workspace_bytes;
+}
+
+std::shared_ptr<plan_t> kernel_manager_t::make_plan(einsummable_t const& e) const
+{
     std::shared_ptr<plan_t> p = plan_contraction(e, device_);
     if (!p) p = plan_complex_contraction(e, device_);
     if (!p) p = plan_transpose(e, device_);
     if (!p) p = plan_staged_elementwise(e, device_);
     if (!p) p = plan_codegen(e, device_);
-    if (!p) return std::nullopt;
-    p->n_inns = int(e.inns.size());
-    plans_.emplace(key, p);
-    return p->workspace_bytes;
+    if (p) p->n_inns = int(e.inns.size());
+    return p;
+}
+
+std::vector<std::optional<uint64_t>> kernel_manager_t::build_many(
+    std::vector<einsummable_t> const& es)
+{
+    struct job_t {
+        einsummable_t           e;
+        std::string             key;
+        std::shared_ptr<plan_t> plan;
+        std::exception_ptr      error;
+    };
+    std::vector<job_t>       jobs;
+    std::vector<std::string> keys(es.size());
+    std::unordered_map<std::string, size_t> job_of;
+    for (size_t i = 0; i != es.size(); ++i) {
+        if (es[i].join.has_variables()) continue;  // build() answers nullopt
+        einsummable_t merged = es[i].merge_adjacent_dims();
+        keys[i] = merged.key();
+        if (plans_.count(keys[i]) || job_of.count(keys[i])) continue;
+        job_of.emplace(keys[i], jobs.size());
+        jobs.push_back(job_t{std::move(merged), keys[i], nullptr, nullptr});
+    }
+    if (!jobs.empty()) {
+        std::atomic<size_t> next{0};
+        auto work = [&]() {
+            // a thread of its own has no current device yet
+            if (hipSetDevice(device_) != hipSuccess) return;
+            for (size_t i = next++; i < jobs.size(); i = next++) {
+                try {
+                    jobs[i].plan = make_plan(jobs[i].e);
+                } catch (...) {
+                    jobs[i].error = std::current_exception();
+                }
+            }
+        };
+        // each generated kernel already compiles its two variants on two threads
+        size_t const hw = std::max(1u, std::thread::hardware_concurrency());
+        size_t const n_threads = std::min<size_t>({jobs.size(), 8, std::max<size_t>(hw / 2, 1)});
+        std::vector<std::thread> pool;
+        for (size_t t = 1; t < n_threads; ++t) pool.emplace_back(work);
+        work();
+        for (std::thread& t : pool) t.join();
+        // entered (and errors raised) in list order, as a loop over build() would
+        for (job_t& j : jobs) {
+            if (j.error) std::rethrow_exception(j.error);
+            if (j.plan) plans_.emplace(j.key, j.plan);
+        }
+    }
+    std::vector<std::optional<uint64_t>> ret(es.size());
+    for (size_t i = 0; i != es.size(); ++i) {
+        if (keys[i].empty()) continue;
+        auto it = plans_.find(keys[i]);
+        if (it != plans_.end()) ret[i] = it->second->workspace_bytes;
+    }
+    return ret;
 }
 
 uint64_t kernel_manager_t::workspace_size(einsummable_t const& e) const

@@ -49,6 +49,11 @@ public:
     ~kernel_manager_t();
 
     std::optional<uint64_t> build(einsummable_t const& e);
+    // build() for a list: the einsummables not yet planned are planned on several threads
+    // (runtime compilation of the generated kernels is nearly all of a cold build) and
+    // entered into the map by the calling thread.  Same results and same error contract as
+    // build() called for each in turn; like build(), not to be called concurrently.
+    std::vector<std::optional<uint64_t>> build_many(std::vector<einsummable_t> const& es);
     uint64_t                workspace_size(einsummable_t const& e) const;
     std::string             describe(einsummable_t const& e) const;
 
@@ -84,6 +89,8 @@ public:
 
 private:
     plan_t const* find(einsummable_t const& merged) const;
+    // the planners in their order; null when none takes it.  Touches no member.
+    std::shared_ptr<plan_t> make_plan(einsummable_t const& merged) const;
 
     int                                                      device_;
     std::unordered_map<std::string, std::shared_ptr<plan_t>> plans_;      // by merged key

@@ -584,7 +584,10 @@ void memgraph_t::populate(apply_graph_t& g, int loc,
                         throw ir_error(where("only allowing touches to have a group"));
                     }
                     mg_einsummable_t const& m = *n.einsummable;
-                    scalarop_t join = scalarop_t::parse(m.join).replace_variables(vars);
+                    // as einsummable_t::replace_scalar_variables does (einsummable.cc:220-233):
+                    // the new join is a scalarop_t built from a node, i.e. simplified
+                    scalarop_t join = scalarop_t::parse(m.join);
+                    if (join.has_variables()) join = join.replace_variables(vars).simplify();
                     einsummable_t e = einsummable_t::make(m.join_shape, m.inns, m.out_rank, join,
                                                           read_castable(m.castable));
                     g.add_einsummable(e, n.mems, n.inns);

@@ -25,6 +25,7 @@ EXPORTS = [
     "es_km_fill_lowertri",
     "es_km_codegen_source",
     "es_km_scalarop_roundtrip",
+    "es_km_scalarop_simplify",
     "es_km_merge_adjacent_dims",
     "es_km_probe_mfma_f16",
     "es_km_graph_create",
@@ -354,6 +355,22 @@ def scalarop_roundtrip(text):
     if rc != OK:
         raise KmError(rc, lib.es_km_last_error(None).decode("utf-8", "replace"))
     return buf.value.decode("utf-8", "replace"), od.value, n.value
+
+
+def scalarop_simplify(text, variables=None):
+    """The reference's canonical form of a scalarop text, after replacing the named variables
+    (a dict name -> value) by constants."""
+    lib = load_library()
+    items = sorted((variables or {}).items())
+    names = (ctypes.c_char_p * max(len(items), 1))(*[k.encode() for k, _ in items])
+    vals = (ctypes.c_double * max(len(items), 1))(*[float(v) for _, v in items])
+    buf = ctypes.create_string_buffer(1 << 14)
+    lib.es_km_scalarop_simplify.argtypes = [ctypes.c_char_p, ctypes.c_void_p, ctypes.c_void_p,
+                                            ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t]
+    rc = lib.es_km_scalarop_simplify(text.encode(), names, vals, len(items), buf, len(buf))
+    if rc != OK:
+        raise KmError(rc, lib.es_km_last_error(None).decode("utf-8", "replace"))
+    return buf.value.decode()
 
 
 def merge_adjacent_dims(e):

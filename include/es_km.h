@@ -154,6 +154,13 @@ int es_km_codegen_source(const uint64_t* join_shape, int join_rank, const int* i
  *   negative error.  Output arrays must hold join_rank / the input's mode count entries. */
 int es_km_scalarop_roundtrip(const char* text, char* out, size_t cap, int* out_dtype,
                              int* n_inputs);
+/* es_km_scalarop_simplify: parse, replace the n_vars named variables by constants
+ *   (scalarop_t::replace_variables; n_vars may be 0), bring the expression to the reference's
+ *   canonical form (node_t::simplify, scalarop.cc:1233-1416, applied by every scalarop_t
+ *   constructor, :1942-1948) and print it.  What es_km_graph_load_memgraph does to a join
+ *   that carries variables (gpu/exec_graph.cc:106-108). */
+int es_km_scalarop_simplify(const char* text, const char* const* var_names,
+                            const double* var_values, int n_vars, char* out, size_t cap);
 int es_km_merge_adjacent_dims(const uint64_t* join_shape, int join_rank, const int* inns_flat,
                               const int* inns_offsets, int n_inns, int out_rank,
                               const char* join_text, char castable, uint64_t* new_join_shape,

@@ -57,6 +57,45 @@ SIMPLIFY_INPUTS = [
     "+[constant{f32|0},hole|f32@0]",
     "*[constant{f32|1},hole|f32@0]",
 ]
+# joins as they stand right after their variables were replaced by constants (what
+# einsummable_t::replace_scalar_variables hands to the scalarop_t constructor), and forms
+# that exercise every rule of simplify_once / normalize_order
+SIMPLIFY_INPUTS += [
+    "*[*[constant{f32|-1},constant{f32|0.25}],hole|f32@0]",
+    "+[hole|f32@0,*[*[constant{f32|-1},constant{f32|0.001}],hole|f32@1]]",
+    "+[*[constant{f32|0.9},hole|f32@0],*[+[constant{f32|1},*[constant{f32|-1},constant{f32|0.9}]],hole|f32@1]]",
+    "*[constant{f32|0.333333},*[constant{f32|0.142857},hole|f32@0]]",
+    "*[constant{f16|0.333252},*[constant{f16|0.142822},hole|f16@0]]",
+    "*[constant{f64|0.333333},*[constant{f64|0.142857},hole|f64@0]]",
+    "*[hole|f32@1,hole|f32@0]",
+    "*[hole|f32@0,constant{f32|0}]",
+    "+[hole|f32@0,constant{f32|INF}]",
+    "+[constant{f32|NINF},hole|f32@0]",
+    "power{0}[hole|f32@0]",
+    "power{1}[exp[hole|f32@0]]",
+    "power{-0.5}[constant{f32|2}]",
+    "power{2}[constant{f16|1.5}]",
+    "exp[constant{f32|1}]",
+    "exp[constant{f16|1}]",
+    "log[constant{f64|10}]",
+    "to_f16[constant{f32|0.1}]",
+    "to_f32[*[constant{f16|0.1},constant{f16|3}]]",
+    "ite_<[constant{f32|1},constant{f32|2},hole|f32@0,hole|f32@1]",
+    "ite_==[hole|f32@0,hole|f32@0,hole|f32@1,constant{f32|7}]",
+    "ite_<[hole|f32@0,hole|f32@1,hole|f32@2,hole|f32@2]",
+    "ite_<[hole|f32@1,hole|f32@0,constant{f32|1},constant{f32|0}]",
+    "ite_>=[hole|f32@1,hole|f32@0,hole|f32@1,hole|f32@0]",
+    "ite_<=[hole|f32@0,constant{f32|0},constant{f32|0},hole|f32@0]",
+    "conj[conj[hole|c64@0]]",
+    "*[constant{c64|(1,0)},hole|c64@0]",
+    "*[constant{c64|(0,1)},constant{c64|(0,1)}]",
+    "+[real[hole|c64@0],*[constant{f32|2},constant{f32|0.5}]]",
+    "complex[constant{f32|1},constant{f32|2}]",
+    "*[+[constant{f32|1},constant{f32|-1}],hole|f32@0]",
+    "+[*[constant{f32|1},hole|f32@1],*[hole|f32@0,constant{f32|1}]]",
+    "*[hole|f16@0,power{-1}[+[constant{f16|1},exp[*[constant{f16|-1},hole|f16@0]]]]]",
+    "exp[*[constant{f32|0.0883883},+[hole|f32@0,*[constant{f32|-1},hole|f32@1]]]]",
+]
 out["simplify"] = {t: oracle.ref_scalarop_simplify(t) for t in SIMPLIFY_INPUTS}
 
 # 4. eval at sampled points, bit patterns in and out

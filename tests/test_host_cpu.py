@@ -529,3 +529,74 @@ def test_exec_graph_optimize_on_the_reference_memgraph_layout():
     assert g.optimize() > 10           # fewer than with private ranges: a reused range is often still read
     assert mp.unordered_conflicts(g) == []
     g.finalize(4)
+
+
+def _random_scalarop(r, dt, depth):
+    """A random well-typed real scalarop text over holes 0..2 and a few constants."""
+    consts = ["0", "1", "-1", "0.5", "2", "3", "0.333333", "INF", "NINF", "1e-06"]
+    if depth == 0 or r.rand() < 0.25:
+        if r.rand() < 0.5:
+            return "hole|%s@%d" % (dt, r.randint(0, 3))
+        return "constant{%s|%s}" % (dt, consts[r.randint(0, len(consts))])
+    k = r.randint(0, 7)
+    sub = lambda: _random_scalarop(r, dt, depth - 1)
+    if k == 0:
+        return "+[%s,%s]" % (sub(), sub())
+    if k == 1:
+        return "*[%s,%s]" % (sub(), sub())
+    if k == 2:
+        return "exp[%s]" % sub()
+    if k == 3:
+        return "power{%s}[%s]" % (["0", "1", "2", "-1", "0.5", "-0.5"][r.randint(0, 6)], sub())
+    if k == 4:
+        return "ite_%s[%s,%s,%s,%s]" % (["<", ">", "==", "<=", ">="][r.randint(0, 5)],
+                                        sub(), sub(), sub(), sub())
+    if k == 5:
+        other = {"f16": "f32", "f32": "f64", "f64": "f32"}[dt]
+        return "to_%s[%s]" % (dt, _random_scalarop(r, other, depth - 1))
+    return "log[%s]" % sub()
+
+
+def test_scalarop_simplify_matches_the_reference():
+    """The library's simplify() against the reference's: on the committed vectors (written
+    from the compiled reference by tests/golden/make_golden.py) and, where the reference
+    build is present, on random expressions."""
+    import json
+    import os
+
+    import numpy as np
+
+    import einsummable_amd as ea
+    import oracle
+
+    here = os.path.dirname(os.path.abspath(__file__))
+    golden = json.load(open(os.path.join(here, "golden", "scalarop_golden.json")))["simplify"]
+    assert len(golden) >= 50
+    for src, want in golden.items():
+        assert ea.scalarop_simplify(src) == want, src
+        assert ea.scalarop_simplify(want) == want, want        # a fixed point
+    # variables become constants first: the learning-rate update of the reference's trainer
+    upd = "+[hole|f32@0,*[*[constant{f32|-1},variable{lr|f32}],hole|f32@1]]"
+    assert ea.scalarop_simplify(upd, {"lr": 0.001}) == \
+        golden["+[hole|f32@0,*[*[constant{f32|-1},constant{f32|0.001}],hole|f32@1]]"]
+    assert ea.scalarop_simplify(upd) == upd                    # an unnamed variable stays
+    if not oracle.ref_available():
+        return
+    r = np.random.RandomState(11)
+    n = 0
+    for _ in range(3000):
+        dt = ["f32", "f64", "f16"][r.randint(0, 3)]
+        text = _random_scalarop(r, dt, 4)
+        try:
+            want = oracle.ref_scalarop_simplify(text)
+        except oracle.OracleError:
+            continue
+        try:
+            got = ea.scalarop_simplify(text)
+        except ea.KmError as err:
+            # the generator may use one hole with two dtypes, which this parser refuses
+            assert "two dtypes" in str(err), text
+            continue
+        assert got == want, text
+        n += 1
+    assert n > 1000
