@@ -47,8 +47,8 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="all",
-                    choices=["c2", "c1", "c3", "c4", "c5", "llama", "copy", "mfma_peak", "build",
-                             "colred", "all"])
+                    choices=["c2", "c1", "c3", "c4", "c5", "c5opt", "llama", "copy", "mfma_peak",
+                             "build", "colred", "all"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     return ap.parse_args()
 
@@ -767,7 +767,7 @@ def run_c5(km, steps, warmup):
     # the same layer through the exec-node layer: one arena, dependencies from the memory
     # ranges, nodes placed on 1 / 2 / 4 streams, one burst of launches per layer
     del graph
-    exec_ms, opt_ms, opt_launches = {}, {}, {}
+    exec_ms, opt_ms, opt_launches, per_launch = {}, {}, {}, []
     state = {name: run.mem[name].clone() for name in g.inputs}
     for ns, optimize in ((1, False), (2, False), (4, False), (1, True), (4, True)):
         del run
@@ -787,6 +787,8 @@ def run_c5(km, steps, warmup):
         (opt_ms if optimize else exec_ms)[str(ns)] = round(
             (time.perf_counter() - t0) / steps * 1e3, 4)
         opt_launches["optimized" if optimize else "as_listed"] = par.graph.launches()
+        if optimize and ns == 1:
+            per_launch = time_graph_nodes(par, max(steps // 2, 5))
         run = par
     del par, run, state
     rows = []
@@ -801,11 +803,100 @@ def run_c5(km, steps, warmup):
             # readers; every range still written holds the same bytes
             "layer_exec_graph_optimized_ms_by_streams": opt_ms,
             "exec_graph_launches": opt_launches,
+            # the optimised layer launch by launch (es_km_graph_launch_node with an event pair
+            # around each): what it moves or multiplies and the fraction of the bound that
+            # applies; the launches' sum against the burst above is the launch gaps
+            "optimized_launches": per_launch,
+            "optimized_launches_sum_ms": round(sum(r["ms"] for r in per_launch), 4),
             "layer_with_node_events_ms": round(timed_wall_ms, 4), "nodes": len(rows), "sum_node_ms": round(sum(r[2] for r in rows), 4),
             "contraction_ms": round(gemm_ms, 4),
             "contraction_TFLOPs": round(g.contraction_flops() / gemm_ms / 1e9, 1),
             "other_ms": round(sum(r[2] for r in rows) - gemm_ms, 4),
             "top_nodes": [{"label": l, "ms": round(ms, 4)} for l, _, ms, _ in top]}
+
+
+def time_graph_nodes(runner, steps):
+    """Every launching node of an ArenaRunner's graph, one at a time through
+    es_km_graph_launch_node, timed with an event pair."""
+    import torch
+
+    g = runner.graph
+    stream = torch.cuda.current_stream().cuda_stream
+    ids = [i for i in range(g.num_nodes()) if g.node_mems(i)[0] != "dummy"]
+    ws_bytes = max([g.node_workspace(i) for i in ids] + [1])
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
+    arena = runner.arena.data_ptr()
+    timers = {i: Timed() for i in ids}
+
+    def one_pass(timed):
+        for i in ids:
+            call = lambda i=i: g.launch_node(i, stream, arena, (ws.data_ptr(), ws_bytes))
+            if timed:
+                timers[i].record(call)
+            else:
+                call()
+
+    for _ in range(3):
+        one_pass(False)
+    for _ in range(steps):
+        one_pass(True)
+    torch.cuda.synchronize()
+    rows = []
+    for i in ids:
+        kind, mems = g.node_mems(i)
+        text = g.describe(i)
+        ms = timers[i].mean_ms()
+        nbytes = sum(size for _, size in mems)
+        row = {"node": text.split(" | ", 1)[1] if " | " in text else kind, "kind": kind,
+               "ms": round(ms, 5), "bytes": nbytes}
+        flop = 0
+        if kind == "einsummable":
+            key = text.split(" | ")[1]
+            shape = [int(x) for x in key[key.index("[") + 1:key.index("]")].split(",")]
+            join = text.split(" | ")[2]
+            product = join.count("hole|") == 2 and join.startswith("*[") and "+[" not in join
+            if key[key.index("]") + 1] == "+" and product:
+                flop = 2
+                for d in shape:
+                    flop *= d
+        intensity = flop / max(nbytes, 1)
+        if flop and intensity >= 150:
+            row.update(flop=flop, bound="mfma",
+                       frac=round(flop / ms / 1e9 / PEAK_TFLOPS["f16"], 4))
+        else:
+            if flop:
+                row["flop"] = flop
+            row.update(bound="hbm", frac=round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4))
+        rows.append(row)
+    return rows
+
+
+def run_c5opt(km, steps, warmup):
+    """The optimised LLaMA-7B layer alone (for a kernel trace of exactly its launches)."""
+    import numpy as np
+    import torch
+
+    from einsummable_amd.llama_layer import ArenaRunner, LayerGraph, freqs_cis_table
+
+    g = LayerGraph()
+    par = ArenaRunner(km, g, 1, optimize=True)
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    for name, (dt, shape) in g.inputs.items():
+        n = int(np.prod(shape))
+        if name == "full_freqs_cis":
+            par.set_input(name, freqs_cis_table(shape[0], shape[1]))
+            continue
+        t = torch.randn(n, device="cuda", dtype=torch.float32, generator=gen) * (1.0 if name == "x" else 0.02)
+        if name.endswith("norm.weight"):
+            t = t + 1.0
+        par.view(name).copy_(t.half().view(torch.uint8))
+    warm(par.run, max(warmup, 2))
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        par.run()
+    torch.cuda.synchronize()
+    return {"node": "c5 optimised layer, one stream", "launches": par.graph.launches(),
+            "layer_ms": round((time.perf_counter() - t0) / steps * 1e3, 4)}
 
 
 def run_mfma_peak(km):
@@ -982,13 +1073,26 @@ def targets_block(others):
     line cannot be read as its headline alone."""
     mfma, hbm = [], []
     for r in others.get("llama7b_contractions", []):
-        if "mfma_frac" in r and ("proj" in r["node"] or "w1" in r["node"] or "w2" in r["node"] or
-                                 "^3" in r["node"]):
+        if "mfma_frac" not in r:
+            continue
+        # arithmetic intensity below 150 flop per byte (attention's scores and values): the
+        # HBM bound applies (the planner's own rule for giving a product the small tile)
+        nbytes = r["hbm_frac"] * HBM_PEAK_GBPS * 1e6 * r["ms"]
+        if r["flop"] / max(nbytes, 1.0) < 150.0:
+            hbm.append((r["hbm_frac"], r["node"]))
+        else:
             mfma.append((r["mfma_frac"], r["node"], r.get("torch_matmul_TFLOPs")))
     for key in ("c2_nodes", "c3", "c4", "column_reductions"):
         for r in others.get(key, []):
             if isinstance(r, dict) and "hbm_frac" in r and "[not part" not in r["node"]:
                 hbm.append((r["hbm_frac"], r["node"]))
+    for r in others.get("c5", {}).get("optimized_launches", []):
+        label = "c5 optimised layer: " + r["node"][:90]
+        if r["bound"] == "mfma":
+            mfma.append((r["frac"], label, None))
+        elif r["bytes"] >= (8 << 20):
+            # (a node that moves less than 8 MiB is bound by its launch, not by memory)
+            hbm.append((r["frac"], label))
     mfma.sort()
     hbm.sort()
     out = {
@@ -1028,6 +1132,10 @@ def main():
         return
     if args.workload == "copy":
         print(json.dumps(run_copy(km, args.steps, args.warmup)))
+        return
+    if args.workload == "c5opt":
+        # nothing but the optimised layer: a kernel trace of this run lists its launches only
+        print(json.dumps(run_c5opt(km, args.steps, args.warmup)))
         return
 
     c2 = run_c2(km, args.steps, args.warmup)

@@ -11,6 +11,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <future>
+#include <set>
 #include <map>
 #include <mutex>
 #include <sstream>
@@ -1321,9 +1322,13 @@ namespace
 
 // Loaded modules of this process, one per (device, source): a module belongs to the device
 // that was current when it was loaded.
+struct loaded_t {
+    hipModule_t mod;
+    std::string suffix;  // appended to the source's entry points (programs compiled together)
+};
 struct module_cache_t {
-    std::mutex                                              mu;
-    std::map<std::pair<int, std::string>, hipModule_t> by_source;
+    std::mutex                                      mu;
+    std::map<std::pair<int, std::string>, loaded_t> by_source;
 };
 
 module_cache_t& module_cache()
@@ -1353,9 +1358,11 @@ void load_kernel(variant_t& v, int device, std::vector<char> const& code)
     auto&                       cache = module_cache();
     std::lock_guard<std::mutex> lock(cache.mu);
     hipModule_t                 mod;
+    std::string                 suffix;
     auto                        it = cache.by_source.find({device, v.k.source});
     if (it != cache.by_source.end()) {
-        mod = it->second;
+        mod = it->second.mod;
+        suffix = it->second.suffix;
     } else {
         std::vector<char> compiled;
         if (code.empty()) compiled = code_object_for(v.k.source, nullptr);
@@ -1364,9 +1371,10 @@ void load_kernel(variant_t& v, int device, std::vector<char> const& code)
             throw km_error(km_status::device,
                            std::string("hipModuleLoadData: ") + hipGetErrorString(err));
         }
-        cache.by_source.emplace(std::make_pair(device, v.k.source), mod);
+        cache.by_source.emplace(std::make_pair(device, v.k.source), loaded_t{mod, ""});
     }
-    auto get = [&](std::string const& name) {
+    auto get = [&](std::string const& base) {
+        std::string const name = base + suffix;
         hipFunction_t fn;
         hipError_t    err = hipModuleGetFunction(&fn, mod, name.c_str());
         if (err != hipSuccess) {
@@ -1385,6 +1393,11 @@ struct codegen_plan_t : plan_t {
     variant_t         narrow;  // scalar accesses: for buffers that are not 16-byte aligned
 
     explicit codegen_plan_t(einsummable_t const& e_) : e(e_) {}
+    bool waiting = false;  // the variants' kernels are not loaded yet
+    void deferred(std::vector<plan_t*>& out) override
+    {
+        if (waiting) out.push_back(this);
+    }
 
     static void launch(variant_t const& v, hipStream_t stream, void* out, void const* const* inns,
                        void* workspace)
@@ -1465,7 +1478,7 @@ struct codegen_plan_t : plan_t {
 
 }  // namespace
 
-std::shared_ptr<plan_t> plan_codegen(einsummable_t const& e, int device)
+std::shared_ptr<plan_t> plan_codegen(einsummable_t const& e, int device, bool defer)
 {
     cg_kernel_t k;
     try {
@@ -1478,22 +1491,14 @@ std::shared_ptr<plan_t> plan_codegen(einsummable_t const& e, int device)
     auto p = std::make_shared<codegen_plan_t>(e);
     p->wide.k = std::move(k);
     p->narrow.k = generate_kernel(e, 1);
-    // Both variants are compiled and loaded here, the scalar one on a second thread while
-    // this one compiles the wide one: run() only ever launches.
-    std::future<std::vector<char>> narrow_code;
-    bool const narrow_distinct = p->narrow.k.source != p->wide.k.source;
-    if (narrow_distinct && !module_loaded(device, p->narrow.k.source)) {
-        narrow_code = std::async(std::launch::async, [src = p->narrow.k.source]() {
-            return code_object_for(src, nullptr);
-        });
-    }
-    try {
+    // Both variants are compiled and loaded at build time -- here, or with the other
+    // kernels of the caller's list (finish_codegen_plans): run() only ever launches.
+    if (defer) {
+        p->waiting = true;
+    } else {
         load_kernel(p->wide, device, {});
-    } catch (...) {
-        if (narrow_code.valid()) narrow_code.wait();
-        throw;
+        load_kernel(p->narrow, device, {});
     }
-    load_kernel(p->narrow, device, narrow_code.valid() ? narrow_code.get() : std::vector<char>());
     switch (p->wide.k.kind) {
         case cg_kind::elementwise:
             p->description = "elementwise";
@@ -1511,6 +1516,72 @@ std::shared_ptr<plan_t> plan_codegen(einsummable_t const& e, int device)
     if (p->wide.k.splits > 1) p->description += " splits=" + std::to_string(p->wide.k.splits);
     p->workspace_bytes = std::max(p->wide.k.ws_bytes, p->narrow.k.ws_bytes);
     return p;
+}
+
+void finish_codegen_plans(std::vector<plan_t*> const& plans, int device)
+{
+    std::vector<codegen_plan_t*> ps;
+    for (plan_t* p : plans) {
+        if (auto* c = dynamic_cast<codegen_plan_t*>(p)) ps.push_back(c);
+    }
+    if (ps.empty()) return;
+    // the distinct sources that no module of this device holds yet, in order of appearance
+    std::vector<variant_t*> fresh;
+    {
+        std::set<std::string> seen;
+        for (codegen_plan_t* p : ps) {
+            for (variant_t* v : {&p->wide, &p->narrow}) {
+                if (seen.count(v->k.source) || module_loaded(device, v->k.source)) continue;
+                seen.insert(v->k.source);
+                fresh.push_back(v);
+            }
+        }
+    }
+    if (fresh.size() > 1) {
+        // One program: the prelude once, every kernel's own text (its join function, argument
+        // block and entry points share their names with the others') in a namespace of its
+        // own, the entry points, which have C linkage, told apart by a suffix.
+        size_t const pre = std::strlen(PRELUDE);
+        std::string  text = PRELUDE;
+        for (size_t i = 0; i != fresh.size(); ++i) {
+            cg_kernel_t const& k = fresh[i]->k;
+            if (k.source.compare(0, pre, PRELUDE) != 0) {
+                throw km_error(km_status::invalid, "generated source without its prelude");
+            }
+            std::string       body = k.source.substr(pre);
+            std::string const suffix = "_u" + std::to_string(i);
+            for (std::string const& name : {k.entry, k.splits > 1 ? k.entry2 : std::string()}) {
+                if (name.empty()) continue;
+                std::string const from = name + "(";
+                size_t            hits = 0;
+                for (size_t at = body.find(from); at != std::string::npos;
+                     at = body.find(from, at + from.size() + suffix.size())) {
+                    body.insert(at + name.size(), suffix);
+                    ++hits;
+                }
+                if (hits == 0) throw km_error(km_status::invalid, "entry point not found: " + name);
+            }
+            text += "namespace es_unit_" + std::to_string(i) + "\n{\n" + body + "\n}\n";
+        }
+        std::vector<char> const code = code_object_for(text, nullptr);
+        hipModule_t             mod;
+        hipError_t              err = hipModuleLoadData(&mod, code.data());
+        if (err != hipSuccess) {
+            throw km_error(km_status::device,
+                           std::string("hipModuleLoadData: ") + hipGetErrorString(err));
+        }
+        auto&                       cache = module_cache();
+        std::lock_guard<std::mutex> lock(cache.mu);
+        for (size_t i = 0; i != fresh.size(); ++i) {
+            cache.by_source.emplace(std::make_pair(device, fresh[i]->k.source),
+                                    loaded_t{mod, "_u" + std::to_string(i)});
+        }
+    }
+    for (codegen_plan_t* p : ps) {
+        load_kernel(p->wide, device, {});
+        load_kernel(p->narrow, device, {});
+        p->waiting = false;
+    }
 }
 
 }  // namespace es

@@ -1,9 +1,5 @@
 #include "kernel_manager.h"
 
-#include <atomic>
-#include <exception>
-#include <thread>
-
 #include "launch.h"
 #include "static_workspace.h"
 
@@ -54,9 +50,10 @@ struct staged_plan_t : plan_t {
         main->run(stream, out, ptrs.data(), main->workspace_bytes ? ws + main_offset : nullptr,
                   main->workspace_bytes);
     }
+    void deferred(std::vector<plan_t*>& out) override { main->deferred(out); }
 };
 
-std::shared_ptr<plan_t> plan_staged_elementwise(einsummable_t const& e, int device)
+std::shared_ptr<plan_t> plan_staged_elementwise(einsummable_t const& e, int device, bool defer = false)
 {
     if (e.has_aggregation()) return nullptr;
     int const R = int(e.join_shape.size());
@@ -102,7 +99,7 @@ std::shared_ptr<plan_t> plan_staged_elementwise(einsummable_t const& e, int devi
     }
     if (plan->stages.empty()) return nullptr;
     main = main.merge_adjacent_dims();
-    plan->main = plan_codegen(main, device);
+    plan->main = plan_codegen(main, device, defer);
     if (!plan->main) return nullptr;
     plan->main->n_inns = int(main.inns.size());
     plan->main_offset = offset;
@@ -152,13 +149,13 @@ std::optional<uint64_t> kernel_manager_t::build(einsummable_t const& e_)
     return p->workspace_bytes;
 }
 
-std::shared_ptr<plan_t> kernel_manager_t::make_plan(einsummable_t const& e) const
+std::shared_ptr<plan_t> kernel_manager_t::make_plan(einsummable_t const& e, bool defer) const
 {
     std::shared_ptr<plan_t> p = plan_contraction(e, device_);
     if (!p) p = plan_complex_contraction(e, device_);
     if (!p) p = plan_transpose(e, device_);
-    if (!p) p = plan_staged_elementwise(e, device_);
-    if (!p) p = plan_codegen(e, device_);
+    if (!p) p = plan_staged_elementwise(e, device_, defer);
+    if (!p) p = plan_codegen(e, device_, defer);
     if (p) p->n_inns = int(e.inns.size());
     return p;
 }
@@ -166,48 +163,24 @@ std::shared_ptr<plan_t> kernel_manager_t::make_plan(einsummable_t const& e) cons
 std::vector<std::optional<uint64_t>> kernel_manager_t::build_many(
     std::vector<einsummable_t> const& es)
 {
-    struct job_t {
-        einsummable_t           e;
-        std::string             key;
-        std::shared_ptr<plan_t> plan;
-        std::exception_ptr      error;
-    };
-    std::vector<job_t>       jobs;
-    std::vector<std::string> keys(es.size());
-    std::unordered_map<std::string, size_t> job_of;
+    std::vector<std::string>                                 keys(es.size());
+    std::vector<std::pair<std::string, std::shared_ptr<plan_t>>> fresh;
+    std::unordered_map<std::string, size_t>                  seen;
     for (size_t i = 0; i != es.size(); ++i) {
         if (es[i].join.has_variables()) continue;  // build() answers nullopt
         einsummable_t merged = es[i].merge_adjacent_dims();
         keys[i] = merged.key();
-        if (plans_.count(keys[i]) || job_of.count(keys[i])) continue;
-        job_of.emplace(keys[i], jobs.size());
-        jobs.push_back(job_t{std::move(merged), keys[i], nullptr, nullptr});
+        if (plans_.count(keys[i]) || seen.count(keys[i])) continue;
+        seen.emplace(keys[i], fresh.size());
+        fresh.emplace_back(keys[i], make_plan(merged, true));
     }
-    if (!jobs.empty()) {
-        std::atomic<size_t> next{0};
-        auto work = [&]() {
-            // a thread of its own has no current device yet
-            if (hipSetDevice(device_) != hipSuccess) return;
-            for (size_t i = next++; i < jobs.size(); i = next++) {
-                try {
-                    jobs[i].plan = make_plan(jobs[i].e);
-                } catch (...) {
-                    jobs[i].error = std::current_exception();
-                }
-            }
-        };
-        // each generated kernel already compiles its two variants on two threads
-        size_t const hw = std::max(1u, std::thread::hardware_concurrency());
-        size_t const n_threads = std::min<size_t>({jobs.size(), 8, std::max<size_t>(hw / 2, 1)});
-        std::vector<std::thread> pool;
-        for (size_t t = 1; t < n_threads; ++t) pool.emplace_back(work);
-        work();
-        for (std::thread& t : pool) t.join();
-        // entered (and errors raised) in list order, as a loop over build() would
-        for (job_t& j : jobs) {
-            if (j.error) std::rethrow_exception(j.error);
-            if (j.plan) plans_.emplace(j.key, j.plan);
-        }
+    std::vector<plan_t*> waiting;
+    for (auto const& kp : fresh) {
+        if (kp.second) kp.second->deferred(waiting);
+    }
+    finish_codegen_plans(waiting, device_);
+    for (auto& kp : fresh) {
+        if (kp.second) plans_.emplace(kp.first, std::move(kp.second));
     }
     std::vector<std::optional<uint64_t>> ret(es.size());
     for (size_t i = 0; i != es.size(); ++i) {

@@ -40,6 +40,9 @@ struct plan_t {
     uint64_t    workspace_bytes = 0;
     int         n_inns = 0;
     std::string description;
+    // Plans whose generated kernels were planned without being compiled (plan_codegen with
+    // `defer`) add themselves: finish_codegen_plans compiles and loads them together.
+    virtual void deferred(std::vector<plan_t*>&) {}
 };
 
 class kernel_manager_t
@@ -49,10 +52,11 @@ public:
     ~kernel_manager_t();
 
     std::optional<uint64_t> build(einsummable_t const& e);
-    // build() for a list: the einsummables not yet planned are planned on several threads
-    // (runtime compilation of the generated kernels is nearly all of a cold build) and
-    // entered into the map by the calling thread.  Same results and same error contract as
-    // build() called for each in turn; like build(), not to be called concurrently.
+    // build() for a list: the generated kernels of the einsummables not yet planned are
+    // compiled together, as one program (runtime compilation is nearly all of a cold build,
+    // and nearly all of it is the compiler's fixed cost per program).  Same results and same
+    // error contract as build() called for each in turn; like build(), not to be called
+    // concurrently.
     std::vector<std::optional<uint64_t>> build_many(std::vector<einsummable_t> const& es);
     uint64_t                workspace_size(einsummable_t const& e) const;
     std::string             describe(einsummable_t const& e) const;
@@ -90,7 +94,7 @@ public:
 private:
     plan_t const* find(einsummable_t const& merged) const;
     // the planners in their order; null when none takes it.  Touches no member.
-    std::shared_ptr<plan_t> make_plan(einsummable_t const& merged) const;
+    std::shared_ptr<plan_t> make_plan(einsummable_t const& merged, bool defer = false) const;
 
     int                                                      device_;
     std::unordered_map<std::string, std::shared_ptr<plan_t>> plans_;      // by merged key
@@ -102,6 +106,13 @@ private:
 std::shared_ptr<plan_t> plan_contraction(einsummable_t const& e, int device);
 std::shared_ptr<plan_t> plan_complex_contraction(einsummable_t const& e, int device);
 std::shared_ptr<plan_t> plan_transpose(einsummable_t const& e, int device);
-std::shared_ptr<plan_t> plan_codegen(einsummable_t const& e, int device);
+// `defer`: generate the kernels' source only; finish_codegen_plans compiles and loads
+std::shared_ptr<plan_t> plan_codegen(einsummable_t const& e, int device, bool defer = false);
+// Compiles the generated kernels of all these plans as ONE runtime-compiled program (the
+// compiler's fixed cost per program is most of the time of a small kernel, and it compiles
+// one program at a time whatever the number of calling threads: the 25 distinct generated
+// kernels of a LLaMA layer take 9.3 s one by one and 0.8 s as one program on the same
+// machine) and loads the module on `device`.
+void finish_codegen_plans(std::vector<plan_t*> const& plans, int device);
 
 }  // namespace es
