@@ -1161,6 +1161,14 @@ bool is_row_reduction(einsummable_t const& e)
     return false;
 }
 
+// The options every generated kernel is compiled with; the on-disk cache keys on this very
+// list.
+std::vector<std::string> compile_options(std::string const& arch)
+{
+    return {"--offload-arch=" + arch, "-O3",     "-std=c++17",       "-Xclang",
+            "-target-feature",        "-Xclang", "-packed-fp32-ops", "-ffp-contract=off"};
+}
+
 std::vector<char> compile_hip_source(std::string const& source, std::string const& name,
                                      std::string const& arch)
 {
@@ -1169,17 +1177,17 @@ std::vector<char> compile_hip_source(std::string const& source, std::string cons
         HIPRTC_SUCCESS) {
         throw km_error(km_status::device, "hiprtcCreateProgram failed");
     }
-    std::string arch_opt = "--offload-arch=" + arch;
     // packed-fp32 instruction selection is switched off for all device code of this library.
     // No contraction of a product and a sum into a fused multiply-add: every node of a join
     // rounds by itself, as the reference's interpreter does, and -- what matters when the
     // exec graph merges two einsummables into one kernel -- the same expression gives the same
     // bits in whatever kernel it ends up (left to the compiler, 1.7 * x + y became an FMA in
     // a kernel of its own and a product and a sum inside a larger join).
-    const char* opts[] = {arch_opt.c_str(), "-O3",      "-std=c++17",       "-Xclang",
-                          "-target-feature", "-Xclang", "-packed-fp32-ops", "-ffp-contract=off"};
-    int         n_opts = 8;
-    hiprtcResult rc = hiprtcCompileProgram(prog, n_opts, opts);
+    std::vector<std::string> const options = compile_options(arch);
+    std::vector<const char*>       opts;
+    for (std::string const& o : options) opts.push_back(o.c_str());
+    int const n_opts = int(opts.size());
+    hiprtcResult rc = hiprtcCompileProgram(prog, n_opts, opts.data());
     if (rc != HIPRTC_SUCCESS) {
         size_t n = 0;
         hiprtcGetProgramLogSize(prog, &n);
@@ -1205,12 +1213,10 @@ namespace
 // ---- code objects on disk.  A runtime compile costs a good part of a second per kernel, and
 // a server process builds the same einsummables every time it starts.  The code object of a
 // source is kept in a file named by a 128-bit hash of (runtime-compiler version, options,
-// source); the file repeats the length of that text so that a truncated or foreign file is not
-// taken for a hit.  ES_KM_CACHE_DIR names the directory ("off" or "" switches the cache off);
+// source); the file holds that whole text in front of the code object and a hit is one whose
+// text is the same, byte for byte.  ES_KM_CACHE_DIR names the directory ("off" or "" switches the cache off);
 // by default it is $XDG_CACHE_HOME/es_km or $HOME/.cache/es_km.  Files are written under a
 // temporary name and renamed, so concurrent processes never see half a file.
-
-constexpr char COMPILE_OPTIONS[] = "gfx950 -O3 -std=c++17 -packed-fp32-ops -ffp-contract=off";
 
 std::string cache_dir()
 {
@@ -1240,10 +1246,17 @@ uint64_t fnv1a(std::string const& text, uint64_t h)
 
 std::string cache_text(std::string const& source)
 {
-    int major = 0, minor = 0;
+    // the compiler that would compile it: its version as the library reports it, the
+    // runtime's full version number (patch level included) and the build the headers of this
+    // library came from
+    int major = 0, minor = 0, runtime = 0;
     hiprtcVersion(&major, &minor);
-    return "hiprtc " + std::to_string(major) + "." + std::to_string(minor) + "\n" +
-           COMPILE_OPTIONS + "\n" + source;
+    (void)hipRuntimeGetVersion(&runtime);
+    std::string text = "hiprtc " + std::to_string(major) + "." + std::to_string(minor) +
+                       " runtime " + std::to_string(runtime) + " headers " +
+                       std::to_string(HIP_VERSION) + " " + HIP_VERSION_GITHASH + "\n";
+    for (std::string const& o : compile_options("gfx950")) text += o + " ";
+    return text + "\n" + source;
 }
 
 std::string cache_file(std::string const& dir, std::string const& text)
@@ -1256,19 +1269,24 @@ std::string cache_file(std::string const& dir, std::string const& text)
 }
 
 struct cache_header_t {
-    char     magic[8];  // "ESKMCO1\0"
+    char     magic[8];  // "ESKMCO2\0"
     uint64_t text_bytes;
     uint64_t code_bytes;
 };
 
-bool read_cached(std::string const& path, uint64_t text_bytes, std::vector<char>& code)
+bool read_cached(std::string const& path, std::string const& text, std::vector<char>& code)
 {
     std::FILE* f = std::fopen(path.c_str(), "rb");
     if (!f) return false;
     cache_header_t h;
     bool           ok = std::fread(&h, sizeof(h), 1, f) == 1 &&
-              std::memcmp(h.magic, "ESKMCO1", 8) == 0 && h.text_bytes == text_bytes &&
+              std::memcmp(h.magic, "ESKMCO2", 8) == 0 && h.text_bytes == text.size() &&
               h.code_bytes > 0 && h.code_bytes < (1ull << 30);
+    if (ok) {
+        // two texts with one hash would share a file name: the text itself decides
+        std::string stored(text.size(), 0);
+        ok = std::fread(&stored[0], 1, stored.size(), f) == stored.size() && stored == text;
+    }
     if (ok) {
         code.resize(size_t(h.code_bytes));
         ok = std::fread(code.data(), 1, code.size(), f) == code.size() && std::fgetc(f) == EOF;
@@ -1277,7 +1295,7 @@ bool read_cached(std::string const& path, uint64_t text_bytes, std::vector<char>
     return ok;
 }
 
-void write_cached(std::string const& dir, std::string const& path, uint64_t text_bytes,
+void write_cached(std::string const& dir, std::string const& path, std::string const& text,
                   std::vector<char> const& code)
 {
     // failures only mean that the next process compiles again
@@ -1289,10 +1307,11 @@ void write_cached(std::string const& dir, std::string const& path, uint64_t text
     std::FILE*  f = std::fopen(tmp.c_str(), "wb");
     if (!f) return;
     cache_header_t h;
-    std::memcpy(h.magic, "ESKMCO1", 8);
-    h.text_bytes = text_bytes;
+    std::memcpy(h.magic, "ESKMCO2", 8);
+    h.text_bytes = text.size();
     h.code_bytes = code.size();
     bool ok = std::fwrite(&h, sizeof(h), 1, f) == 1 &&
+              std::fwrite(text.data(), 1, text.size(), f) == text.size() &&
               std::fwrite(code.data(), 1, code.size(), f) == code.size();
     ok = (std::fclose(f) == 0) && ok;
     if (!ok || std::rename(tmp.c_str(), path.c_str()) != 0) std::remove(tmp.c_str());
@@ -1308,12 +1327,12 @@ std::vector<char> code_object_for(std::string const& source, bool* from_disk)
     std::string const text = cache_text(source);
     std::string const path = cache_file(dir, text);
     std::vector<char> code;
-    if (read_cached(path, text.size(), code)) {
+    if (read_cached(path, text, code)) {
         if (from_disk) *from_disk = true;
         return code;
     }
     code = compile_hip_source(source, "es_generated.hip", "gfx950");
-    write_cached(dir, path, text.size(), code);
+    write_cached(dir, path, text, code);
     return code;
 }
 

@@ -165,7 +165,8 @@ struct contraction_plan_t : plan_t {
         // the wide epilogue lives in the direct-to-LDS kernel and in the register-staged
         // one (A along k, B along k or n)
         bool const dma = (dtype == dtype_t::f16 && gemm_dma_eligible<_Float16>(a)) ||
-                         (dtype == dtype_t::f32 && gemm_dma_eligible<float>(a));
+                         (dtype == dtype_t::f32 && gemm_dma_eligible<float>(a)) ||
+                         (dtype == dtype_t::f64 && gemm_dma_wide_eligible<double>(a, 4));
         if (a.c_mode == 3 && !dma && !(a.a_mode == 0 && a.b_mode != 2)) a.c_mode = 0;
         // what build() described is what runs, unless a buffer's alignment forbids it
         if (!dma) a.splits = 1;  // only the direct-to-LDS kernel splits k
@@ -303,7 +304,8 @@ std::shared_ptr<plan_t> plan_contraction(einsummable_t const& e, int)
                        e.inn_nelem(1) * dtype_size(dt) < (1ull << 32);
 
     bool const dma_ok = (dt == dtype_t::f16 && gemm_dma_eligible<_Float16>(a)) ||
-                        (dt == dtype_t::f32 && gemm_dma_eligible<float>(a));
+                        (dt == dtype_t::f32 && gemm_dma_eligible<float>(a)) ||
+                        (dt == dtype_t::f64 && gemm_dma_wide_eligible<double>(a, 4));
     // large tiles exist in the direct-to-LDS kernel (both operands on a vector path) and, for
     // A along k, in the register-staged one
     if (dma_ok || (a.a_mode == 0 && a.b_mode != 2)) {
@@ -320,8 +322,9 @@ std::shared_ptr<plan_t> plan_contraction(einsummable_t const& e, int)
     if (uint64_t(a.tiles_m) * a.tiles_n >= lim) return nullptr;
 
     bool const dma = dma_ok;  // every tile has a direct-to-LDS kernel
-    p->planned_dma = dma && (dt == dtype_t::f16 ? gemm_dma_eligible<_Float16>(a)
-                                                : gemm_dma_eligible<float>(a));
+    p->planned_dma = dma && (dt == dtype_t::f16   ? gemm_dma_eligible<_Float16>(a)
+                             : dt == dtype_t::f32 ? gemm_dma_eligible<float>(a)
+                                                  : gemm_dma_wide_eligible<double>(a, 4));
     // Too few tiles for the device and a long reduction (skinny products, e.g. one token
     // against a weight matrix): several workgroups share a tile's k range and a second
     // kernel sums their fp32 partial tiles, which live in the workspace.
@@ -342,7 +345,8 @@ std::shared_ptr<plan_t> plan_contraction(einsummable_t const& e, int)
         a.xcd_total = Bt > 1 && tiles < (1ull << 32) && !(env && env[0] == '0') ? uint32_t(tiles) : 0;
     }
     uint64_t const nk = K * dtype_size(dt) / 64;
-    if (p->planned_dma && nk >= 16) {
+    // (the partial tiles of a split product are fp32: not for f64)
+    if (p->planned_dma && nk >= 16 && dt != dtype_t::f64) {
         uint64_t S = tiles <= 128 ? std::min<uint64_t>({256 / tiles, nk / 8, 64}) : 1;
         if (const char* env = std::getenv("ES_KM_GEMM_SPLITS")) {  // tuning and tests
             S = std::min<uint64_t>(uint64_t(std::max(1, std::atoi(env))), nk / 4);

@@ -86,8 +86,11 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dma_kernel(gemm_args_t a)
     // load instructions per thread per slice: one moves 1 KiB per wavefront
     constexpr int NLA = BM * RB / (NW * 1024), NLB = BN * RB / (NW * 1024);
     static_assert(NLA >= 1 && NLB >= 1 && (NW == 4 || NW == 8), "whole load instructions");
-    static_assert(MI == 32 && tr::KG == 2 && (STEPS == 2 || STEPS == 4) && (RB == 64 || RB == 128),
-                  "layout below assumes 32x32 tiles");
+    // 32 x 32 matrix tiles with two lane groups along k (f16, f32) or 16 x 16 tiles with four
+    // (f64: v_mfma_f64_16x16x4_f64); a lane group reads one 16-byte chunk per k-step
+    static_assert(((MI == 32 && tr::KG == 2) || (MI == 16 && tr::KG == 4)) &&
+                      (STEPS == 2 || STEPS == 4) && (RB == 64 || RB == 128),
+                  "fragment layout");
     static_assert(BM % 64 == 0 && BN % 64 == 0, "");
     // An operand contiguous along m / n (mode 1) stays [k][m] / [k][n] in LDS: BK rows of
     // BM / BN elements
@@ -171,8 +174,10 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dma_kernel(gemm_args_t a)
     // reads (which walk down k for a fixed m / n) spread over the banks; bits of the k row
     // select which 64-byte (2-byte elements: rows k..k+3 are read together) or 128-byte
     // (4-byte elements: rows k and k+4) segment a chunk lands in
+    // (8-byte elements: a lane group reads rows k and k + 1, the four groups rows 0, 2, 4, 6
+    // of a k-step: bit 1 of the row picks the half)
     auto kn_swizzle = [](uint32_t r) {
-        return sizeof(T) == 2 ? (r & 3) << 2 : ((r >> 2) & 1) << 3;
+        return sizeof(T) == 2 ? (r & 3) << 2 : (sizeof(T) == 4 ? ((r >> 2) & 1) << 3 : ((r >> 1) & 1) << 3);
     };
 #pragma unroll
     for (int i = 0; i != NLA; ++i) {
@@ -294,13 +299,13 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dma_kernel(gemm_args_t a)
         }
     }
 
-    // Fragment of k-step s for MFMA tile row r0 + lane % 32: k-chunk 2 s + lane / 32, found
-    // in slot chunk ^ bits 2..3 of the row
+    // Fragment of k-step s for MFMA tile row r0 + lane % MI: k-chunk KG s + lane / MI, found
+    // in slot chunk ^ bits 2..3 (64-byte rows) or 1..3 (128-byte rows) of the row
     int const f_sw = RB == 64 ? (lane >> 2) & 3 : ((lane % MI) >> 1) & 7;
     int       f_off[STEPS];
 #pragma unroll
     for (int s = 0; s != STEPS; ++s) {
-        f_off[s] = (lane % MI) * RB + (((2 * s + lane / MI) ^ f_sw) * 16);
+        f_off[s] = (lane % MI) * RB + (((tr::KG * s + lane / MI) ^ f_sw) * 16);
     }
     int const fa_base = wm * WM * RB;
     int const fb_base = A_BYTES + wn * WN * RB;
@@ -319,7 +324,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dma_kernel(gemm_args_t a)
             } else {
                 int const m0 = wm * WM + i * MI + lane % MI;
                 int const k0 = (lane / MI) * VL;
-                f_km[i] = k0 * RAM + ((m0 * 4) ^ int(kn_swizzle(uint32_t(k0)) * 16));
+                f_km[i] = k0 * RAM + ((m0 * int(sizeof(T))) ^ int(kn_swizzle(uint32_t(k0)) * 16));
             }
         }
     }
@@ -337,7 +342,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dma_kernel(gemm_args_t a)
             } else {
                 int const n0 = wn * WN + j * MI + lane % MI;
                 int const k0 = (lane / MI) * VL;
-                f_kn[j] = k0 * RBN + ((n0 * 4) ^ int(kn_swizzle(uint32_t(k0)) * 16));
+                f_kn[j] = k0 * RBN + ((n0 * int(sizeof(T))) ^ int(kn_swizzle(uint32_t(k0)) * 16));
             }
         }
     }
@@ -356,13 +361,18 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dma_kernel(gemm_args_t a)
                 (__attribute__((address_space(3))) tr_t*)(p + 4 * row_bytes));
             tr8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
             return __builtin_bit_cast(chunk_t, both);
-        } else {
+        } else if constexpr (sizeof(T) == 4) {
             chunk_t v;
 #pragma unroll
             for (int t = 0; t != VL; ++t) {
                 v[t] = *reinterpret_cast<uint32_t const*>(p + t * row_bytes);
             }
             return v;
+        } else {
+            typedef uint32_t pair_t __attribute__((ext_vector_type(2)));
+            pair_t const lo = *reinterpret_cast<pair_t const*>(p);
+            pair_t const hi = *reinterpret_cast<pair_t const*>(p + row_bytes);
+            return chunk_t{lo[0], lo[1], hi[0], hi[1]};
         }
     };
     auto read_a = [&](char const* stage, int s, int i) {
@@ -548,12 +558,21 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dma_kernel(gemm_args_t a)
         for (int j = 0; j != TN; ++j) {
 #pragma unroll
             for (int e0 = 0; e0 < tr::NACC; e0 += 4) {
-                quad_t q;
+                if constexpr (tr::QUAD) {
+                    quad_t q;
 #pragma unroll
-                for (int t = 0; t != 4; ++t) q[t] = T(acc[i][j][e0 + t] * alpha);
-                int n = j * MI + tr::acc_row(e0, lane);
-                *reinterpret_cast<quad_t*>(strip + (lane % MI) * STRIP_PITCH +
-                                           n * int(sizeof(T))) = q;
+                    for (int t = 0; t != 4; ++t) q[t] = T(acc[i][j][e0 + t] * alpha);
+                    int n = j * MI + tr::acc_row(e0, lane);
+                    *reinterpret_cast<quad_t*>(strip + (lane % MI) * STRIP_PITCH +
+                                               n * int(sizeof(T))) = q;
+                } else {
+#pragma unroll
+                    for (int t = 0; t != 4; ++t) {
+                        int n = j * MI + tr::acc_row(e0 + t, lane);
+                        *reinterpret_cast<T*>(strip + (lane % MI) * STRIP_PITCH +
+                                              n * int(sizeof(T))) = T(acc[i][j][e0 + t] * alpha);
+                    }
+                }
             }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");

@@ -237,6 +237,15 @@ struct traits_t<double> {
     // row 4 * i + l / 16, so a lane's four values are four rows apart
     __device__ static __forceinline__ int acc_row(int i, int lane) { return 4 * i + lane / 16; }
     static constexpr bool QUAD = false;
+    // a 16-byte chunk holds two k elements: two matrix instructions
+    static constexpr int SUB = 2;
+    __device__ static __forceinline__ void mma_sub(acc_t& acc, chunk_t const& row,
+                                                   chunk_t const& col, int t)
+    {
+        double2_t r = __builtin_bit_cast(double2_t, row);
+        double2_t c = __builtin_bit_cast(double2_t, col);
+        acc = __builtin_amdgcn_mfma_f64_16x16x4f64(r[t], c[t], acc, 0, 0, 0);
+    }
 };
 
 constexpr int ROW_BYTES = 128;  // bytes of k per tile row per stage

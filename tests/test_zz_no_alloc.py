@@ -31,12 +31,17 @@ def both_ways(km, e, inputs):
     d_ws = torch.empty(max(ws, 1), dtype=torch.uint8, device="cuda")
     torch.cuda.synchronize()
     # nothing below this line may allocate on the device: torch's counters see torch's own
-    # allocations, and the library has no allocating call on this path
-    before = torch.cuda.memory_stats()["allocation.all.allocated"]
+    # allocations, the driver's free-memory figure sees the library's as well (a hipMalloc,
+    # a stream or an event of its own would lower it)
     km(e, stream_handle(), d_a.data_ptr(), ptrs, (d_ws.data_ptr(), ws) if ws else None)
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_stats()["allocation.all.allocated"]
+    free_before = torch.cuda.mem_get_info()[0]
+    km.execute_static_workspace(e, stream_handle(), d_b.data_ptr(), ptrs)
     km.execute_static_workspace(e, stream_handle(), d_b.data_ptr(), ptrs)
     torch.cuda.synchronize()
     assert torch.cuda.memory_stats()["allocation.all.allocated"] == before
+    assert torch.cuda.mem_get_info()[0] == free_before
     return to_host(d_a, NP[od]), to_host(d_b, NP[od]), ws
 
 
