@@ -429,15 +429,18 @@ std::shared_ptr<plan_t> plan_contraction(einsummable_t const& e, int)
                 a.persistent = 2;
             }
         }
-        if (a.persistent) {
-            int dev = 0, cus = 0;
-            if (hipGetDevice(&dev) != hipSuccess ||
-                hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
-                cus <= 0) {
-                a.persistent = 0;
-            }
-            a.workgroups = uint32_t(cus);
+    }
+    if (a.persistent || a.shortk) {
+        // one workgroup per compute unit
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+            cus <= 0) {
+            a.persistent = 0;
+            a.shortk = 0;
+            cus = 0;
         }
+        a.workgroups = uint32_t(cus);
     }
     static const char* mode_name[] = {"k", "mn", "elem"};
     p->description = std::string("contraction_mfma_") + dtype_name(dt) + " tile=" +

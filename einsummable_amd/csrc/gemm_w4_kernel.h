@@ -63,6 +63,15 @@ __device__ __forceinline__ void mma(chunk_t const& x, chunk_t const& y)
                  : "n"(16 * T), "n"(16 * T + 15), "v"(x), "v"(y));
 }
 
+// the same with a zero addend: the first product of a sum
+template <int T>
+__device__ __forceinline__ void mma_first(chunk_t const& x, chunk_t const& y)
+{
+    asm volatile("v_mfma_f32_32x32x16_f16 a[%0:%1], %2, %3, 0"
+                 :
+                 : "n"(16 * T), "n"(16 * T + 15), "v"(x), "v"(y));
+}
+
 template <int R>
 __device__ __forceinline__ float acc_read()
 {

@@ -454,6 +454,30 @@ def test_resident_lhs_kernel_for_head_dimension_reductions(km, monkeypatch, case
     assert_close(np.ascontiguousarray(got).reshape(-1), want, DT["f16"], what=spec)
 
 
+@pytest.mark.parametrize("grid,resident_min", [(24, 1), (8, 1), (4096, 1)])
+def test_resident_lhs_kernel_streams_of_walks(monkeypatch, grid, resident_min):
+    """The resident-lhs kernel with a forced number of workgroups: few (every workgroup works
+    through many walks, among them the short last walk of a row of 19 tiles), and more than
+    there are walks (workgroups without work).  Bitwise against the kernel that takes a
+    workgroup per tile."""
+    spec, sizes = "bid,bjd->bij", dict(b=5, i=300, j=2400, d=128)
+    e = contraction(spec, sizes, "f16")
+    monkeypatch.setenv("ES_KM_GEMM_RESIDENT_MIN", str(resident_min))
+    monkeypatch.setenv("ES_KM_GEMM_RESIDENT_GRID", str(grid))
+    streamed = ea.KernelManager(0)
+    streamed.build(e)
+    assert "resident_a" in streamed.describe(e), streamed.describe(e)
+    monkeypatch.setenv("ES_KM_GEMM_RESIDENT_A", "0")
+    per_tile = ea.KernelManager(0)
+    per_tile.build(e)
+    assert "resident_a" not in per_tile.describe(e)
+    r = rng(77)
+    xs = [normal(r, int(np.prod(e.inn_shape(k))), np.float16) for k in range(2)]
+    a = run_einsummable(streamed, e, xs)
+    b = run_einsummable(per_tile, e, xs)
+    np.testing.assert_array_equal(a.view(np.uint16), b.view(np.uint16))
+
+
 def scaled(spec, sizes, dt, const, form=0):
     c = "constant{%s|%s}" % (dt, const)
     prod = ["*[hole|%s@0,hole|%s@1]", "*[hole|%s@1,hole|%s@0]"][form & 1] % (dt, dt)
