@@ -553,8 +553,13 @@ void kernel_manager_t::touch_batch(std::vector<touch_t> const& touches_, hipStre
             }
             uint32_t const W = uint32_t(touch_list_item_words(R));
             int const      ND = R > 2 ? 4 : 2;
+            double         covered = 0;  // elements, counted once per window
+            uint32_t const first_op = uint32_t(items[first].op);
+            bool           all_vectors = true;  // ... and all with the first item's op
             for (size_t i = 0; i != cnt; ++i) {
                 touch_item_t const& it = items[first + i];
+                all_vectors = all_vectors && it.vec_rows && uint32_t(it.op) == first_op;
+                covered += double(it.size[0]) * it.size[1] * it.size[2] * it.size[3];
                 uint32_t* const     w = b.w + i * W;
                 std::memset(w, 0, W * sizeof(uint32_t));
                 uint64_t const p = reinterpret_cast<uint64_t>(it.inn);
@@ -587,6 +592,8 @@ void kernel_manager_t::touch_batch(std::vector<touch_t> const& touches_, hipStre
                     rows *= hi[s] - lo[s];
                 }
             }
+            b.eager = covered >= 0.5 * double(rows) * double(hi[3] - lo[3]);
+            b.uniform_op = all_vectors ? 1 + first_op : 0;
             uint64_t const vpr = (hi[3] - lo[3]) / uint64_t(b.vec);
             b.chunks_per_row = uint32_t((vpr + TOUCH_LIST_BLOCK_HOST - 1) / TOUCH_LIST_BLOCK_HOST);
             if (rows * b.chunks_per_row >= (1ull << 31)) {

@@ -61,6 +61,8 @@ struct touch_list_t {
     uint32_t rank;            // 1..4: of the touches; > 2 selects the four-dimensional items
     uint32_t vec;             // elements per output vector
     uint32_t chunks_per_row;  // workgroups per row of the bounding box
+    uint32_t eager;           // the windows cover at least half of the bounding box
+    uint32_t uniform_op;      // 0, or 1 + the op that all items share, all taking whole vectors
     uint32_t box_lo[4];       // bounding box of the windows, four normalised dimensions
     uint32_t box_size[4];     // inner extent in elements, a multiple of vec
     uint64_t out_str[3];      // element strides of the output's outer dimensions

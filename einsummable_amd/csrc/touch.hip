@@ -210,31 +210,44 @@ __device__ __forceinline__ T apply_dyn(int op, T out, T inn)
 }
 
 constexpr int TOUCH_LIST_BLOCK = TOUCH_LIST_BLOCK_HOST;
+constexpr int TOUCH_LIST_WAVES = 4;  // wavefronts (row pieces) per workgroup
 
 // ---- a list of touches folded by the owner of each output vector
 //
-// One workgroup = one wavefront = 64 consecutive output vectors of one row of the bounding
-// box.  Lane t tests whether item t reaches the wavefront (at most 64 items per launch), the
+// One wavefront = 64 consecutive output vectors of one row of the bounding box (a workgroup's
+// wavefronts take consecutive rows).  Lane t tests whether item t reaches the wavefront (at most 64 items per launch), the
 // ballot is the wavefront's list, and the items on it are folded in list order; everything
 // about an item except the lane's own column is uniform and sits in one wide scalar load.
 // What this replaces, on 64 accumulating windows of 512 x 512 at odd offsets of a 4096 x 4096
 // f16 output: the same fold unrolled over 32 items per launch (the code outgrew the
 // instruction cache: 2 x 77 us), a scalar walk over all items (several dependent scalar loads
 // each: 189 us), workgroups of 256 (seven items each on average, one latency chain after the
-// other: 48 us).
+// other: 48 us).  The wavefronts are short-lived and execute some six hundred instructions
+// each, so the kernel is bound by instruction issue as much as by memory: folding two items
+// per round instead of four (a wavefront meets one or two) took that case from 32 to 29 us,
+// compiling the items' op and load path in (UOP) to 22 us; several rows per wavefront or
+// more wavefronts per workgroup changed nothing.
 //
 // R4: items keep four dimensions (16 words); otherwise two (12 words; leading extents are 1).
 // Words of an item, ND = 4 or 2: input pointer (2), base_inn (2), lo[ND], size[ND],
 // str_inn[ND - 1], op | vec_rows << 8 | shift << 16.
-template <typename T, int V, bool R4>
-__global__ __launch_bounds__(TOUCH_LIST_BLOCK) void touch_list_kernel(touch_list_t b,
-                                                                      T* __restrict__ out)
+//
+// UOP: -1, or every item of the launch has this op and takes its input as shifted whole
+// vectors (the usual case -- all of a tensor's partial blocks are added or copied, from
+// buffers with aligned rows): the per-item choices are then made by the compiler.
+template <typename T, int V, bool R4, int UOP>
+__global__ __launch_bounds__(TOUCH_LIST_BLOCK* TOUCH_LIST_WAVES) void touch_list_kernel(
+    touch_list_t b, T* __restrict__ out, uint32_t n_rows)
 {
+    static_assert(UOP < 0 || V * sizeof(T) == 16, "");
     using vt = vec_t<T, V>;
     constexpr int ND = R4 ? 4 : 2;
     constexpr int WI = R4 ? 16 : 12;
+    uint32_t const lane = threadIdx.x % TOUCH_LIST_BLOCK;
     uint32_t       row = blockIdx.x / b.chunks_per_row;
     uint32_t const chunk = blockIdx.x - row * b.chunks_per_row;
+    row = row * TOUCH_LIST_WAVES + threadIdx.x / TOUCH_LIST_BLOCK;
+    if (row >= n_rows) return;
     uint32_t       u[3] = {0, 0, 0};  // the row's coordinates, right-aligned
     uint64_t       row_off = 0;
     if constexpr (R4) {
@@ -253,7 +266,7 @@ __global__ __launch_bounds__(TOUCH_LIST_BLOCK) void touch_list_kernel(touch_list
     uint32_t const col_lo = b.box_lo[3] + chunk * uint32_t(TOUCH_LIST_BLOCK) * V;
     uint32_t const col_hi =
         col_lo + uint32_t(TOUCH_LIST_BLOCK) * V < box_hi3 ? col_lo + uint32_t(TOUCH_LIST_BLOCK) * V : box_hi3;
-    uint32_t const c3 = col_lo + threadIdx.x * V;
+    uint32_t const c3 = col_lo + lane * V;
     bool const     live = c3 < box_hi3;
     uint64_t const oo = row_off + c3;
     // The item table is read through the kernel-argument pointer (`b` is the first argument):
@@ -263,11 +276,15 @@ __global__ __launch_bounds__(TOUCH_LIST_BLOCK) void touch_list_kernel(touch_list
     typedef char const __attribute__((address_space(4))) const_byte_t;
     const_word_t* const table = (const_word_t*)((const_byte_t*)__builtin_amdgcn_kernarg_segment_ptr() +
                                                 offsetof(touch_list_t, w));
+    // Where the windows cover most of the bounding box the old value is asked for before the
+    // wavefront knows whether a window reaches it (the test is a round trip to the item table)
+    vt val;
+    if (b.eager && live) val = *reinterpret_cast<vt const*>(out + oo);
     uint64_t todo;
     {
         // every word is loaded before the first comparison (a test that stops at the first
         // miss waits for one load after the other)
-        uint32_t const      t = threadIdx.x;
+        uint32_t const      t = lane;
         const_word_t* const it = table + (t < b.n ? t : 0u) * WI;
         uint32_t            lo[ND], sz[ND];
 #pragma unroll
@@ -281,15 +298,14 @@ __global__ __launch_bounds__(TOUCH_LIST_BLOCK) void touch_list_kernel(touch_list
         todo = __ballot(hit);
     }
     if (todo == 0) return;
-    // the old value is on its way while the first item's words arrive; lanes that no window
-    // reaches never store
-    vt val;
-    if (live) val = *reinterpret_cast<vt const*>(out + oo);
+    // otherwise the old value is on its way while the first item's words arrive; lanes that
+    // no window reaches never store
+    if (!b.eager && live) val = *reinterpret_cast<vt const*>(out + oo);
     bool have = false;
     // K items at a time: the words of all K, then the input vectors of all K, are under way
     // before the first one is folded in -- one item after the other, each a chain of a scalar
     // load, two vector loads and the update, a wavefront lived 14 k cycles for two items
-    constexpr int K = R4 ? 2 : 4;
+    constexpr int K = 2;
     while (todo) {
         uint32_t w[K][WI];
         bool     valid[K];
@@ -325,7 +341,7 @@ __global__ __launch_bounds__(TOUCH_LIST_BLOCK) void touch_list_kernel(touch_list
 #pragma unroll
             for (int i = 0; i != 8; ++i) d[k][i] = 0;
             if constexpr (V * sizeof(T) == 16) {
-                if (covered[k] && (flags & 0x100)) {
+                if (covered[k] && (UOP >= 0 || (flags & 0x100))) {
                     // The input's rows are 16-byte aligned but the window sits `sh` elements
                     // off the output's vector grid: the vector's elements come out of two
                     // aligned input vectors, shifted by a whole number of bytes that is the
@@ -352,11 +368,11 @@ __global__ __launch_bounds__(TOUCH_LIST_BLOCK) void touch_list_kernel(touch_list
         for (int k = 0; k != K; ++k) {
             if (!covered[k]) continue;
             uint32_t const flags = w[k][4 + 3 * ND - 1];
-            int const      op = int(flags & 0xff);
+            int const      op = UOP >= 0 ? UOP : int(flags & 0xff);
             bool const     full = j_lo[k] == 0 && j_hi[k] == uint32_t(V - 1);
             vt             x;
             bool           by_vector = false;
-            if constexpr (V * sizeof(T) == 16) by_vector = (flags & 0x100) != 0;
+            if constexpr (V * sizeof(T) == 16) by_vector = UOP >= 0 || (flags & 0x100) != 0;
             if (by_vector) {
                 uint32_t const bytes = ((flags >> 16) & 0xf) * uint32_t(sizeof(T));
                 uint32_t const q = bytes >> 2, r = bytes & 3;
@@ -420,22 +436,33 @@ __global__ __launch_bounds__(TOUCH_LIST_BLOCK) void touch_list_kernel(touch_list
 template <typename T>
 void launch_touch_list_t(touch_list_t const& b, hipStream_t stream, void* out)
 {
-    constexpr int  VMAX = 16 / sizeof(T);
+    constexpr int VMAX = 16 / sizeof(T);
+    dim3 const    block(TOUCH_LIST_BLOCK * TOUCH_LIST_WAVES);
+    T* const      o = static_cast<T*>(out);
+    bool const    r4 = b.rank > 2;
+    // (the planner bounds rows x chunks of the bounding box)
     uint64_t const rows = uint64_t(b.box_size[0]) * b.box_size[1] * b.box_size[2];
-    dim3 const     grid(unsigned(rows * b.chunks_per_row));
-    dim3 const     block(TOUCH_LIST_BLOCK);
-    T* const       o = static_cast<T*>(out);
-    bool const     r4 = b.rank > 2;
+    uint64_t const row_groups = (rows + TOUCH_LIST_WAVES - 1) / TOUCH_LIST_WAVES;
+    dim3 const     grid(unsigned(row_groups * b.chunks_per_row));
+    uint32_t const n_rows = uint32_t(rows);
     if (int(b.vec) == VMAX) {
         if (r4) {
-            hipLaunchKernelGGL((touch_list_kernel<T, VMAX, true>), grid, block, 0, stream, b, o);
+            hipLaunchKernelGGL((touch_list_kernel<T, VMAX, true, -1>), grid, block, 0, stream, b, o,
+                               n_rows);
+        } else if (b.uniform_op == OP_ADD + 1) {
+            hipLaunchKernelGGL((touch_list_kernel<T, VMAX, false, OP_ADD>), grid, block, 0, stream, b,
+                               o, n_rows);
+        } else if (b.uniform_op == OP_COPY + 1) {
+            hipLaunchKernelGGL((touch_list_kernel<T, VMAX, false, OP_COPY>), grid, block, 0, stream,
+                               b, o, n_rows);
         } else {
-            hipLaunchKernelGGL((touch_list_kernel<T, VMAX, false>), grid, block, 0, stream, b, o);
+            hipLaunchKernelGGL((touch_list_kernel<T, VMAX, false, -1>), grid, block, 0, stream, b, o,
+                               n_rows);
         }
     } else if (r4) {
-        hipLaunchKernelGGL((touch_list_kernel<T, 1, true>), grid, block, 0, stream, b, o);
+        hipLaunchKernelGGL((touch_list_kernel<T, 1, true, -1>), grid, block, 0, stream, b, o, n_rows);
     } else {
-        hipLaunchKernelGGL((touch_list_kernel<T, 1, false>), grid, block, 0, stream, b, o);
+        hipLaunchKernelGGL((touch_list_kernel<T, 1, false, -1>), grid, block, 0, stream, b, o, n_rows);
     }
 }
 

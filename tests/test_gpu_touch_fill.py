@@ -216,6 +216,27 @@ def test_touch_batch_stacked_partial_sums(km, dt):
     assert_bits_equal(to_host(d_out, NP[dt]), want, "stacked partial sums")
 
 
+@pytest.mark.parametrize("castable", [None, "+"])
+def test_touch_batch_of_one_op_with_aligned_rows(km, castable):
+    """Every touch of the batch has the same op and an input whose rows are 16-byte aligned
+    (the form the batch kernel specialises on): overlapping windows at odd column offsets,
+    more than one launch's worth of touches, in list order (with plain copies the last writer
+    of an element wins)."""
+    r = rng(91 if castable else 90)
+    n, touches, blocks = 520, [], []
+    for _ in range(90):
+        h, w = int(r.randint(1, 200)), 8 * int(r.randint(1, 30))
+        ro, co = int(r.randint(0, n - h + 1)), int(r.randint(0, n - w + 1))
+        touches.append(ea.Touch([(h, n, 0, ro, h), (w, n, 0, co, w)], castable, ea.F16))
+        blocks.append(normal(r, h * w, np.float16))
+    out0 = normal(r, n * n, np.float16)
+    want = _apply_sequentially(touches, blocks, out0)
+    d_out = to_device(out0)
+    d_blocks = [to_device(x) for x in blocks]
+    km.touch_batch(touches, stream_handle(), d_out.data_ptr(), [x.data_ptr() for x in d_blocks])
+    assert_bits_equal(to_host(d_out, np.float16), want, "one-op batch")
+
+
 def test_touch_batch_errors(km):
     d = to_device(np.zeros(64, np.float32))
     a = ea.Touch([(4, 8, 0, 0, 4)], None, ea.F32)
