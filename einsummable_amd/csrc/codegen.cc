@@ -968,11 +968,14 @@ cg_kernel_t gen_reduce_col(einsummable_t const& e, int max_vec)
     // Few outputs and a long aggregation: one thread per output vector leaves the device
     // idle.  The outermost aggregated mode is then cut into slices that run side by side
     // (grid z), each leaving partial results in the workspace; a second kernel folds the
-    // slices in order, so the result does not depend on scheduling.
+    // slices in order, so the result does not depend on scheduling.  (One launch, in which
+    // the slices raise flags in the workspace and the last one folds, was measured on 8192 x
+    // 8192 f16: the fences that make partial results and flags visible across the device's
+    // L2 caches cost 23 us in all, the second launch costs 4.)
     uint64_t const outer = L.shape[O];
     // measured with the slice-parallel fold below: 128 K threads with 4 rows in flight each
     // (8192 x 8192 f16: 4.2 TB/s with 64 K, 4.6 with 128 K, 4.9 with 256 K, where 2048 x 4096
-    // f32 and 64 x 2048 x 1024 f16 lose 6-9 %)
+    // f32 and 64 x 2048 x 1024 f16 lose 6-9 %); eight rows in flight are 3 % faster than four
     uint64_t const want_threads = 1ull << 17;
     uint64_t       S = 1;
     if (n_vec * 2 <= want_threads && outer >= 16) {
@@ -1069,11 +1072,11 @@ cg_kernel_t gen_reduce_col(einsummable_t const& e, int max_vec)
             s << indent << "const idx_t hi" << m << " = lo" << m << " + " << g.P(p_chunk) << " < "
               << g.P(p_shape[m]) << " ? lo" << m << " + " << g.P(p_chunk) << " : "
               << g.P(p_shape[m]) << ";\n";
-            if (m == R - 1) s << "#pragma unroll 4\n";  // several rows' loads in flight
+            if (m == R - 1) s << "#pragma unroll 8\n";  // several rows' loads in flight
             s << indent << "for (idx_t g" << m << " = lo" << m << "; g" << m << " < hi" << m
               << "; ++g" << m << ") {\n";
         } else {
-            if (m == R - 1) s << "#pragma unroll 4\n";
+            if (m == R - 1) s << "#pragma unroll 8\n";
             s << indent << "for (idx_t g" << m << " = 0; g" << m << " != " << g.P(p_shape[m])
               << "; ++g" << m << ") {\n";
         }

@@ -7,8 +7,8 @@ import pytest
 
 import einsummable_amd as ea
 import oracle
-from helpers import (NP, assert_bits_equal, assert_close, assert_values_equal, normal, oracle_einsummable, rng,
-                     run_einsummable, uniform)
+from helpers import (NP, assert_bits_equal, assert_close, assert_values_equal, empty_device, normal,
+                     oracle_einsummable, rng, run_einsummable, stream_handle, to_device, to_host, uniform)
 
 pytestmark = pytest.mark.gpu
 
@@ -253,6 +253,32 @@ def test_split_column_reductions(km, case):
     assert ws is not None and ws > 0, "expected a two-pass plan"
     assert "splits=" in km.describe(e) and km.workspace_size(e) == ws
     check(km, e, seed=60 + case, exact=exact)
+
+
+def test_sliced_column_reduction_on_a_used_workspace(km):
+    """The slices of a column reduction leave their partial results in the workspace, which
+    holds whatever the last user left: the same workspace, first filled with a byte pattern,
+    serves launches with different inputs one after the other, and each result is right."""
+    import torch
+
+    for e, exact in ((E([4096, 2048], [[1, 0]], 1, "hole|f16@0", "^"), True),
+                     (E([64, 4096], [[1, 0]], 1, "hole|f32@0", "+"), False),
+                     (E([3, 1000, 72], [[0, 2, 1]], 2, "hole|f32@0", "+"), False)):
+        ws = km.build(e)
+        assert ws > 0 and "splits=" in km.describe(e)
+        od, _ = oracle.scalarop_info(e.join)
+        d_ws = torch.full((ws,), 0xAB, dtype=torch.uint8, device="cuda")
+        for rep in range(3):
+            xs = inputs_for(e, rng(900 + rep), 1.0, False)
+            d_in = [to_device(x) for x in xs]
+            d_out = empty_device(e.out_nelem(), NP[od])
+            km(e, stream_handle(), d_out.data_ptr(), [t.data_ptr() for t in d_in], (d_ws.data_ptr(), ws))
+            torch.cuda.synchronize()
+            got = to_host(d_out, NP[od])
+            if exact:
+                assert_values_equal(got, oracle_einsummable(e, xs, oracle.EXACT), "launch %d" % rep)
+            else:
+                assert_close(got, oracle_einsummable(e, xs, oracle.WIDE), od, what="launch %d" % rep)
 
 
 def test_workspace_contract_of_a_two_pass_reduction(km):
