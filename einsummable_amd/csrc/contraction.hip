@@ -106,7 +106,13 @@ void choose_tile(dtype_t dt, uint64_t M, uint64_t N, uint64_t K, uint64_t batch,
     double const elem = double(dtype_size(dt));
     double const intensity = 2.0 * double(M) * double(N) * double(K) /
                              ((double(M) * K + double(N) * K + double(M) * N) * elem);
-    if (dt == dtype_t::f16 && intensity < 150.0) return;
+    if (dt == dtype_t::f16 && intensity < 150.0) {
+        // ... unless the streamed operand has rows for 256 of them and that still leaves a
+        // tile for every compute unit: twice the bytes of it under way per workgroup, with
+        // three stages (P.V of 32 and of 128 heads of 2048 x 2048: 7 % faster)
+        if (N <= 128 && M >= 256 && ((M + 255) / 256) * batch >= 256) bm = 256;
+        return;
+    }
     static tile_option_t const options[] = {{256, 256, 1.00, 1.00},
                                             {128, 256, 0.88, 1.00},
                                             {256, 128, 0.88, 1.00},
