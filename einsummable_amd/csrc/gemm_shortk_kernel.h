@@ -23,6 +23,13 @@
 //     stall on a multiplying wave (measured: the time to write C simply added to the time
 //     of everything else) keeps the matrix cores and the loads idle.
 //
+// A staging tile has rows of 256 bytes without padding; the 16-byte chunk c of row m lies at
+// chunk c ^ (m % 16) and its two 8-byte halves are exchanged when bit 3 of m is set.  With
+// that the multiplying waves' 8-byte writes (32 rows per instruction) and the storing waves'
+// 16-byte reads (four whole rows per instruction) are both free of bank conflicts; rows
+// padded by 16 bytes cost every one of those instructions four extra cycles
+// (SQ_LDS_BANK_CONFLICT: 1.1 conflict cycles per active LDS cycle of the whole kernel).
+//
 // One workgroup barrier per tile orders the three roles: a B buffer is refilled after
 // everyone has read it, a staging tile is rewritten after it has been read out.  Step g of a
 // workgroup's stream of tiles multiplies tile g, stages tile g - 1 and stores tile g - 2; one
@@ -50,7 +57,7 @@ constexpr int SK_RB = SK_K * 2;                   // bytes of one operand row
 constexpr int SK_BM = 128, SK_BN = 128;           // tile
 constexpr int SK_BUF = SK_BN * SK_RB;             // one B buffer
 constexpr int SK_NBUF = 2;                        // ring of B buffers
-constexpr int SK_OUT_PITCH = SK_BN * 2 + 16;      // staging row: 128 outputs + pad
+constexpr int SK_OUT_PITCH = SK_BN * 2;           // staging row: 128 outputs, chunks swizzled
 constexpr int SK_OUT = SK_BM * SK_OUT_PITCH;      // one staging tile
 constexpr int SK_LDS = SK_NBUF * SK_BUF + 2 * SK_OUT + 512;  // + scratch of the prefetches
 constexpr int SK_PF_DIST = 4;                     // tiles the L2 prefetch runs ahead
@@ -274,7 +281,11 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_shortk_kernel(gemm_args_t a,
         int const      half = wave - 6;
         uint32_t const lr = uint32_t(lane) >> 4, lch = uint32_t(lane) & 15;
         uint32_t const lane_off = (lr * ldc + lch * 8) * 2;
-        int const      lds_off = int(uint32_t(half) * 64 + lr) * SK_OUT_PITCH + int(lch) * 16;
+        // instruction c reads rows 4 c + lr: chunk lch of such a row lies at lch ^ (4 (c % 4) + lr)
+        int const      lds_row = int(uint32_t(half) * 64 + lr) * SK_OUT_PITCH;
+        int            lds_chunk[4];
+#pragma unroll
+        for (int k = 0; k != 4; ++k) lds_chunk[k] = int((lch ^ (4 * uint32_t(k) + lr)) * 16);
         constexpr int  NST = 16;
         cursor_t       sc;
         seek(sc, blockIdx.x / 8);
@@ -282,13 +293,16 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_shortk_kernel(gemm_args_t a,
         __builtin_amdgcn_s_barrier();  // the first tile is multiplied
         for (uint32_t g = 0; g != steps; ++g) {
             __builtin_amdgcn_s_barrier();  // tile g is staged
-            char const* const out = lds + SK_NBUF * SK_BUF + (g & 1) * SK_OUT + lds_off;
+            char const* const out = lds + SK_NBUF * SK_BUF + (g & 1) * SK_OUT + lds_row;
             uint32_t const    n0 = sc.t * SK_BN;
             uint32_t const    mrow = sc.tm * SK_BM + uint32_t(half) * 64;  // first row of this wave
             chunk_t           v[NST];
 #pragma unroll
             for (int c = 0; c != NST; ++c) {
-                v[c] = *reinterpret_cast<chunk_t const*>(out + c * 4 * SK_OUT_PITCH);
+                chunk_t const x =
+                    *reinterpret_cast<chunk_t const*>(out + c * 4 * SK_OUT_PITCH + lds_chunk[c % 4]);
+                // (bit 3 of the row 4 c + lr is bit 1 of c)
+                v[c] = (c & 2) ? chunk_t{x[2], x[3], x[0], x[1]} : x;
             }
             char* const corner =
                 reinterpret_cast<char*>(static_cast<T*>(a.C) + sc.boc + int64_t(mrow) * ldc + n0);
@@ -383,16 +397,28 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_shortk_kernel(gemm_args_t a,
         return __builtin_bit_cast(uint32_t, v);
     };
     // quad q of half j of the staging tile at `stage`
-    auto stage_quad = [&](char* stage, auto j_tag, auto q_tag, uint32_t lo, uint32_t hi) ES_INLINE {
+    // (the lane's row is wm * 64 + i * 32 + lane % 32: its low four bits are the lane's; the
+    // quad's byte column wn * 128 + j * 64 + (q % 4) * 16 + (lane / 32) * 8 goes through the
+    // row's swizzle, which is an XOR with a value of the lane)
+    uint32_t const stage_swz = (uint32_t(wn) * 128 + uint32_t(lane / 32) * 8) ^
+                               ((uint32_t(lane) & 15) << 4) ^ (((uint32_t(lane) >> 3) & 1) << 3);
+    uint32_t stage_at[8];  // j * 4 + q % 4 -> the quad's address in the current staging tile, row i = 0
+    auto stage_quad = [&](auto j_tag, auto q_tag, uint32_t lo, uint32_t hi) ES_INLINE {
         constexpr int j = decltype(j_tag)::value, q = decltype(q_tag)::value;
-        constexpr int off = (q / 4) * 32 * SK_OUT_PITCH + (j * 32 + (q % 4) * 8) * int(sizeof(T));
-        uint2 v;
-        v.x = lo;
-        v.y = hi;
-        *reinterpret_cast<uint2*>(stage + off) = v;
+        typedef uint32_t pair_t __attribute__((ext_vector_type(2)));
+        typedef __attribute__((address_space(3))) pair_t* lds_pair_ptr;
+        pair_t v;
+        v[0] = lo;
+        v[1] = hi;
+        *(lds_pair_ptr)(uintptr_t)(stage_at[j * 4 + q % 4] + (q / 4) * 32 * SK_OUT_PITCH) = v;
     };
-    char* const stage_lane = lds + SK_NBUF * SK_BUF + (wm * 64 + lane % 32) * SK_OUT_PITCH +
-                             (wn * 64 + (lane / 32) * 4) * int(sizeof(T));
+    uint32_t const stage_row = lds_base + SK_NBUF * SK_BUF + uint32_t(wm * 64 + lane % 32) * SK_OUT_PITCH;
+    auto stage_into = [&](uint32_t parity) ES_INLINE {
+#pragma unroll
+        for (int k = 0; k != 8; ++k) {
+            stage_at[k] = stage_row + parity * SK_OUT + (uint32_t((k / 4) * 64 + (k % 4) * 16) ^ stage_swz);
+        }
+    };
     uint32_t    held = 0;
     // One step on the tile in B buffer `par`; with PREV, the staging tile of the tile before
     // (the other parity) is written.
@@ -404,10 +430,10 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_shortk_kernel(gemm_args_t a,
             fb_at[s] = lds_base + ((fb_lane ^ uint32_t(s << 5)) | (par << 15));
         }
         typedef __attribute__((address_space(3))) chunk_t const* lds_chunk_ptr;
-        char* const stage = stage_lane + (par ^ 1) * SK_OUT;
-        fb[0] = *(lds_chunk_ptr)(fb_at[0]);
-        fb[1] = *(lds_chunk_ptr)(fb_at[1]);
-        fb[2] = *(lds_chunk_ptr)(fb_at[2]);
+        if constexpr (PREV) stage_into(par ^ 1);
+        fb[0] = *(lds_chunk_ptr)(uintptr_t)(fb_at[0]);
+        fb[1] = *(lds_chunk_ptr)(uintptr_t)(fb_at[1]);
+        fb[2] = *(lds_chunk_ptr)(uintptr_t)(fb_at[2]);
         static_for<2>([&](auto j_tag) ES_INLINE {
             constexpr int j = decltype(j_tag)::value;
             static_for<8>([&](auto s_tag) ES_INLINE {
@@ -425,18 +451,18 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_shortk_kernel(gemm_args_t a,
                     tr::mma(acc[j][i], fb[n % 4], fa[i][s]);
                     if constexpr (i == 0 && n + 3 < 16) {
                         constexpr int s2 = (n + 3) % 8, j2 = (n + 3) / 8;
-                        fb[(n + 3) % 4] = *(lds_chunk_ptr)(fb_at[s2] + j2 * 32 * SK_RB);
+                        fb[(n + 3) % 4] = *(lds_chunk_ptr)(uintptr_t)(fb_at[s2] + j2 * 32 * SK_RB);
                     }
                     if constexpr (j == 0 && PREV) {
                         // j = 1 of the tile before, and its packed j = 0
                         uint32_t const w = pack(integral_constant<int, 1>{}, integral_constant<int, h>{});
                         if constexpr (h % 2 == 0) {
                             held = w;
-                            stage_quad(stage, integral_constant<int, 0>{},
-                                       integral_constant<int, h / 2>{}, packed[h], packed[h + 1]);
+                            stage_quad(integral_constant<int, 0>{}, integral_constant<int, h / 2>{},
+                                       packed[h], packed[h + 1]);
                         } else {
-                            stage_quad(stage, integral_constant<int, 1>{},
-                                       integral_constant<int, h / 2>{}, held, w);
+                            stage_quad(integral_constant<int, 1>{}, integral_constant<int, h / 2>{},
+                                       held, w);
                         }
                     }
                     if constexpr (j == 1) {
@@ -472,17 +498,16 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_shortk_kernel(gemm_args_t a,
     }
     // the last tile
     {
-        char* const stage = stage_lane + ((steps - 1) & 1) * SK_OUT;
+        stage_into((steps - 1) & 1);
         static_for<16>([&](auto h_tag) ES_INLINE {
             constexpr int  h = decltype(h_tag)::value;
             uint32_t const w = pack(integral_constant<int, 1>{}, h_tag);
             if constexpr (h % 2 == 0) {
                 held = w;
-                stage_quad(stage, integral_constant<int, 0>{}, integral_constant<int, h / 2>{},
-                           packed[h], packed[h + 1]);
+                stage_quad(integral_constant<int, 0>{}, integral_constant<int, h / 2>{}, packed[h],
+                           packed[h + 1]);
             } else {
-                stage_quad(stage, integral_constant<int, 1>{}, integral_constant<int, h / 2>{},
-                           held, w);
+                stage_quad(integral_constant<int, 1>{}, integral_constant<int, h / 2>{}, held, w);
             }
         });
     }
