@@ -15,7 +15,7 @@
 //
 // Barriers: every one is executed by all eight waves.  Per slice g one barrier says both
 // "the multiplying waves have read all of slice g" (its stage may be overwritten) and "slice
-// g + 1 has landed".  Per tile 2 TM - 1 more hand the strips to and fro.  Both roles count
+// g + 1 has landed".  Per tile 2 (BM / 64) - 1 more hand the strips to and fro.  Both roles count
 // them from the same uniform numbers.
 #pragma once
 #include "gemm_w4_kernel.h"
@@ -34,7 +34,10 @@ __global__ __launch_bounds__(512) void gemm_pc_kernel(gemm_args_t a, uint32_t to
     using T = _Float16;
     using std::integral_constant;
     constexpr int NS = 3;
-    constexpr int MI = 32, VL = 8, WGN = 2;
+    constexpr int MI = 16, VL = 8, WGN = 2;
+    constexpr int KS = BK / 32;  // k-steps (16 x 16 x 32 matrix instructions along k) per slice
+    constexpr int BAND = 32;     // rows per turn of the epilogue
+    constexpr int TMB = BM / 2 / BAND;
     constexpr int WM = BM / 2, WN = BN / 2;
     constexpr int TM = WM / MI, TN = WN / MI;
     constexpr int NT = TM * TN;  // accumulator tiles per multiplying wave
@@ -43,11 +46,11 @@ __global__ __launch_bounds__(512) void gemm_pc_kernel(gemm_args_t a, uint32_t to
     constexpr int NLA = BM / 32, NLB = BN / 32;  // load instructions per loading wave per slice
     constexpr int LP = NLA + NLB;
     constexpr int READS = TM + TN;
-    static_assert(NT * 16 <= 128 && READS < NT, "");
+    static_assert(NT * 4 <= 128 && READS < NT && KS == 2, "");
     constexpr int STRIP_PITCH = WN * int(sizeof(T)) + 16;
     constexpr int CPR = WN * int(sizeof(T)) / 16;  // 16-byte chunks per strip row
-    constexpr int CPL = MI * CPR / 64;             // chunks per lane per band
-    static_assert(4 * MI * STRIP_PITCH <= STAGE, "");
+    constexpr int CPL = BAND * CPR / 64;           // chunks per lane per band
+    static_assert(4 * BAND * STRIP_PITCH <= STAGE, "");
 
     extern __shared__ __attribute__((aligned(16))) char lds[];
     uint32_t const lds_base = uint32_t(uintptr_t((__attribute__((address_space(3))) char*)lds));
@@ -91,14 +94,14 @@ __global__ __launch_bounds__(512) void gemm_pc_kernel(gemm_args_t a, uint32_t to
 
     if (wave < 4) {
         // ================================================================ multiplying waves
-        static_for<NT * 16>([](auto r) ES_INLINE { acc_clear<decltype(r)::value>(); });
-        // k-step s, MFMA tile row r0 + lane % 32: k-chunk 2 s + lane / 32, found in slot
+        static_for<NT * 4>([](auto r) ES_INLINE { acc_clear<decltype(r)::value>(); });
+        // k-step s, MFMA tile row r0 + lane % 16: k-chunk 4 s + lane / 16, found in slot
         // chunk ^ bits 1..3 of the row
         int const f_sw = ((lane % MI) >> 1) & 7;
-        int       f_off[STEPS];
+        int       f_off[KS];
 #pragma unroll
-        for (int s = 0; s != STEPS; ++s) {
-            f_off[s] = (lane % MI) * RB + (((2 * s + lane / MI) ^ f_sw) * 16);
+        for (int s = 0; s != KS; ++s) {
+            f_off[s] = (lane % MI) * RB + (((4 * s + lane / MI) ^ f_sw) * 16);
         }
         int const fa_base = wm * WM * RB;
         int const fb_base = A_BYTES + wn * WN * RB;
@@ -121,11 +124,11 @@ __global__ __launch_bounds__(512) void gemm_pc_kernel(gemm_args_t a, uint32_t to
             uint32_t const nx = st + 1 == NS ? 0 : st + 1;
             char const*    cur = lds + st * STAGE;
             char const*    nxt = lds + nx * STAGE;
-            static_for<STEPS - 1>([&](auto s_tag) ES_INLINE {
+            static_for<KS - 1>([&](auto s_tag) ES_INLINE {
                 constexpr int s = decltype(s_tag)::value;
                 static_for<NT>([&](auto q_tag) ES_INLINE {
                     constexpr int q = decltype(q_tag)::value;
-                    mma<q>(fb[s & 1][q % TN], fa[s & 1][q / TN]);
+                    mma16<q>(fb[s & 1][q % TN], fa[s & 1][q / TN]);
                     if constexpr (q < READS) {
                         read_frag(cur, integral_constant<int, s + 1>{}, q_tag, fa[(s + 1) & 1],
                                   fb[(s + 1) & 1]);
@@ -135,7 +138,7 @@ __global__ __launch_bounds__(512) void gemm_pc_kernel(gemm_args_t a, uint32_t to
             });
             static_for<NT>([&](auto q_tag) ES_INLINE {
                 constexpr int q = decltype(q_tag)::value;
-                mma<q>(fb[1][q % TN], fa[1][q / TN]);
+                mma16<q>(fb[(KS - 1) & 1][q % TN], fa[(KS - 1) & 1][q / TN]);
                 if constexpr (q == 0) {
                     // all of this stage has been read; behind the barrier the next has landed
                     asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");
@@ -148,16 +151,19 @@ __global__ __launch_bounds__(512) void gemm_pc_kernel(gemm_args_t a, uint32_t to
             });
             st = nx;
         };
-        // 32 rows of this wave's part of C, converted: band I, the lane's row lane % 32, four
-        // consecutive n per register pair; the accumulators are cleared on the way
+        // 32 rows of this wave's part of C, converted: band I holds the accumulator tiles of rows
+        // 32 I .. 32 I + 31 (quad g: row 16 (g / TN) + lane % 16 of the band, the four
+        // consecutive n from 16 (g % TN) + lane / 16 * 4 on); the accumulators are cleared on
+        // the way
         float const alpha = float(a.alpha);
         typedef T   quad_t __attribute__((ext_vector_type(4)));
-        quad_t      band[TN * 4];
+        constexpr int QB = (BAND / MI) * TN;  // quads per band
+        quad_t      band[QB];
         auto convert = [&](auto i_tag) ES_INLINE {
             constexpr int i = decltype(i_tag)::value;
-            static_for<TN * 4>([&](auto g_tag) ES_INLINE {
+            static_for<QB>([&](auto g_tag) ES_INLINE {
                 constexpr int g = decltype(g_tag)::value;
-                constexpr int R = (i * TN + g / 4) * 16 + (g % 4) * 4;
+                constexpr int R = (i * QB + g) * 4;
                 quad_t        q;
                 q[0] = T(acc_read<R>() * alpha);
                 q[1] = T(acc_read<R + 1>() * alpha);
@@ -182,24 +188,24 @@ __global__ __launch_bounds__(512) void gemm_pc_kernel(gemm_args_t a, uint32_t to
             for (uint32_t kt = 0; kt + 1 < nk; ++kt) slice();
             uint32_t const freed = st;
             slice();
-            char* const strip = lds + freed * STAGE + role_wave * (MI * STRIP_PITCH);
+            char* const strip = lds + freed * STAGE + role_wave * (BAND * STRIP_PITCH);
 #ifdef ES_W4_STAMP
             uint64_t const stamp1 = __builtin_amdgcn_s_memtime();
 #endif
             settle();
             convert(integral_constant<int, 0>{});
-            static_for<TM>([&](auto i_tag) ES_INLINE {
+            static_for<TMB>([&](auto i_tag) ES_INLINE {
                 constexpr int i = decltype(i_tag)::value;
                 if constexpr (i > 0) __builtin_amdgcn_s_barrier();  // the strips have been read
-                static_for<TN * 4>([&](auto g_tag) ES_INLINE {
+                static_for<QB>([&](auto g_tag) ES_INLINE {
                     constexpr int g = decltype(g_tag)::value;
-                    int const     n = (g / 4) * MI + (g % 4) * 8 + (lane / 32) * 4;
-                    *reinterpret_cast<quad_t*>(strip + (lane % MI) * STRIP_PITCH +
+                    int const     n = (g % TN) * MI + (lane / MI) * 4;
+                    *reinterpret_cast<quad_t*>(strip + ((g / TN) * MI + lane % MI) * STRIP_PITCH +
                                                n * int(sizeof(T))) = band[g];
                 });
                 asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");
                 __builtin_amdgcn_s_barrier();  // the strips are written
-                if constexpr (i + 1 < TM) convert(integral_constant<int, i + 1>{});
+                if constexpr (i + 1 < TMB) convert(integral_constant<int, i + 1>{});
             });
 #ifdef ES_W4_STAMP
             {
@@ -359,8 +365,8 @@ __global__ __launch_bounds__(512) void gemm_pc_kernel(gemm_args_t a, uint32_t to
             }
         }
         T* const          C = static_cast<T*>(a.C) + boc;
-        char const* const strip = lds + freed * STAGE + role_wave * (MI * STRIP_PITCH);
-        static_for<TM>([&](auto i_tag) ES_INLINE {
+        char const* const strip = lds + freed * STAGE + role_wave * (BAND * STRIP_PITCH);
+        static_for<TMB>([&](auto i_tag) ES_INLINE {
             constexpr int i = decltype(i_tag)::value;
             __builtin_amdgcn_s_barrier();  // the strips are written
             chunk_t v[CPL];
@@ -371,11 +377,11 @@ __global__ __launch_bounds__(512) void gemm_pc_kernel(gemm_args_t a, uint32_t to
                                                          (idx % CPR) * 16);
             }
             asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");
-            if constexpr (i + 1 < TM) __builtin_amdgcn_s_barrier();  // the strips have been read
+            if constexpr (i + 1 < TMB) __builtin_amdgcn_s_barrier();  // the strips have been read
 #pragma unroll
             for (int c = 0; c != CPL; ++c) {
                 int const      idx = c * 64 + lane;
-                uint32_t const m = t.tm * BM + wm * WM + i * MI + uint32_t(idx / CPR);
+                uint32_t const m = t.tm * BM + wm * WM + i * BAND + uint32_t(idx / CPR);
                 uint32_t const n = t.tn * BN + wn * WN + uint32_t(idx % CPR) * VL;
                 if (m < a.M && n < a.N) {
                     int64_t mo_a, mo_c, no_b, no_c;

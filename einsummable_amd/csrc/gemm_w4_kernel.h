@@ -63,6 +63,20 @@ __device__ __forceinline__ void mma(chunk_t const& x, chunk_t const& y)
                  : "n"(16 * T), "n"(16 * T + 15), "v"(x), "v"(y));
 }
 
+// The 16 x 16 x 32 instruction on accumulator tile T (a[4 T .. 4 T + 3]): x holds, per lane,
+// eight k elements (k = lane / 16 * 8 ..) of row lane % 16 of the 16 rows of the result, y
+// the same of its 16 columns; the lane gets rows lane / 16 * 4 .. + 3 of column lane % 16.
+// Per flop it moves half the accumulator registers of the 32 x 32 x 16 instruction, and under
+// the board's power limit that is worth a tenth of the clock: the same kernel, instruction
+// exchanged, ran 8192^3 at 1449 instead of 1311 TFLOP/s.
+template <int T>
+__device__ __forceinline__ void mma16(chunk_t const& x, chunk_t const& y)
+{
+    asm volatile("v_mfma_f32_16x16x32_f16 a[%0:%1], %2, %3, a[%0:%1]"
+                 :
+                 : "n"(4 * T), "n"(4 * T + 3), "v"(x), "v"(y));
+}
+
 // the same with a zero addend: the first product of a sum
 template <int T>
 __device__ __forceinline__ void mma_first(chunk_t const& x, chunk_t const& y)
@@ -151,7 +165,9 @@ template <int BM, int BN, int NS, bool KW>
 __global__ __launch_bounds__(256) void gemm_w4_kernel(gemm_args_t a, uint32_t total_tiles)
 {
     using T = _Float16;
-    constexpr int MI = 32, VL = 8, NW = 4, WGN = 2;
+    constexpr int MI = 16, VL = 8, NW = 4, WGN = 2;
+    constexpr int KS = BK / 32;  // k-steps (matrix instructions along k) per slice
+    constexpr int BAND = 32;     // rows per turn of the epilogue
     constexpr int WM = BM / 2, WN = BN / 2;
     constexpr int TM = WM / MI, TN = WN / MI;
     constexpr int NT = TM * TN;  // accumulator tiles per wave
@@ -164,8 +180,9 @@ __global__ __launch_bounds__(256) void gemm_w4_kernel(gemm_args_t a, uint32_t to
     // that frees the stage, the others in the first k-steps of the slice after it.  With two
     // stages a load must land within one slice of being issued: two parts; with three there
     // is a slice more
-    constexpr int PARTS = NS >= 3 ? STEPS : 2;
-    static_assert(NT * 16 <= 256 && READS < NT && LOADS % PARTS == 0, "");
+    constexpr int PARTS = 2;
+    static_assert(NS == 2 && KS == 2, "the schedule below: two stages, two k-steps per slice");
+    static_assert(NT * 4 <= 256 && READS < NT / 2 && LOADS % PARTS == 0 && NT % 2 == 0, "");
 
     extern __shared__ __attribute__((aligned(16))) char lds[];
     uint32_t const lds_base = uint32_t(uintptr_t((__attribute__((address_space(3))) char*)lds));
@@ -177,7 +194,7 @@ __global__ __launch_bounds__(256) void gemm_w4_kernel(gemm_args_t a, uint32_t to
     uint32_t const lds_wave = lds_base + uint32_t(wave) * 1024;
 
     claim_accumulators();
-    static_for<NT * 16>([](auto r) ES_INLINE { acc_clear<decltype(r)::value>(); });
+    static_for<NT * 4>([](auto r) ES_INLINE { acc_clear<decltype(r)::value>(); });
 
     uint32_t const n_tiles = a.tiles_m * a.tiles_n;
     uint32_t const nk = a.K / BK;  // >= NS (checked by the launcher)
@@ -309,13 +326,13 @@ __global__ __launch_bounds__(256) void gemm_w4_kernel(gemm_args_t a, uint32_t to
     };
 
     // ---- fragments
-    // k-step s, MFMA tile row r0 + lane % 32: k-chunk 2 s + lane / 32, found in slot
+    // k-step s, MFMA tile row r0 + lane % 16: k-chunk 4 s + lane / 16, found in slot
     // chunk ^ bits 1..3 of the row
     int const f_sw = ((lane % MI) >> 1) & 7;
-    int       f_off[STEPS];
+    int       f_off[KS];
 #pragma unroll
-    for (int s = 0; s != STEPS; ++s) {
-        f_off[s] = (lane % MI) * RB + (((2 * s + lane / MI) ^ f_sw) * 16);
+    for (int s = 0; s != KS; ++s) {
+        f_off[s] = (lane % MI) * RB + (((4 * s + lane / MI) ^ f_sw) * 16);
     }
     int const fa_base = wm * WM * RB;
     int const fb_base = A_BYTES + wn * WN * RB;
@@ -354,35 +371,32 @@ __global__ __launch_bounds__(256) void gemm_w4_kernel(gemm_args_t a, uint32_t to
     });
 
     // One slice, computed from stage st, in two halves with the loader's step between them.
-    // k-steps 0 .. 2: the other parts of the loader's slice go to the stage before st.
+    // k-step 0: the fragments of k-step 1 are read, and the second part of the loader's slice
+    // goes to the stage before st -- in the first half of the step, a load per four matrix
+    // instructions (more would fill the load path; later ones would land too late).
     uint32_t st = 0;  // stage of the slice being computed
     auto head = [&]() ES_INLINE {
         char const*    cur = lds + st * STAGE;
         uint32_t const ld_slot = lds_wave + (st == 0 ? NS - 1 : st - 1) * STAGE;
-        static_for<STEPS - 1>([&](auto s_tag) ES_INLINE {
-            constexpr int s = decltype(s_tag)::value;
-            static_for<NT>([&](auto q_tag) ES_INLINE {
-                constexpr int q = decltype(q_tag)::value;
-                mma<q>(fb[s & 1][q % TN], fa[s & 1][q / TN]);
-                if constexpr (q < READS) {
-                    read_frag(cur, integral_constant<int, s + 1>{}, q_tag, fa[(s + 1) & 1],
-                              fb[(s + 1) & 1]);
-                }
-                if constexpr (s + 1 < PARTS) {
-                    // part s + 1 of the loader's slice, spread over the step
-                    constexpr int lo = (s + 1) * LOADS / PARTS, n = LOADS / PARTS;
-                    static_for<(q + 1) * n / NT - q * n / NT>([&](auto r_tag) ES_INLINE {
-                        issue(ld_slot,
-                              integral_constant<int, lo + q * n / NT + decltype(r_tag)::value>{});
-                    });
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            });
+        static_for<NT>([&](auto q_tag) ES_INLINE {
+            constexpr int q = decltype(q_tag)::value;
+            mma16<q>(fb[0][q % TN], fa[0][q / TN]);
+            if constexpr (q < READS) {
+                read_frag(cur, integral_constant<int, 1>{}, q_tag, fa[1], fb[1]);
+            }
+            if constexpr (q < NT / 2) {
+                constexpr int lo = LOADS / PARTS, n = LOADS / PARTS, h = NT / 2;
+                static_for<(q + 1) * n / h - q * n / h>([&](auto r_tag) ES_INLINE {
+                    issue(ld_slot, integral_constant<int, lo + q * n / h + decltype(r_tag)::value>{});
+                });
+            }
+            __builtin_amdgcn_sched_barrier(0);
         });
     };
-    // The last k-step: the next slice has landed, this stage is free and takes part 0 of the
-    // loader's new slice -- unless this is the tile's LAST slice: then the freed stage is the
-    // epilogue's first.
+    // k-step 1.  Half-way through it the next slice must have landed; this stage has been
+    // read in full by then (its k-step 1 went to registers during k-step 0), so behind the
+    // barrier it takes the first part of the loader's new slice -- unless this is the tile's
+    // LAST slice: then the freed stage is the epilogue's first.
     auto tail = [&](auto last_tag) ES_INLINE {
         constexpr bool LAST = decltype(last_tag)::value;
         uint32_t const nx = st + 1 == NS ? 0 : st + 1;
@@ -390,22 +404,23 @@ __global__ __launch_bounds__(256) void gemm_w4_kernel(gemm_args_t a, uint32_t to
         uint32_t const ld_slot = lds_wave + st * STAGE;
         static_for<NT>([&](auto q_tag) ES_INLINE {
             constexpr int q = decltype(q_tag)::value;
-            mma<q>(fb[1][q % TN], fa[1][q / TN]);
-            if constexpr (q == 0) {
+            mma16<q>(fb[1][q % TN], fa[1][q / TN]);
+            if constexpr (q == NT / 2) {
                 // this wave's part of the next slice has landed and its reads of this stage
                 // are complete; after the barrier that holds for the whole workgroup
                 wait_vm_lgkm<(NS - 2) * LOADS>();
                 __builtin_amdgcn_s_barrier();
-            } else {
-                if constexpr (q - 1 < READS) {
-                    read_frag(nxt, integral_constant<int, 0>{}, integral_constant<int, q - 1>{},
-                              fa[0], fb[0]);
+            } else if constexpr (q > NT / 2) {
+                constexpr int r = q - NT / 2 - 1, left = NT / 2 - 1;
+                if constexpr (r < READS) {
+                    read_frag(nxt, integral_constant<int, 0>{}, integral_constant<int, r>{}, fa[0],
+                              fb[0]);
                 }
                 if constexpr (!LAST) {
                     constexpr int n = LOADS / PARTS;
-                    static_for<q * n / (NT - 1) - (q - 1) * n / (NT - 1)>([&](auto r_tag) ES_INLINE {
-                        issue(ld_slot, integral_constant<int, (q - 1) * n / (NT - 1) +
-                                                                  decltype(r_tag)::value>{});
+                    static_for<(r + 1) * n / left - r * n / left>([&](auto r_tag) ES_INLINE {
+                        issue(ld_slot,
+                              integral_constant<int, r * n / left + decltype(r_tag)::value>{});
                     });
                 }
             }
@@ -420,8 +435,8 @@ __global__ __launch_bounds__(256) void gemm_w4_kernel(gemm_args_t a, uint32_t to
     // are read back before the first store, so the LDS latency is paid once per band.
     constexpr int STRIP_PITCH = WN * int(sizeof(T)) + 16;
     constexpr int CPR = WN * int(sizeof(T)) / 16;
-    constexpr int CPL = MI * CPR / 64;  // chunks per lane per band
-    static_assert(NW * MI * STRIP_PITCH <= STAGE, "");
+    constexpr int CPL = BAND * CPR / 64;  // chunks per lane per band
+    static_assert(NW * BAND * STRIP_PITCH <= STAGE, "");
     float const alpha = float(a.alpha);
     auto epilogue = [&](uint32_t L, uint32_t freed_stage) ES_INLINE {
         tile_t const t = locate(L);
@@ -439,7 +454,7 @@ __global__ __launch_bounds__(256) void gemm_w4_kernel(gemm_args_t a, uint32_t to
             }
         }
         T* const    C = static_cast<T*>(a.C) + boc;
-        char* const strip = lds + freed_stage * STAGE + wave * (MI * STRIP_PITCH);
+        char* const strip = lds + freed_stage * STAGE + wave * (BAND * STRIP_PITCH);
         typedef T   quad_t __attribute__((ext_vector_type(4)));
         // this lane's chunks of a band: rows lane / CPR + c * (64 / CPR), 16 bytes at
         // (lane % CPR) * 8 elements
@@ -452,13 +467,16 @@ __global__ __launch_bounds__(256) void gemm_w4_kernel(gemm_args_t a, uint32_t to
         char* const    c_lin = reinterpret_cast<char*>(C) + int64_t(t.tm * BM + wm * WM) * a.gm.sy[0] * int64_t(sizeof(T));
         uint32_t const v_lin = uint32_t(lane / CPR) * ldc_bytes + n0 * uint32_t(sizeof(T));
         settle();
-        static_for<TM>([&](auto i_tag) ES_INLINE {
+        // band i: the accumulator tiles of rows 32 i .. 32 i + 31; a tile's lane holds column
+        // lane % 16 of the instruction's result, i.e. row lane % 16 of C, and four
+        // consecutive n from lane / 16 * 4 on
+        static_for<WM / BAND>([&](auto i_tag) ES_INLINE {
             constexpr int i = decltype(i_tag)::value;
-            static_for<TN>([&](auto j_tag) ES_INLINE {
-                constexpr int j = decltype(j_tag)::value;
-                static_for<4>([&](auto g_tag) ES_INLINE {
-                    constexpr int e0 = decltype(g_tag)::value * 4;
-                    constexpr int R = (i * TN + j) * 16 + e0;
+            static_for<BAND / MI>([&](auto h_tag) ES_INLINE {
+                constexpr int h = decltype(h_tag)::value;
+                static_for<TN>([&](auto j_tag) ES_INLINE {
+                    constexpr int j = decltype(j_tag)::value;
+                    constexpr int R = ((i * (BAND / MI) + h) * TN + j) * 4;
                     quad_t        q;
                     q[0] = T(acc_read<R>() * alpha);
                     q[1] = T(acc_read<R + 1>() * alpha);
@@ -468,8 +486,8 @@ __global__ __launch_bounds__(256) void gemm_w4_kernel(gemm_args_t a, uint32_t to
                     acc_clear<R + 1>();
                     acc_clear<R + 2>();
                     acc_clear<R + 3>();
-                    int const n = j * MI + (e0 / 4) * 8 + (lane / 32) * 4;
-                    *reinterpret_cast<quad_t*>(strip + (lane % MI) * STRIP_PITCH +
+                    int const n = j * MI + (lane / MI) * 4;
+                    *reinterpret_cast<quad_t*>(strip + (h * MI + lane % MI) * STRIP_PITCH +
                                                n * int(sizeof(T))) = q;
                 });
             });
@@ -485,7 +503,7 @@ __global__ __launch_bounds__(256) void gemm_w4_kernel(gemm_args_t a, uint32_t to
             }
 #pragma unroll
             for (int c = 0; c != CPL; ++c) {
-                uint32_t const m = m0 + uint32_t(i * MI + c * (64 / CPR));
+                uint32_t const m = m0 + uint32_t(i * BAND + c * (64 / CPR));
 #ifdef ES_W4_ABL_NO_STORE
                 if (m < a.M && n0 < a.N && v[c][0] == 0x12345678u) {
 #else
@@ -494,7 +512,7 @@ __global__ __launch_bounds__(256) void gemm_w4_kernel(gemm_args_t a, uint32_t to
                     chunk_t* dst;
                     if (lin) {
                         dst = reinterpret_cast<chunk_t*>(
-                            c_lin + (v_lin + uint32_t(i * MI + c * (64 / CPR)) * ldc_bytes));
+                            c_lin + (v_lin + uint32_t(i * BAND + c * (64 / CPR)) * ldc_bytes));
                     } else {
                         int64_t mo_a, mo_c, no_b, no_c;
                         group_offsets(a.gm, m, mo_a, mo_c);
