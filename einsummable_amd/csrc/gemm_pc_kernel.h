@@ -28,6 +28,16 @@ namespace pc
 {
 using namespace w4;
 
+// Fragment read i of R goes behind matrix instruction i (N - 1) / R of a k-step's N: the index of
+// the read behind instruction q, or -1
+constexpr int spread_read(int q, int n, int r)
+{
+    for (int i = 0; i != r; ++i) {
+        if (i * (n - 1) / r == q) return i;
+    }
+    return -1;
+}
+
 template <int BM, int BN, bool KW>
 __global__ __launch_bounds__(512) void gemm_pc_kernel(gemm_args_t a, uint32_t total_tiles)
 {
@@ -119,6 +129,10 @@ __global__ __launch_bounds__(512) void gemm_pc_kernel(gemm_args_t a, uint32_t to
                                                                (q - TN) * MI * RB + f_off[s]);
             }
         };
+        // The four multiplying waves share one LDS port of 128 bytes a cycle and a fragment
+        // read is 1 KiB per wave, a matrix instruction 16 cycles: one read per instruction
+        // from every wave asks for twice what the port gives, and the instructions behind
+        // the full queue wait.  Read i of a k-step goes behind instruction i (NT - 1) / READS.
         uint32_t st = 0;  // stage of the slice being computed
         auto slice = [&]() ES_INLINE {
             uint32_t const nx = st + 1 == NS ? 0 : st + 1;
@@ -129,8 +143,9 @@ __global__ __launch_bounds__(512) void gemm_pc_kernel(gemm_args_t a, uint32_t to
                 static_for<NT>([&](auto q_tag) ES_INLINE {
                     constexpr int q = decltype(q_tag)::value;
                     mma16<q>(fb[s & 1][q % TN], fa[s & 1][q / TN]);
-                    if constexpr (q < READS) {
-                        read_frag(cur, integral_constant<int, s + 1>{}, q_tag, fa[(s + 1) & 1],
+                    if constexpr (spread_read(q, NT, READS) >= 0) {
+                        read_frag(cur, integral_constant<int, s + 1>{},
+                                  integral_constant<int, spread_read(q, NT, READS)>{}, fa[(s + 1) & 1],
                                   fb[(s + 1) & 1]);
                     }
                     __builtin_amdgcn_sched_barrier(0);
@@ -143,9 +158,9 @@ __global__ __launch_bounds__(512) void gemm_pc_kernel(gemm_args_t a, uint32_t to
                     // all of this stage has been read; behind the barrier the next has landed
                     asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");
                     __builtin_amdgcn_s_barrier();
-                } else if constexpr (q - 1 < READS) {
-                    read_frag(nxt, integral_constant<int, 0>{}, integral_constant<int, q - 1>{},
-                              fa[0], fb[0]);
+                } else if constexpr (spread_read(q - 1, NT, READS) >= 0) {
+                    read_frag(nxt, integral_constant<int, 0>{},
+                              integral_constant<int, spread_read(q - 1, NT, READS)>{}, fa[0], fb[0]);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             });

@@ -371,9 +371,18 @@ __global__ __launch_bounds__(256) void gemm_w4_kernel(gemm_args_t a, uint32_t to
     });
 
     // One slice, computed from stage st, in two halves with the loader's step between them.
-    // k-step 0: the fragments of k-step 1 are read, and the second part of the loader's slice
-    // goes to the stage before st -- in the first half of the step, a load per four matrix
-    // instructions (more would fill the load path; later ones would land too late).
+    // The four waves' fragment reads share one LDS port of 128 bytes a cycle, and a read is
+    // 1 KiB per wave: more than one read per two matrix instructions (16 cycles each) fills
+    // the port's queue and the matrix instructions behind it wait.  So the reads are spread:
+    // k-step 0 reads the fragments of k-step 1 one per four instructions, and -- one per
+    // eight, two rows of tiles ahead of their use -- the A fragments of its own k-step from
+    // the fourth on (JIT), which leaves the second half of k-step 1 with the eleven reads
+    // k-step 0 starts on.  The second part of the loader's slice goes to the stage before st
+    // in the first half of k-step 0, a load per four matrix instructions (more would fill
+    // the load path; later ones would land too late).
+    constexpr int JIT = 3;             // first A fragment of k-step 0 that k-step 0 reads itself
+    constexpr int EARLY = TN + JIT;    // reads of k-step 0 left to the k-step before it
+    static_assert(NT == 64 && TN == 8 && READS == 16 && LOADS / PARTS == 8, "");
     uint32_t st = 0;  // stage of the slice being computed
     auto head = [&]() ES_INLINE {
         char const*    cur = lds + st * STAGE;
@@ -381,14 +390,16 @@ __global__ __launch_bounds__(256) void gemm_w4_kernel(gemm_args_t a, uint32_t to
         static_for<NT>([&](auto q_tag) ES_INLINE {
             constexpr int q = decltype(q_tag)::value;
             mma16<q>(fb[0][q % TN], fa[0][q / TN]);
-            if constexpr (q < READS) {
-                read_frag(cur, integral_constant<int, 1>{}, q_tag, fa[1], fb[1]);
+            if constexpr (q % 4 == 1) {
+                read_frag(cur, integral_constant<int, 1>{}, integral_constant<int, q / 4>{}, fa[1],
+                          fb[1]);
             }
-            if constexpr (q < NT / 2) {
-                constexpr int lo = LOADS / PARTS, n = LOADS / PARTS, h = NT / 2;
-                static_for<(q + 1) * n / h - q * n / h>([&](auto r_tag) ES_INLINE {
-                    issue(ld_slot, integral_constant<int, lo + q * n / h + decltype(r_tag)::value>{});
-                });
+            if constexpr (q % TN == 0 && q / TN + 2 >= JIT && q / TN + 2 < TM) {
+                read_frag(cur, integral_constant<int, 0>{},
+                          integral_constant<int, TN + q / TN + 2>{}, fa[0], fb[0]);
+            }
+            if constexpr (q % 4 == 3 && q < NT / 2) {
+                issue(ld_slot, integral_constant<int, LOADS / PARTS + q / 4>{});
             }
             __builtin_amdgcn_sched_barrier(0);
         });
@@ -411,17 +422,13 @@ __global__ __launch_bounds__(256) void gemm_w4_kernel(gemm_args_t a, uint32_t to
                 wait_vm_lgkm<(NS - 2) * LOADS>();
                 __builtin_amdgcn_s_barrier();
             } else if constexpr (q > NT / 2) {
-                constexpr int r = q - NT / 2 - 1, left = NT / 2 - 1;
-                if constexpr (r < READS) {
-                    read_frag(nxt, integral_constant<int, 0>{}, integral_constant<int, r>{}, fa[0],
-                              fb[0]);
+                constexpr int r = q - NT / 2 - 1;
+                if constexpr (r % 3 == 0 && r / 3 < EARLY) {
+                    read_frag(nxt, integral_constant<int, 0>{}, integral_constant<int, r / 3>{},
+                              fa[0], fb[0]);
                 }
-                if constexpr (!LAST) {
-                    constexpr int n = LOADS / PARTS;
-                    static_for<(r + 1) * n / left - r * n / left>([&](auto r_tag) ES_INLINE {
-                        issue(ld_slot,
-                              integral_constant<int, r * n / left + decltype(r_tag)::value>{});
-                    });
+                if constexpr (!LAST && r % 3 == 1 && r / 3 < LOADS / PARTS) {
+                    issue(ld_slot, integral_constant<int, r / 3>{});
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
