@@ -18,8 +18,8 @@
 // padded to 144 bytes, which makes the 16-byte-per-lane fragment reads conflict free.  The
 // MFMA is issued with the B fragment as the row operand so that every lane ends up holding
 // four consecutive n of one m: the epilogue stores them with one 8 / 16-byte write.
-// fp16 inputs accumulate in fp32 (v_mfma_f32_32x32x16_f16), fp32 uses v_mfma_f32_32x32x2_f32,
-// f64 uses v_mfma_f64_16x16x4_f64.
+// fp16 inputs accumulate in fp32 (v_mfma_f32_32x32x16_f16; the persistent kernels use
+// v_mfma_f32_16x16x32_f16), fp32 uses v_mfma_f32_32x32x2_f32, f64 uses v_mfma_f64_16x16x4_f64.
 #include "gemm_dma_kernel.h"
 #include "gemm_pc_kernel.h"
 #include "gemm_kernel.h"

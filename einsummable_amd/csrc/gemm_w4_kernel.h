@@ -9,10 +9,10 @@
 //     holds 256 of them, all of a[0:255]; left to the register allocator they are split
 //     between a and v registers, moved to and fro around every matrix instruction and
 //     spilled.  Here the matrix instructions, the clearing and the reads are assembly
-//     statements on fixed registers (a[16 t : 16 t + 15] is accumulator tile t), so the main
-//     loop is matrix instructions, LDS reads and load issues and nothing else.  With one wave
-//     per SIMD a wave reads 0.5 LDS vectors per matrix instruction where two waves of
-//     128 x 64 read 0.75.
+//     statements on fixed registers (a[4 t : 4 t + 3] is accumulator tile t of 16 x 16), so
+//     the main loop is matrix instructions, LDS reads and load issues and nothing else.  With
+//     one wave per SIMD a wave reads 0.25 LDS vectors per matrix instruction where two waves
+//     of 128 x 64 read 0.375.
 //   * The load path of a compute unit takes 64 bytes per cycle and a 256 x 256 x 64 slice is
 //     64 KiB: half of the time the matrix instructions of the slice take.  Four waves that
 //     issue all their loads of a slice behind one barrier fill the queue and then stand at
@@ -54,16 +54,7 @@ __device__ __forceinline__ void static_for(F&& f)
     static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
-// accumulator tile T += x (rows of the instruction: n) * y (columns: m)
-template <int T>
-__device__ __forceinline__ void mma(chunk_t const& x, chunk_t const& y)
-{
-    asm volatile("v_mfma_f32_32x32x16_f16 a[%0:%1], %2, %3, a[%0:%1]"
-                 :
-                 : "n"(16 * T), "n"(16 * T + 15), "v"(x), "v"(y));
-}
-
-// The 16 x 16 x 32 instruction on accumulator tile T (a[4 T .. 4 T + 3]): x holds, per lane,
+// Accumulator tile T (a[4 T .. 4 T + 3]) += x * y with the 16 x 16 x 32 instruction: x holds, per lane,
 // eight k elements (k = lane / 16 * 8 ..) of row lane % 16 of the 16 rows of the result, y
 // the same of its 16 columns; the lane gets rows lane / 16 * 4 .. + 3 of column lane % 16.
 // Per flop it moves half the accumulator registers of the 32 x 32 x 16 instruction, and under
@@ -75,15 +66,6 @@ __device__ __forceinline__ void mma16(chunk_t const& x, chunk_t const& y)
     asm volatile("v_mfma_f32_16x16x32_f16 a[%0:%1], %2, %3, a[%0:%1]"
                  :
                  : "n"(4 * T), "n"(4 * T + 3), "v"(x), "v"(y));
-}
-
-// the same with a zero addend: the first product of a sum
-template <int T>
-__device__ __forceinline__ void mma_first(chunk_t const& x, chunk_t const& y)
-{
-    asm volatile("v_mfma_f32_32x32x16_f16 a[%0:%1], %2, %3, 0"
-                 :
-                 : "n"(16 * T), "n"(16 * T + 15), "v"(x), "v"(y));
 }
 
 template <int R>
@@ -158,7 +140,6 @@ __device__ __forceinline__ void wait_vm_lgkm()
 
 constexpr int RB = 128;  // bytes of k per row per slice
 constexpr int BK = 64;   // elements of k per slice
-constexpr int STEPS = 4; // k-steps (matrix instructions along k) per slice
 
 // KW: several k modes (the slice walker steps digit by digit); otherwise a slice is one stride on
 template <int BM, int BN, int NS, bool KW>
