@@ -1141,6 +1141,278 @@ cg_kernel_t gen_reduce_col(einsummable_t const& e, int max_vec)
 
 }  // namespace
 
+// ------------------------------------------------------------------- chains over rows
+//
+// One team of lanes per row, as in gen_reduce_row (the same team size, vector width and
+// order of accumulation: a sum comes out with the bits the reduction kernel gives it), but
+// the row's vectors stay in registers from the first stage to the last.
+cg_kernel_t gen_row_chain(cg_chain_t const& c, int max_vec)
+{
+    int const R = int(c.shape.size());
+    int const NE = int(c.exts.size());
+    int const NS = int(c.stages.size());
+    if (R < 1 || NS < 2 || NE < 1) throw ir_error("row chain: nothing to chain");
+    int const O = R - 1;
+    uint64_t const n = c.shape[size_t(R - 1)];
+    uint64_t n_rows = 1;
+    for (int m = 0; m != O; ++m) n_rows *= c.shape[size_t(m)];
+
+    // what every stage yields, and which inputs are whole rows
+    std::vector<dtype_t> result(static_cast<size_t>(NS));
+    std::vector<bool>    is_vec(static_cast<size_t>(NE));
+    for (int k = 0; k != NE; ++k) {
+        auto const& modes = c.exts[size_t(k)].modes;
+        for (size_t i = 1; i < modes.size(); ++i) {
+            if (modes[i] <= modes[i - 1]) throw ir_error("row chain: an input is permuted");
+        }
+        is_vec[size_t(k)] = !modes.empty() && modes.back() == R - 1;
+        if (c.exts[size_t(k)].dtype == dtype_t::c64) throw ir_error("row chain: complex input");
+    }
+    int vcap = max_vec;
+    bool any_vec = false;
+    for (int t = 0; t != NS; ++t) {
+        auto const& st = c.stages[size_t(t)];
+        result[size_t(t)] = st.join.out_dtype();
+        if (result[size_t(t)] == dtype_t::c64) throw ir_error("row chain: complex stage");
+        if (int(st.args.size()) != st.join.num_inputs()) throw ir_error("row chain: argument count");
+        bool const last = t + 1 == NS;
+        if (last && st.castable) throw ir_error("row chain: the last stage writes the tensor");
+        int smallest = int(dtype_size(result[size_t(t)]));
+        for (size_t h = 0; h != st.args.size(); ++h) {
+            int const a = st.args[h];
+            if (a >= NE || a < -t) throw ir_error("row chain: argument out of range");
+            if (!st.join.hole_dtypes[h]) throw ir_error("row chain: unused argument");
+            dtype_t const d = a >= 0 ? c.exts[size_t(a)].dtype : result[size_t(-1 - a)];
+            if (d != st.join.hole_dtypes[h].value()) throw ir_error("row chain: argument dtype");
+            if (a >= 0 && is_vec[size_t(a)]) {
+                if (!st.castable && !last) throw ir_error("row chain: a per-row step reads a whole row");
+                any_vec = true;
+            }
+            smallest = std::min(smallest, int(dtype_size(d)));
+        }
+        // the width the stage's own kernel would use (gen_reduce_row); stages that add must
+        // agree in it, the others do not care
+        if (st.castable) vcap = std::min(vcap, row_reduction_lane_elems(smallest));
+    }
+    if (!any_vec) throw ir_error("row chain: no stage reads a row");
+    for (int k = 0; k != NE; ++k) {
+        if (is_vec[size_t(k)] && dtype_size(c.exts[size_t(k)].dtype) == 8) vcap = std::min(vcap, 2);
+    }
+    int const V = pow2_divisor(n, std::max(1, vcap));
+    for (int t = 0; t != NS; ++t) {
+        auto const& st = c.stages[size_t(t)];
+        if (!st.castable) continue;
+        int smallest = int(dtype_size(result[size_t(t)]));
+        for (int a : st.args) {
+            smallest = std::min(smallest, int(dtype_size(a >= 0 ? c.exts[size_t(a)].dtype
+                                                                  : result[size_t(-1 - a)])));
+        }
+        if (pow2_divisor(n, std::min(max_vec, row_reduction_lane_elems(smallest))) != V) {
+            throw ir_error("row chain: stages deal a row to the lanes differently");
+        }
+    }
+    uint64_t const nvec = n / uint64_t(V);
+    int const      TEAM = env_int("ES_KM_RED_TEAM", (nvec >= 512) ? 256 : 64) == 256 ? 256 : 64;
+    int const      BLOCK = 256;
+    uint64_t const vpl = (nvec + uint64_t(TEAM) - 1) / uint64_t(TEAM);
+    if (vpl > 8) throw ir_error("row chain: the row does not fit the team's registers");
+    int const VPL = int(vpl);
+    uint64_t regs = 0;
+    for (int k = 0; k != NE; ++k) {
+        if (is_vec[size_t(k)]) regs += uint64_t(VPL) * uint64_t(V) * dtype_size(c.exts[size_t(k)].dtype) / 4;
+    }
+    if (regs > 128) throw ir_error("row chain: the row does not fit the team's registers");
+    // (a row reduction with fewer than 1024 rows of 16 steps and more is cut into slices)
+    if (TEAM == 256 && n_rows < 1024 && nvec >= uint64_t(TEAM) * 4 * 16) {
+        throw ir_error("row chain: the reduction would be split");
+    }
+
+    cg_kernel_t k;
+    k.kind = cg_kind::row_chain;
+    k.n_inns = NE;
+    k.vec = V;
+    uint64_t biggest = n_rows * n;
+    for (int e = 0; e != NE; ++e) {
+        uint64_t ne = 1;
+        for (int m : c.exts[size_t(e)].modes) ne *= c.shape[size_t(m)];
+        biggest = std::max(biggest, ne);
+    }
+    k.idx64 = biggest >= (1ull << 32) - 1;
+    auto param = [&](uint64_t v) {
+        k.params.push_back(v);
+        return "a.p[" + std::to_string(k.params.size() - 1) + "]";
+    };
+    std::string const p_rows = param(n_rows), p_nvec = param(nvec), p_n = param(n);
+    std::vector<std::string> p_shape(static_cast<size_t>(R));
+    for (int m = 0; m != R; ++m) p_shape[size_t(m)] = param(c.shape[size_t(m)]);
+    std::vector<std::vector<std::string>> p_str(static_cast<size_t>(NE));
+    for (int e = 0; e != NE; ++e) {
+        auto const& modes = c.exts[size_t(e)].modes;
+        p_str[size_t(e)].assign(size_t(R), "");
+        uint64_t stride = 1;
+        for (int i = int(modes.size()) - 1; i >= 0; --i) {
+            p_str[size_t(e)][size_t(modes[size_t(i)])] = param(stride);
+            stride *= c.shape[size_t(modes[size_t(i)])];
+        }
+    }
+
+    // the name: the stages' joins and castables, the shape's rank and the dtypes
+    {
+        uint32_t h = 2166136261u;
+        auto mix = [&](std::string const& text) {
+            for (char ch : text) h = (h ^ uint8_t(ch)) * 16777619u;
+        };
+        for (auto const& st : c.stages) {
+            mix(st.join.str());
+            mix(std::string(1, castable_to_char(st.castable)));
+            for (int a : st.args) mix(std::to_string(a) + ",");
+        }
+        for (auto const& e : c.exts) {
+            mix(dtype_name(e.dtype));
+            for (int m : e.modes) mix(std::to_string(m) + ".");
+        }
+        char buf[96];
+        std::snprintf(buf, sizeof(buf), "es_rowchain__%dstages_%dinputs__%s_%08x", NS, NE,
+                      dtype_name(result[size_t(NS - 1)]), h);
+        k.entry = buf;
+    }
+
+    std::ostringstream s;
+    s << PRELUDE;
+    s << "typedef " << (k.idx64 ? "unsigned long long" : "unsigned int") << " idx_t;\n";
+    for (int t = 0; t != NS; ++t) {
+        auto const& st = c.stages[size_t(t)];
+        emitter_t   em;
+        std::string r = em.emit(st.join.root);
+        s << "__device__ __forceinline__ " << compute_type(result[size_t(t)]) << " join_fn" << t << "(";
+        for (int i = 0; i != st.join.num_inputs(); ++i) {
+            s << (i ? ", " : "") << compute_type(st.join.hole_dtypes[size_t(i)].value()) << " x" << i;
+        }
+        s << ")\n{\n" << em.body.str() << "    return " << r << ";\n}\n";
+        if (st.castable) {
+            std::string const ACC = compute_type(result[size_t(t)]);
+            s << "__device__ __forceinline__ " << ACC << " comb" << t << "(" << ACC << " x, " << ACC
+              << " y) { return " << combine_expr(st.castable.value(), result[size_t(t)], "x", "y")
+              << "; }\n";
+        }
+    }
+    dtype_t const od = result[size_t(NS - 1)];
+    s << "struct args_t {\n    " << storage_type(od) << "* out;\n";
+    for (int e = 0; e != NE; ++e) {
+        s << "    const " << storage_type(c.exts[size_t(e)].dtype) << "* in" << e << ";\n";
+    }
+    s << "    idx_t p[" << k.params.size() << "];\n};\n";
+    s << "#define V " << V << "\n#define TEAM " << TEAM << "\n#define VPL " << VPL << "\n";
+    s << "extern \"C\" __global__ __launch_bounds__(" << BLOCK << ") void " << k.entry << "(args_t a)\n{\n";
+    s << "    const unsigned lane = threadIdx.x % TEAM;\n";
+    s << "    const idx_t row = ((idx_t)blockIdx.y * gridDim.x + blockIdx.x) * (" << BLOCK
+      << " / TEAM) + threadIdx.x / TEAM;\n";
+    // (with a team of 256 the workgroup holds one row: all of it leaves, or none)
+    s << "    if (row >= " << p_rows << ") return;\n";
+    s << "    const idx_t nvec = " << p_nvec << ";\n";
+    s << "    idx_t rem = row;\n";
+    for (int m = O - 1; m >= 1; --m) {
+        s << "    const idx_t d" << m << " = rem % " << p_shape[size_t(m)] << ";\n";
+        s << "    rem /= " << p_shape[size_t(m)] << ";\n";
+    }
+    if (O >= 1) s << "    const idx_t d0 = rem;\n";
+    for (int e = 0; e != NE; ++e) {
+        std::string off = "0";
+        for (int m = 0; m != O; ++m) {
+            if (!p_str[size_t(e)][size_t(m)].empty()) {
+                off += " + d" + std::to_string(m) + " * " + p_str[size_t(e)][size_t(m)];
+            }
+        }
+        s << "    const idx_t b" << e << " = " << off << ";\n";
+        std::string const T = storage_type(c.exts[size_t(e)].dtype);
+        if (is_vec[size_t(e)]) {
+            s << "    vec_t<" << T << ", V> r" << e << "[VPL];\n";
+        } else {
+            s << "    const " << compute_type(c.exts[size_t(e)].dtype) << " c" << e << " = cvt_in(a.in"
+              << e << "[b" << e << "]);\n";
+        }
+    }
+    // every load of the row before anything is stored: the output may lie on an input
+    s << "#pragma unroll\n    for (int i = 0; i != VPL; ++i) {\n";
+    s << "        const idx_t vv = lane + (idx_t)i * TEAM;\n";
+    s << "        if (vv < nvec) {\n";
+    for (int e = 0; e != NE; ++e) {
+        if (!is_vec[size_t(e)]) continue;
+        std::string const T = storage_type(c.exts[size_t(e)].dtype);
+        s << "            r" << e << "[i] = *reinterpret_cast<const vec_t<" << T << ", V>*>(a.in" << e
+          << " + (b" << e << " + vv * V));\n";
+    }
+    s << "        }\n    }\n";
+    auto call = [&](int t, std::string const& i, std::string const& j) {
+        auto const& st = c.stages[size_t(t)];
+        std::string x = "join_fn" + std::to_string(t) + "(";
+        for (size_t h = 0; h != st.args.size(); ++h) {
+            int const a = st.args[h];
+            x += h ? ", " : "";
+            if (a < 0) {
+                x += "s" + std::to_string(-1 - a);
+            } else if (is_vec[size_t(a)]) {
+                x += "cvt_in(r" + std::to_string(a) + "[" + i + "].v[" + j + "])";
+            } else {
+                x += "c" + std::to_string(a);
+            }
+        }
+        return x + ")";
+    };
+    auto rounded = [&](dtype_t d, std::string const& v) {
+        // through the dtype a kernel of its own would have stored it in
+        return d == dtype_t::f16 ? "(float)(f16)(" + v + ")" : v;
+    };
+    if (TEAM == 256) s << "    __shared__ double part[" << NS << "][4];\n";
+    for (int t = 0; t + 1 != NS; ++t) {
+        auto const&       st = c.stages[size_t(t)];
+        std::string const ACC = compute_type(result[size_t(t)]);
+        std::string const T = std::to_string(t);
+        if (!st.castable) {
+            s << "    const " << ACC << " s" << T << " = " << rounded(result[size_t(t)], call(t, "0", "0"))
+              << ";\n";
+            continue;
+        }
+        s << "    " << ACC << " acc" << T << " = " << identity_of(st.castable.value(), result[size_t(t)])
+          << ";\n";
+        s << "#pragma unroll\n    for (int i = 0; i != VPL; ++i) {\n";
+        s << "        if (lane + (idx_t)i * TEAM < nvec) {\n";
+        s << "#pragma unroll\n            for (int j = 0; j != V; ++j) acc" << T << " = comb" << T << "(acc"
+          << T << ", " << call(t, "i", "j") << ");\n";
+        s << "        }\n    }\n";
+        s << "#pragma unroll\n    for (int m = 32; m >= 1; m >>= 1) acc" << T << " = comb" << T << "(acc" << T
+          << ", lane_xor(acc" << T << ", m));\n";
+        if (TEAM == 256) {
+            s << "    if ((threadIdx.x & 63) == 0) part[" << T << "][threadIdx.x >> 6] = acc" << T << ";\n";
+            s << "    __syncthreads();\n";
+            s << "    acc" << T << " = comb" << T << "(comb" << T << "((" << ACC << ")part[" << T << "][0], ("
+              << ACC << ")part[" << T << "][1]), comb" << T << "((" << ACC << ")part[" << T << "][2], ("
+              << ACC << ")part[" << T << "][3]));\n";
+        }
+        s << "    const " << ACC << " s" << T << " = " << rounded(result[size_t(t)], "acc" + T) << ";\n";
+    }
+    s << "#pragma unroll\n    for (int i = 0; i != VPL; ++i) {\n";
+    s << "        const idx_t vv = lane + (idx_t)i * TEAM;\n";
+    s << "        if (vv < nvec) {\n";
+    s << "            vec_t<" << storage_type(od) << ", V> o;\n";
+    s << "#pragma unroll\n            for (int j = 0; j != V; ++j) o.v[j] = "
+      << (od == dtype_t::f16 ? "(f16)(" : "(") << call(NS - 1, "i", "j") << ");\n";
+    s << "            *reinterpret_cast<vec_t<" << storage_type(od) << ", V>*>(a.out + (row * " << p_n
+      << " + vv * V)) = o;\n";
+    s << "        }\n    }\n}\n";
+
+    k.source = s.str();
+    uint64_t const rows_per_block = uint64_t(BLOCK / TEAM);
+    k.grid = (n_rows + rows_per_block - 1) / rows_per_block;
+    k.block = unsigned(BLOCK);
+    k.out_inn_align.push_back(std::min(16, V * int(dtype_size(od))));
+    for (int e = 0; e != NE; ++e) {
+        k.out_inn_align.push_back(
+            std::min(16, (is_vec[size_t(e)] ? V : 1) * int(dtype_size(c.exts[size_t(e)].dtype))));
+    }
+    return k;
+}
+
 cg_kernel_t generate_kernel(einsummable_t const& e, int max_vec)
 {
     if (e.join_shape.size() > 12 || e.inns.size() > 8) {
@@ -1153,6 +1425,8 @@ cg_kernel_t generate_kernel(einsummable_t const& e, int max_vec)
     }
     return is_row_reduction(e) ? gen_reduce_row(e, max_vec) : gen_reduce_col(e, max_vec);
 }
+
+cg_kernel_t generate_row_chain(cg_chain_t const& c, int max_vec) { return gen_row_chain(c, max_vec); }
 
 bool is_row_reduction(einsummable_t const& e)
 {
@@ -1415,6 +1689,8 @@ struct codegen_plan_t : plan_t {
     variant_t         narrow;  // scalar accesses: for buffers that are not 16-byte aligned
 
     explicit codegen_plan_t(einsummable_t const& e_) : e(e_) {}
+    codegen_plan_t() = default;  // a chain of einsummables
+    bool has_narrow = true;
     bool waiting = false;  // the variants' kernels are not loaded yet
     void deferred(std::vector<plan_t*>& out) override
     {
@@ -1494,6 +1770,10 @@ struct codegen_plan_t : plan_t {
             launch(wide, stream, out, inns, workspace);
             return;
         }
+        if (!has_narrow) {
+            throw km_error(km_status::invalid,
+                           "this kernel needs its buffers aligned to 16 bytes");
+        }
         launch(narrow, stream, out, inns, workspace);
     }
 };
@@ -1537,6 +1817,30 @@ std::shared_ptr<plan_t> plan_codegen(einsummable_t const& e, int device, bool de
     if (p->wide.k.row_pairs) p->description += " row_pairs";
     if (p->wide.k.splits > 1) p->description += " splits=" + std::to_string(p->wide.k.splits);
     p->workspace_bytes = std::max(p->wide.k.ws_bytes, p->narrow.k.ws_bytes);
+    return p;
+}
+
+std::shared_ptr<plan_t> plan_row_chain(cg_chain_t const& c, int device)
+{
+    auto p = std::make_shared<codegen_plan_t>();
+    p->wide.k = generate_row_chain(c);  // throws ir_error when the chain has no kernel
+    if (p->wide.k.grid >= (1ull << 36) ||
+        8 * (1 + p->wide.k.n_inns) + 8 * p->wide.k.params.size() > 1000) {
+        throw ir_error("row chain: too large");
+    }
+    try {
+        p->narrow.k = generate_row_chain(c, 1);
+    } catch (ir_error const&) {
+        p->has_narrow = false;  // rows too long for one element per lane and step
+    }
+    p->n_inns = p->wide.k.n_inns;
+    if (device >= 0) {
+        load_kernel(p->wide, device, {});
+        if (p->has_narrow) load_kernel(p->narrow, device, {});
+    }
+    p->description = "row_chain stages=" + std::to_string(c.stages.size()) +
+                     " vec=" + std::to_string(p->wide.k.vec);
+    if (p->wide.k.idx64) p->description += " idx64";
     return p;
 }
 

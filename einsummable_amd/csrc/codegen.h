@@ -14,7 +14,7 @@
 namespace es
 {
 
-enum class cg_kind { elementwise, reduce_row, reduce_col };
+enum class cg_kind { elementwise, reduce_row, reduce_col, row_chain };
 
 // Everything needed to launch a generated kernel: the source, its entry point, the launch
 // geometry and the packed argument block minus the pointers.
@@ -42,6 +42,36 @@ struct cg_kernel_t {
 // Generate the kernel for a (merged) einsummable.  `max_vec` caps the vector width (1 forces
 // the scalar variant used when a buffer is not 16-byte aligned).
 cg_kernel_t generate_kernel(einsummable_t const& e, int max_vec = 16);
+
+// A chain of nodes over the rows of one tensor whose intermediate results never leave the
+// registers: reductions over a row (the innermost mode), pointwise steps on the per-row
+// values, and a last elementwise node that writes the tensor -- softmax (row max, sum of
+// exp(x - max), exp(x - max) / sum), normalisations.  Each row is held by a team of lanes,
+// read once and written once; every stage computes what its own kernel would have computed,
+// in the same order and with the same roundings (a stage's result passes through its output
+// dtype before the next stage uses it), so the last node's output is bit for bit what the
+// nodes give one after the other.  The reference runs such chains node by node
+// (src/engine/gpu/gpu_kernel_manager.cc:326-430 are its hand-matched pieces of softmax).
+struct cg_chain_t {
+    std::vector<uint64_t> shape;  // join shape of every stage; the last mode is the row
+    struct ext_t {
+        dtype_t          dtype;
+        std::vector<int> modes;  // increasing; with the last mode: a tensor read by vectors,
+                                 // without: one value per row (or per kernel)
+    };
+    std::vector<ext_t> exts;  // the chain's inputs, in the order of the kernel's pointers
+    struct stage_t {
+        scalarop_t                join;
+        std::optional<castable_t> castable;  // set: a reduction over the row
+        std::vector<int>          args;      // per hole: k >= 0 external k, -1 - t: stage t's result
+    };
+    // reductions and pointwise steps on per-row values in any order, then the elementwise node
+    std::vector<stage_t> stages;
+};
+
+// Throws ir_error when the chain has no such kernel (rows too long for the registers, inputs
+// that are gathered, a stage the row reduction would have split ...).
+cg_kernel_t generate_row_chain(cg_chain_t const& c, int max_vec = 16);
 
 // Elements of a row per lane and step in the generated row reductions, by the smallest element
 // among output and inputs: two reductions that agree in it (and in the row's length) add a

@@ -226,12 +226,15 @@ void apply_graph_t::storage_read(int storage_id, void* dst, uint64_t size) const
 
 std::string apply_graph_t::describe(int id) const
 {
-    static const char* names[] = {"einsummable", "touch", "constant", "lowertri",
-                                  "copy",        "dummy", "evict",    "load"};
+    static const char* names[] = {"einsummable", "touch", "constant", "lowertri", "copy",
+                                  "dummy",       "evict", "load",     "chain"};
     node_t const& n = nodes_[size_t(id)];
     std::string   s = names[int(n.kind)];
     for (mem_t const& m : n.mems) s += " " + std::to_string(m.offset) + ":" + std::to_string(m.size);
     if (n.kind == kind_t::einsummable) s += " | " + n.e.key();
+    if (n.kind == kind_t::chain) {
+        s += " | " + std::to_string(n.chain_stages) + " stages, the last " + n.e.key();
+    }
     return s;
 }
 
@@ -577,12 +580,247 @@ bool apply_graph_t::absorb_into_readers(int u)
     return true;
 }
 
+// Tries to make node v, an elementwise einsummable, the last stage of a chain over rows: the
+// producers of its per-row inputs (and of theirs) that are row reductions over v's shape or
+// pointwise nodes over its rows, whose outputs nobody else reads and which are deleted
+// afterwards.  Returns the number of nodes absorbed (0: v stays as it is).
+int apply_graph_t::fuse_row_chain(int v)
+{
+    int const n = int(nodes_.size());
+    node_t&   nv = nodes_[size_t(v)];
+    if (nv.kind != kind_t::einsummable || nv.e.has_aggregation() || nv.e.join.has_variables()) return 0;
+    int const R = int(nv.e.join_shape.size());
+    if (R < 2) return 0;
+    int const O = R - 1;
+    std::vector<uint64_t> const shape = nv.e.join_shape;
+    std::vector<uint64_t> const rows(shape.begin(), shape.begin() + O);
+
+    // members in the order found; producer_of[(member, slot)] = member index
+    std::vector<int> members{v};
+    struct link_t {
+        int member, slot, producer;
+    };
+    std::vector<link_t> links;
+    auto writer_of = [&](mem_t const& m, int before) {
+        for (int u = before - 1; u >= 0; --u) {
+            node_t const& nu = nodes_[size_t(u)];
+            if (nu.kind == kind_t::dummy || nu.kind == kind_t::evict) continue;
+            if (overlaps(nu.mems[0], m)) return same_range(nu.mems[0], m) ? u : -1;
+        }
+        return -1;
+    };
+    auto stage_kind = [&](einsummable_t const& e) {  // 1 reduction over the row, 2 pointwise on rows
+        if (e.join.has_variables()) return 0;
+        if (e.has_aggregation()) return e.join_shape == shape && e.out_rank == O ? 1 : 0;
+        return e.join_shape == rows ? 2 : 0;
+    };
+    for (size_t at = 0; at != members.size(); ++at) {
+        node_t const& nm = nodes_[size_t(members[at])];
+        for (size_t k = 0; k != nm.e.inns.size(); ++k) {
+            if (!is_iota(nm.e.inns[k], O)) continue;
+            int const u = writer_of(nm.mems[k + 1], members[at]);
+            if (u < 0 || nodes_[size_t(u)].kind != kind_t::einsummable) continue;
+            if (!stage_kind(nodes_[size_t(u)].e)) continue;
+            if (std::find(members.begin(), members.end(), u) == members.end()) members.push_back(u);
+            links.push_back({members[at], int(k), u});
+        }
+    }
+    if (members.size() < 2) return 0;
+
+    // A producer stays a member only if its output is read by members alone, through the
+    // links found, and deleted after the last of them.  One that does not qualify is an
+    // ordinary input; members that hang on it alone go with it.
+    auto qualifies = [&](int u, std::vector<int> const& in) {
+        mem_t const S = nodes_[size_t(u)].mems[0];
+        if (S.size == 0) return false;
+        for (size_t i = 1; i != nodes_[size_t(u)].mems.size(); ++i) {
+            if (overlaps(nodes_[size_t(u)].mems[i], S)) return false;
+        }
+        int  last_reader = -1;
+        bool deleted = false;
+        for (int w = u + 1; w < n && !deleted; ++w) {
+            node_t const& nw = nodes_[size_t(w)];
+            if (nw.kind == kind_t::dummy) {
+                deleted = nw.is_del && last_reader >= 0 && covers(nw.mems[0], S) &&
+                          std::binary_search(nw.deps.begin(), nw.deps.end(), last_reader);
+                continue;
+            }
+            bool reads = false;
+            for (size_t i = 1; i < nw.mems.size(); ++i) {
+                if (!overlaps(nw.mems[i], S)) continue;
+                bool linked = false;
+                for (link_t const& l : links) {
+                    linked = linked || (l.member == w && l.slot + 1 == int(i) && l.producer == u);
+                }
+                if (!linked || std::find(in.begin(), in.end(), w) == in.end()) return false;
+                reads = true;
+            }
+            if (reads) last_reader = w;
+            if (nw.kind != kind_t::evict && overlaps(nw.mems[0], S)) return false;
+        }
+        return deleted;
+    };
+    for (bool changed = true; changed;) {
+        changed = false;
+        for (size_t i = 1; i < members.size(); ++i) {
+            if (qualifies(members[i], members)) continue;
+            members.erase(members.begin() + long(i));
+            changed = true;
+            break;
+        }
+        // members no link from a member reaches any more
+        for (size_t i = 1; i < members.size() && !changed; ++i) {
+            bool reached = false;
+            for (link_t const& l : links) {
+                reached = reached || (l.producer == members[i] &&
+                                      std::find(members.begin(), members.end(), l.member) != members.end());
+            }
+            if (!reached) {
+                members.erase(members.begin() + long(i));
+                changed = true;
+            }
+        }
+    }
+    if (members.size() < 2) return 0;
+    std::sort(members.begin(), members.end());  // insertion order is a valid order of execution
+    bool any_reduction = false;
+    for (int m : members) any_reduction = any_reduction || nodes_[size_t(m)].e.has_aggregation();
+    if (!any_reduction) return 0;
+    auto stage_of = [&](int node) {
+        return int(std::find(members.begin(), members.end(), node) - members.begin());
+    };
+
+    // the chain's inputs and stages
+    cg_chain_t         c;
+    std::vector<mem_t> ext_mems;
+    c.shape = shape;
+    mem_t const P = nv.mems[0];
+    if (P.offset % 16) return 0;
+    for (int m : members) {
+        node_t const&       nm = nodes_[size_t(m)];
+        cg_chain_t::stage_t st;
+        st.join = nm.e.join;
+        st.castable = nm.e.castable;
+        for (size_t k = 0; k != nm.e.inns.size(); ++k) {
+            int producer = -1;
+            for (link_t const& l : links) {
+                if (l.member == m && l.slot == int(k) &&
+                    std::find(members.begin(), members.end(), l.producer) != members.end()) {
+                    producer = l.producer;
+                }
+            }
+            if (producer >= 0) {
+                st.args.push_back(-1 - stage_of(producer));
+                continue;
+            }
+            mem_t const&     mem = nm.mems[k + 1];
+            dtype_t const    dt = nm.e.inn_dtype(int(k));
+            std::vector<int> modes = nm.e.inns[k];
+            if (!is_increasing(modes) || mem.offset % 16) return 0;
+            if (!modes.empty() && modes.back() > R - 1) return 0;
+            int found = -1;
+            for (size_t x = 0; x != ext_mems.size(); ++x) {
+                if (same_range(ext_mems[x], mem) && c.exts[x].dtype == dt && c.exts[x].modes == modes) {
+                    found = int(x);
+                }
+            }
+            if (found < 0) {
+                // the output may lie exactly on an input it is computed from, nowhere else
+                if (overlaps(P, mem) &&
+                    !(same_range(P, mem) && is_iota(modes, R) &&
+                      dtype_size(dt) == dtype_size(nv.e.out_dtype()))) {
+                    return 0;
+                }
+                found = int(ext_mems.size());
+                ext_mems.push_back(mem);
+                c.exts.push_back({dt, modes});
+            }
+            st.args.push_back(found);
+        }
+        c.stages.push_back(std::move(st));
+    }
+    if (c.exts.size() > 8) return 0;
+    // nobody between the first member and v may rewrite what the chain reads (it is read at
+    // v's place now)
+    for (int w = members.front() + 1; w < v; ++w) {
+        node_t const& nw = nodes_[size_t(w)];
+        if (nw.kind == kind_t::dummy || nw.kind == kind_t::evict) continue;
+        if (std::find(members.begin(), members.end(), w) != members.end()) continue;
+        for (mem_t const& m : ext_mems) {
+            if (overlaps(nw.mems[0], m)) return 0;
+        }
+    }
+    std::shared_ptr<plan_t> plan;
+    try {
+        if (km_) check(hipSetDevice(km_->device()), "hipSetDevice");
+        plan = plan_row_chain(c, km_ ? km_->device() : -1);
+    } catch (ir_error const&) {
+        return 0;
+    } catch (km_error const&) {
+        return 0;
+    }
+
+    // v stands for the whole chain; the others become dummies
+    std::vector<char> waits_for(size_t(n), 0);
+    std::vector<int>  deps;
+    for (int m : members) {
+        if (m != v) waits_for[size_t(m)] = 1;
+        deps.insert(deps.end(), nodes_[size_t(m)].deps.begin(), nodes_[size_t(m)].deps.end());
+    }
+    for (int w = members.front() + 1; w < n; ++w) {
+        node_t const& nw = nodes_[size_t(w)];
+        if (nw.kind != kind_t::dummy) continue;
+        for (int d : nw.deps) {
+            if (waits_for[size_t(d)]) {
+                waits_for[size_t(w)] = 1;
+                break;
+            }
+        }
+    }
+    deps.erase(std::remove_if(deps.begin(), deps.end(),
+                              [&](int d) {
+                                  return std::find(members.begin(), members.end(), d) != members.end();
+                              }),
+               deps.end());
+    std::sort(deps.begin(), deps.end());
+    deps.erase(std::unique(deps.begin(), deps.end()), deps.end());
+    // whoever waited for an absorbed node to be done with its inputs waits for v, which reads
+    // them now
+    for (int w = v + 1; w < n; ++w) {
+        std::vector<int>& d = nodes_[size_t(w)].deps;
+        bool const promised =
+            std::any_of(d.begin(), d.end(), [&](int x) { return waits_for[size_t(x)] != 0; });
+        if (promised && !std::binary_search(d.begin(), d.end(), v)) {
+            d.insert(std::upper_bound(d.begin(), d.end(), v), v);
+        }
+    }
+    for (int m : members) {
+        if (m == v) continue;
+        node_t& nm = nodes_[size_t(m)];
+        mem_t const S = nm.mems[0];
+        nm.kind = kind_t::dummy;
+        nm.mems = {S};
+        nm.is_del = false;
+    }
+    nv.kind = kind_t::chain;
+    nv.mems = {P};
+    nv.mems.insert(nv.mems.end(), ext_mems.begin(), ext_mems.end());
+    nv.deps = std::move(deps);
+    nv.chain_plan = std::move(plan);
+    nv.chain_stages = int(members.size());
+    return int(members.size()) - 1;
+}
+
 int apply_graph_t::optimize()
 {
     if (finalized_) throw km_error(km_status::invalid, "apply graph: already finalized");
     int absorbed = 0;
     for (int u = 0; u != int(nodes_.size()); ++u) {
         if (absorb_into_readers(u)) ++absorbed;
+    }
+    const char* env = std::getenv("ES_KM_ROW_CHAINS");
+    if (!(env && env[0] == '0')) {
+        for (int v = 0; v != int(nodes_.size()); ++v) absorbed += fuse_row_chain(v);
     }
     return absorbed;
 }
@@ -867,6 +1105,14 @@ void apply_graph_t::launch(node_t const& n, hipStream_t stream, char* arena) con
                                  hipMemcpyHostToDevice, stream),
                   "hipMemcpyAsync");
             break;
+        case kind_t::chain: {
+            if (!n.chain_plan) throw km_error(km_status::not_built, "apply graph: chain not built");
+            void const*  ptrs[8];
+            size_t const k = n.mems.size() - 1;
+            for (size_t i = 0; i != k; ++i) ptrs[i] = arena + n.mems[i + 1].offset;
+            km_->run_plan(*n.chain_plan, stream, out, ptrs, int(k), nullptr, 0);
+            break;
+        }
         case kind_t::dummy:
             break;
     }

@@ -98,6 +98,15 @@ public:
     // dependencies on either, stay valid.  Einsummables the kernel manager cannot build stay as they are.
     // Before finalize; returns the number of nodes absorbed.  The reference has no such pass
     // at this level: its graphs reach the engine with these nodes in them.
+    //
+    // And a chain over rows becomes one launch: row reductions (and pointwise steps on their
+    // per-row results) whose outputs only feed each other and one last elementwise node over
+    // the same rows -- softmax as row max, sum of exp(x - max), exp(x - max) / sum; a
+    // normalisation as sum of squares, power, scale -- with intermediate results that are
+    // deleted afterwards.  The last node then reads each row once, keeps it in registers
+    // through every stage and writes it once (codegen.h: cg_chain_t); its output has the bits
+    // the nodes give one after the other.  The absorbed nodes become dummies.  Counted in the
+    // return value; ES_KM_ROW_CHAINS=0 switches it off.
     int optimize();
 
     // Builds every einsummable on the kernel manager (throws km_error when one has no
@@ -133,7 +142,7 @@ public:
     // smallest arena that holds every range a node touches
     uint64_t arena_bytes() const;
     // 0 einsummable, 1 touch, 2 constant fill, 3 lowertri fill, 4 copy, 5 dummy, 6 evict,
-    // 7 load
+    // 7 load, 8 chain over rows (made by optimize)
     int                       kind_of(int id) const { return int(nodes_[id].kind); }
     std::vector<mem_t> const& mems_of(int id) const { return nodes_[id].mems; }
     // after finalize: launch position, stream and dependencies (own + implied) of a node
@@ -146,7 +155,7 @@ public:
     int n_launches() const;
 
 private:
-    enum class kind_t { einsummable, touch, constant, lowertri, copy, dummy, evict, load };
+    enum class kind_t { einsummable, touch, constant, lowertri, copy, dummy, evict, load, chain };
     struct node_t {
         kind_t             kind;
         einsummable_t      e;
@@ -170,10 +179,15 @@ private:
         // holds the ids of all of them.
         int                batch_head = -1;
         std::vector<int>   batch;
+        // chain over rows: its kernel (null without a kernel manager) and how many nodes it
+        // stands for; `e` is the last node's einsummable, mems the output and the chain's inputs
+        std::shared_ptr<plan_t> chain_plan;
+        int                     chain_stages = 0;
     };
 
     int  insert(node_t&& n, std::vector<int> const& deps);
     bool absorb_into_readers(int u);
+    int  fuse_row_chain(int v);
     void launch(node_t const& n, hipStream_t stream, char* arena) const;
 
     kernel_manager_t*        km_;

@@ -108,6 +108,11 @@ std::shared_ptr<plan_t> plan_complex_contraction(einsummable_t const& e, int dev
 std::shared_ptr<plan_t> plan_transpose(einsummable_t const& e, int device);
 // `defer`: generate the kernels' source only; finish_codegen_plans compiles and loads
 std::shared_ptr<plan_t> plan_codegen(einsummable_t const& e, int device, bool defer = false);
+// The kernel of a chain of nodes over rows (codegen.h: cg_chain_t), compiled and loaded on
+// `device` (a negative device: generated only, for inspection).  run() takes the last node's
+// output and the chain's inputs.  Throws ir_error when the chain has no such kernel.
+struct cg_chain_t;
+std::shared_ptr<plan_t> plan_row_chain(cg_chain_t const& c, int device);
 // Compiles the generated kernels of all these plans as ONE runtime-compiled program (the
 // compiler's fixed cost per program is most of the time of a small kernel, and it compiles
 // one program at a time whatever the number of calling threads: the 25 distinct generated

@@ -720,7 +720,7 @@ class ApplyGraph:
         return int(self._lib.es_km_graph_arena_bytes(self._g))
 
     NODE_KINDS = ("einsummable", "touch", "constant", "lowertri", "copy", "dummy", "evict",
-                  "load")
+                  "load", "chain")
 
     def node_mems(self, node):
         """(kind name, [(offset, size)]) of a node."""

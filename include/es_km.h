@@ -234,7 +234,12 @@ int es_km_graph_add_memory_dependencies(es_km_graph_t* g);
  * smaller than the traffic its output caused; a sum is only merged when its order of addition
  * stays what it was.  Both need the range's del node (memgraph.h: del_t) in the graph, as a
  * dummy that covers the range and depends on its last reader: without it the range counts as
- * a result and stays.  Node ids stay valid: an absorbed node becomes a dummy.  *n_absorbed
+ * a result and stays.  Last, a chain over rows -- row reductions, pointwise steps on their
+ * per-row results and the elementwise node that uses them, over the same rows, with every
+ * intermediate result deleted afterwards (softmax: row max, sum of exp(x - max), the
+ * quotient) -- becomes one launch that reads each row once and writes it once; the last
+ * node's output keeps its bits (ES_KM_ROW_CHAINS=0 in the environment leaves chains alone).
+ * Node ids stay valid: an absorbed node becomes a dummy.  *n_absorbed
  * (may be null) receives how many were absorbed.  No counterpart in the reference, whose
  * engine launches the nodes as the memgraph lists them. */
 int es_km_graph_optimize(es_km_graph_t* g, int* n_absorbed);
@@ -354,7 +359,8 @@ int es_km_graph_load_memgraph(es_km_graph_t* g, const void* bytes, uint64_t size
 
 /* Inspection: node count, the smallest arena holding every range, and a node's kind
  * (0 einsummable, 1 touch, 2 constant fill, 3 lowertri fill, 4 copy, 5 dummy, 6 evict,
- * 7 load) and ranges (for a dummy made of an inputmem: where the caller puts that input). */
+ * 7 load, 8 a chain over rows that es_km_graph_optimize made) and ranges (for a dummy made of
+ * an inputmem: where the caller puts that input). */
 int      es_km_graph_num_nodes(es_km_graph_t* g);
 uint64_t es_km_graph_arena_bytes(es_km_graph_t* g);
 int es_km_graph_node_mems(es_km_graph_t* g, int id, int* kind, uint64_t* offsets, uint64_t* sizes,

@@ -1,0 +1,214 @@
+"""Chains over rows (apply_graph_t::optimize, cg_chain_t): row reductions, pointwise steps on
+their per-row results and the elementwise node that uses them run as one launch that keeps a
+row in registers.  The chain computes every stage as its own kernel would, in the same order
+and with the same roundings, so the arena must hold, in every range that is still written,
+exactly the bytes of the node-by-node run; one case is also checked against the oracle."""
+import numpy as np
+import pytest
+
+import einsummable_amd as ea
+from helpers import NP, assert_close, normal, oracle_einsummable, rng, stream_handle
+
+pytestmark = pytest.mark.gpu
+
+E = ea.Einsummable
+DT = {"f16": ea.F16, "f32": ea.F32}
+
+
+@pytest.fixture(scope="module")
+def km():
+    return ea.KernelManager(0)
+
+
+def layout(sizes, misalign=0):
+    """Arena offsets (256-byte aligned, plus `misalign` bytes on every one) of buffers of
+    these byte sizes."""
+    offs, at = [], 0
+    for s in sizes:
+        offs.append(at + misalign)
+        at += (s + misalign + 255) // 256 * 256
+    return offs, at
+
+
+def run_both(km, build, arena_bytes, init, env=None):
+    """build(g) adds the nodes and returns the ranges to compare; runs the graph as listed
+    and optimised.  Returns (arena bytes plain, arena bytes optimised, graphs, absorbed)."""
+    import torch
+
+    arenas, graphs, absorbed = [], [], 0
+    for optimize in (False, True):
+        g = ea.ApplyGraph(km)
+        build(g)
+        g.add_memory_dependencies()
+        if optimize:
+            absorbed = g.optimize()
+        g.finalize(1)
+        arena = torch.from_numpy(init.copy()).cuda()
+        assert arena.numel() >= arena_bytes
+        g.run(stream_handle(), arena.data_ptr())
+        torch.cuda.synchronize()
+        arenas.append(arena.cpu().numpy())
+        graphs.append(g)
+    return arenas[0], arenas[1], graphs, absorbed
+
+
+def softmax_nodes(lead, n, xdt, with_mask):
+    """row max, sum of exp(x - max), exp(x - max) / sum over [lead..., n]; statistics in f32"""
+    R = len(lead) + 1
+    full, rows = list(range(R)), list(range(R - 1))
+    x = "hole|%s@0" % xdt
+    if with_mask:
+        inner = "+[hole|%s@0,hole|%s@1]" % (xdt, xdt)
+        k = 2
+        ins = [full, [R - 2, R - 1]]
+    else:
+        inner = x
+        k = 1
+        ins = [full]
+    up = inner if xdt == "f32" else "to_f32[%s]" % inner
+    shifted = "+[%s,*[constant{f32|-1},hole|f32@%d]]" % (up, k)
+    quotient = "*[exp[%s],power{-1}[hole|f32@%d]]" % (shifted, k + 1)
+    rmax = E(lead + [n], ins, R - 1, up, "^")
+    rsum = E(lead + [n], ins + [rows], R - 1, "exp[%s]" % shifted, "+")
+    norm = E(lead + [n], ins + [rows, rows], R,
+             quotient if xdt == "f32" else "to_f16[%s]" % quotient)
+    return rmax, rsum, norm
+
+
+@pytest.mark.parametrize("lead,n,xdt,with_mask,in_place", [
+    ([4, 64], 2048, "f16", True, False),     # teams of 64 lanes, four vectors each
+    ([3, 5], 1000, "f16", True, False),      # the last vectors of a row are missing
+    ([2, 8], 8192, "f16", False, True),      # teams of 256 lanes, the output on the input
+    ([1, 7], 4104, "f16", False, False),     # 513 vectors: 256 lanes, the third round nearly empty
+    ([6, 32], 2048, "f32", True, False),     # 32-byte vectors
+    ([2, 3], 24, "f16", True, False),        # three vectors in a row
+    ([5, 16], 777, "f32", False, True),      # odd row length: one element per vector
+])
+def test_softmax_chain_keeps_every_bit(km, lead, n, xdt, with_mask, in_place):
+    rmax, rsum, norm = softmax_nodes(lead, n, xdt, with_mask)
+    rows = int(np.prod(lead))
+    esz = 2 if xdt == "f16" else 4
+    sizes = [rows * n * esz, lead[-1] * n * esz, rows * 4, rows * 4, rows * n * esz]
+    (X, M, mx, l, P), total = layout(sizes)
+    if in_place:
+        P = X
+    ins = [(X, sizes[0])] + ([(M, sizes[1])] if with_mask else [])
+
+    def build(g):
+        a = g.add_einsummable(rmax, [(mx, sizes[2])] + ins)
+        b = g.add_einsummable(rsum, [(l, sizes[3])] + ins + [(mx, sizes[2])])
+        c = g.add_einsummable(norm, [(P, sizes[4])] + ins + [(mx, sizes[2]), (l, sizes[3])])
+        g.add_dummy((mx, sizes[2]), [b, c])
+        g.add_dummy((l, sizes[3]), [c])
+
+    r = rng(7 + n)
+    init = np.zeros(total, np.uint8)
+    x = normal(r, rows * n, NP[DT[xdt]], 2.0)
+    m = np.where(r.uniform(size=lead[-1] * n) < 0.3, -30.0, 0.0).astype(NP[DT[xdt]])
+    init[X:X + sizes[0]] = x.view(np.uint8)
+    init[M:M + sizes[1]] = m.view(np.uint8)
+    plain, fused, graphs, absorbed = run_both(km, build, total, init)
+    assert absorbed == 2 and graphs[1].launches() == 1
+    assert graphs[1].describe(2).startswith("chain ")
+    assert np.array_equal(plain[P:P + sizes[4]], fused[P:P + sizes[4]])
+    if not in_place:
+        assert np.array_equal(fused[X:X + sizes[0]], init[X:X + sizes[0]])
+    # the chain's result is a softmax: against the oracle's node-by-node evaluation
+    if n == 2048 and xdt == "f16":
+        xs = x.reshape(lead + [n])
+        inputs = [xs] + ([m.reshape(lead[-1], n)] if with_mask else [])
+        want_max = oracle_einsummable(rmax, inputs)
+        want_sum = oracle_einsummable(rsum, inputs + [want_max])
+        want = oracle_einsummable(norm, inputs + [want_max, want_sum])
+        got = fused[P:P + sizes[4]].view(NP[DT[xdt]]).reshape(-1)
+        assert_close(got, np.asarray(want).reshape(-1), DT[xdt], what="softmax chain")
+
+
+def test_normalisation_chain_with_a_pointwise_step(km):
+    """sum of squares -> (mean + eps)^-1/2 -> x * r * w: a reduction, a step on the per-row
+    value and the elementwise node, with a weight that has the row's mode only."""
+    T, D = 200, 4096
+    sq = E([T, D], [[0, 1]], 1, "power{2}[to_f32[hole|f16@0]]", "+")
+    rstd = E([T], [[0]], 1, "power{-0.5}[+[*[constant{f32|%r},hole|f32@0],constant{f32|1e-06}]]" % (1.0 / D))
+    scale = E([T, D], [[0, 1], [0], [1]], 2, "*[to_f16[*[to_f32[hole|f16@0],hole|f32@1]],hole|f16@2]")
+    sizes = [T * D * 2, D * 2, T * 4, T * 4, T * D * 2]
+    (X, W, ss, rs, Y), total = layout(sizes)
+
+    def build(g):
+        a = g.add_einsummable(sq, [(ss, sizes[2]), (X, sizes[0])])
+        b = g.add_einsummable(rstd, [(rs, sizes[3]), (ss, sizes[2])])
+        c = g.add_einsummable(scale, [(Y, sizes[4]), (X, sizes[0]), (rs, sizes[3]), (W, sizes[1])])
+        g.add_dummy((ss, sizes[2]), [b])
+        g.add_dummy((rs, sizes[3]), [c])
+
+    r = rng(21)
+    init = np.zeros(total, np.uint8)
+    init[X:X + sizes[0]] = normal(r, T * D, np.float16, 1.5).view(np.uint8)
+    init[W:W + sizes[1]] = normal(r, D, np.float16, 1.0).view(np.uint8)
+    plain, fused, graphs, absorbed = run_both(km, build, total, init)
+    assert absorbed == 2 and graphs[1].launches() == 1
+    assert np.array_equal(plain[Y:Y + sizes[4]], fused[Y:Y + sizes[4]])
+
+
+def test_a_statistic_that_is_a_result_stays(km):
+    """Without its del node the row maximum is a result of the graph: it keeps its node and
+    its place in memory, and the chain is what follows it."""
+    lead, n = [2, 16], 512
+    rmax, rsum, norm = softmax_nodes(lead, n, "f16", False)
+    rows = 32
+    sizes = [rows * n * 2, rows * 4, rows * 4, rows * n * 2]
+    (X, mx, l, P), total = layout(sizes)
+
+    def build(g):
+        a = g.add_einsummable(rmax, [(mx, sizes[1]), (X, sizes[0])])
+        b = g.add_einsummable(rsum, [(l, sizes[2]), (X, sizes[0]), (mx, sizes[1])])
+        c = g.add_einsummable(norm, [(P, sizes[3]), (X, sizes[0]), (mx, sizes[1]), (l, sizes[2])])
+        g.add_dummy((l, sizes[2]), [c])       # the maximum is kept, the sum is deleted
+
+    r = rng(5)
+    init = np.zeros(total, np.uint8)
+    init[X:X + sizes[0]] = normal(r, rows * n, np.float16, 2.0).view(np.uint8)
+    plain, fused, graphs, absorbed = run_both(km, build, total, init)
+    # the sum goes into the chain (a reduction that reads the stored maximum), the maximum stays
+    assert absorbed == 1 and graphs[1].launches() == 2
+    assert graphs[1].describe(0).startswith("einsummable ")
+    for lo, nb in ((mx, sizes[1]), (P, sizes[3])):
+        assert np.array_equal(plain[lo:lo + nb], fused[lo:lo + nb])
+
+
+def test_chain_on_buffers_that_are_not_16_byte_aligned_is_left_alone(km):
+    lead, n = [2, 16], 512
+    rmax, rsum, norm = softmax_nodes(lead, n, "f16", False)
+    rows = 32
+    sizes = [rows * n * 2, rows * 4, rows * 4, rows * n * 2]
+    (X, mx, l, P), total = layout(sizes, misalign=8)
+
+    def build(g):
+        a = g.add_einsummable(rmax, [(mx, sizes[1]), (X, sizes[0])])
+        b = g.add_einsummable(rsum, [(l, sizes[2]), (X, sizes[0]), (mx, sizes[1])])
+        c = g.add_einsummable(norm, [(P, sizes[3]), (X, sizes[0]), (mx, sizes[1]), (l, sizes[2])])
+        g.add_dummy((mx, sizes[1]), [b, c])
+        g.add_dummy((l, sizes[2]), [c])
+
+    r = rng(6)
+    init = np.zeros(total, np.uint8)
+    init[X:X + sizes[0]] = normal(r, rows * n, np.float16, 2.0).view(np.uint8)
+    plain, fused, graphs, absorbed = run_both(km, build, total, init)
+    assert absorbed == 0 and graphs[1].launches() == 3
+    assert np.array_equal(plain[P:P + sizes[3]], fused[P:P + sizes[3]])
+
+
+def test_chain_switched_off_by_the_environment(km, monkeypatch):
+    monkeypatch.setenv("ES_KM_ROW_CHAINS", "0")
+    lead, n = [2, 16], 512
+    rmax, rsum, norm = softmax_nodes(lead, n, "f16", False)
+    g = ea.ApplyGraph(km)
+    sizes = [32 * n * 2, 128, 128, 32 * n * 2]
+    (X, mx, l, P), total = layout(sizes)
+    a = g.add_einsummable(rmax, [(mx, sizes[1]), (X, sizes[0])])
+    b = g.add_einsummable(rsum, [(l, sizes[2]), (X, sizes[0]), (mx, sizes[1])])
+    c = g.add_einsummable(norm, [(P, sizes[3]), (X, sizes[0]), (mx, sizes[1]), (l, sizes[2])])
+    g.add_dummy((mx, sizes[1]), [b, c])
+    g.add_dummy((l, sizes[2]), [c])
+    g.add_memory_dependencies()
+    assert g.optimize() == 0

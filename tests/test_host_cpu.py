@@ -354,6 +354,59 @@ def test_exec_graph_optimize_brings_modes_to_their_common_pieces_or_declines():
     assert n == 0
 
 
+def test_exec_graph_optimize_makes_one_launch_of_a_chain_over_rows():
+    """Row max, sum of exp(x - max) and the quotient, statistics deleted afterwards: one chain
+    node at the last one's place, with the tensor and the mask as its inputs."""
+    import einsummable_amd as ea
+
+    E = ea.Einsummable
+    h, s = 4, 64
+    n = h * s * s
+    m = lambda slot, nbytes: (slot * 65536, nbytes)
+    inner = "to_f32[+[hole|f16@0,hole|f16@1]]"
+    shifted = "+[" + inner + ",*[constant{f32|-1},hole|f32@2]]"
+    rmax = E([h, s, s], [[0, 1, 2], [1, 2]], 2, inner, "^")
+    rsum = E([h, s, s], [[0, 1, 2], [1, 2], [0, 1]], 2, "exp[" + shifted + "]", "+")
+    norm = E([h, s, s], [[0, 1, 2], [1, 2], [0, 1], [0, 1]], 3,
+             "to_f16[*[exp[" + shifted + "],power{-1}[hole|f32@3]]]")
+    X, M, mx, l, P = m(0, 2 * n), m(1, 2 * s * s), m(2, 4 * h * s), m(3, 4 * h * s), m(4, 2 * n)
+
+    def graph(dels=True, spoiler=None):
+        g = ea.ApplyGraph(None)
+        a = g.add_einsummable(rmax, [mx, X, M])
+        b = g.add_einsummable(rsum, [l, X, M, mx])
+        if spoiler:
+            spoiler(g)
+        c = g.add_einsummable(norm, [P, X, M, mx, l])
+        if dels:
+            g.add_dummy(mx, [b, c])
+            g.add_dummy(l, [c])
+        g.add_memory_dependencies()
+        return g, (a, b, c)
+
+    g, (a, b, c) = graph()
+    assert g.optimize() == 2
+    assert g.describe(a).startswith("dummy") and g.describe(b).startswith("dummy")
+    assert g.describe(c).startswith("chain 262144:32768 0:32768 65536:8192 | 3 stages, the last [4,64,64]:")
+    g.finalize(1)
+    assert g.launches() == 1
+    assert g.node_mems(c)[0] == "chain"
+
+    # statistics that are results of the graph stay in memory, and so do their nodes
+    g, _ = graph(dels=False)
+    assert g.optimize() == 0
+    # a node between the chain's first and last that rewrites what the chain reads
+    g, _ = graph(spoiler=lambda g: g.add_constant_fill(ea.F16, 0, s * s, M))
+    assert g.optimize() == 0
+    # ... or reads a statistic: that one is needed in memory, its node stays and the chain
+    # begins behind it
+    peek = E([h * s], [[0]], 1, "exp[hole|f32@0]")
+    g, (a, b, c) = graph(spoiler=lambda g: g.add_einsummable(peek, [m(5, 4 * h * s), mx]))
+    assert g.optimize() == 1
+    assert g.describe(a).startswith("einsummable") and g.describe(b).startswith("dummy")
+    assert g.describe(c).startswith("chain 262144:32768 0:32768 65536:8192 131072:1024 | 2 stages")
+
+
 def test_exec_graph_optimize_leaves_what_it_cannot_prove():
     import einsummable_amd as ea
 
