@@ -1332,6 +1332,25 @@ cg_kernel_t gen_row_chain(cg_chain_t const& c, int max_vec)
               << e << "[b" << e << "]);\n";
         }
     }
+    // Streaming loads and stores.  A tensor of the 256 MiB memory-side cache's size or more
+    // is read past the caches (its lines would still be there when the result is stored, and
+    // their write-back would fall into the next node: gen_elementwise); the result is stored
+    // past them only if it is larger than that cache -- one that fits is what the next node
+    // reads (the LLaMA layer's 256 MiB of probabilities: the product behind the softmax 71
+    // against 98 us).  An input the rows share (a mask) always takes the caches.
+    // ES_KM_CHAIN_NT: 1 loads and stores, 2 loads only, 3 stores only, 4 none.
+    uint64_t const out_bytes = n_rows * n * dtype_size(od);
+    std::vector<bool> whole(static_cast<size_t>(NE), false);
+    for (int e = 0; e != NE; ++e) {
+        uint64_t ne = 1;
+        for (int m : c.exts[size_t(e)].modes) ne *= c.shape[size_t(m)];
+        whole[size_t(e)] = ne == n_rows * n;
+    }
+    bool const stream_in = out_bytes >= (256ull << 20);
+    bool const stream_out = out_bytes > (256ull << 20);
+    int const  nt_mode = env_int("ES_KM_CHAIN_NT", stream_out ? 1 : (stream_in ? 2 : 4));
+    int const  NT_LD = (nt_mode == 1 || nt_mode == 2) ? 1 : 0;
+    int const  NT_ST = (nt_mode == 1 || nt_mode == 3) ? 1 : 0;
     // every load of the row before anything is stored: the output may lie on an input
     s << "#pragma unroll\n    for (int i = 0; i != VPL; ++i) {\n";
     s << "        const idx_t vv = lane + (idx_t)i * TEAM;\n";
@@ -1339,8 +1358,9 @@ cg_kernel_t gen_row_chain(cg_chain_t const& c, int max_vec)
     for (int e = 0; e != NE; ++e) {
         if (!is_vec[size_t(e)]) continue;
         std::string const T = storage_type(c.exts[size_t(e)].dtype);
-        s << "            r" << e << "[i] = *reinterpret_cast<const vec_t<" << T << ", V>*>(a.in" << e
-          << " + (b" << e << " + vv * V));\n";
+        s << "            r" << e << "[i] = ldv<" << (whole[size_t(e)] ? NT_LD : 0)
+          << ">(reinterpret_cast<const vec_t<" << T << ", V>*>(a.in" << e << " + (b" << e
+          << " + vv * V)));\n";
     }
     s << "        }\n    }\n";
     auto call = [&](int t, std::string const& i, std::string const& j) {
@@ -1397,8 +1417,8 @@ cg_kernel_t gen_row_chain(cg_chain_t const& c, int max_vec)
     s << "            vec_t<" << storage_type(od) << ", V> o;\n";
     s << "#pragma unroll\n            for (int j = 0; j != V; ++j) o.v[j] = "
       << (od == dtype_t::f16 ? "(f16)(" : "(") << call(NS - 1, "i", "j") << ");\n";
-    s << "            *reinterpret_cast<vec_t<" << storage_type(od) << ", V>*>(a.out + (row * " << p_n
-      << " + vv * V)) = o;\n";
+    s << "            stv<" << NT_ST << ">(reinterpret_cast<vec_t<" << storage_type(od)
+      << ", V>*>(a.out + (row * " << p_n << " + vv * V)), o);\n";
     s << "        }\n    }\n}\n";
 
     k.source = s.str();
