@@ -1352,9 +1352,14 @@ cg_kernel_t gen_row_chain(cg_chain_t const& c, int max_vec)
     int const  NT_LD = (nt_mode == 1 || nt_mode == 2) ? 1 : 0;
     int const  NT_ST = (nt_mode == 1 || nt_mode == 3) ? 1 : 0;
     // every load of the row before anything is stored: the output may lie on an input
+    // Rows that fill every lane's vectors need no tests: the stages are then one straight
+    // piece of code, and what two of them compute alike (softmax: exp(x - max), for the sum
+    // and again for the quotient) the compiler computes once.
+    bool const        full_rows = nvec == uint64_t(TEAM) * uint64_t(VPL);
+    std::string const in_row = full_rows ? "true" : "vv < nvec";
     s << "#pragma unroll\n    for (int i = 0; i != VPL; ++i) {\n";
     s << "        const idx_t vv = lane + (idx_t)i * TEAM;\n";
-    s << "        if (vv < nvec) {\n";
+    s << "        if (" << in_row << ") {\n";
     for (int e = 0; e != NE; ++e) {
         if (!is_vec[size_t(e)]) continue;
         std::string const T = storage_type(c.exts[size_t(e)].dtype);
@@ -1396,7 +1401,8 @@ cg_kernel_t gen_row_chain(cg_chain_t const& c, int max_vec)
         s << "    " << ACC << " acc" << T << " = " << identity_of(st.castable.value(), result[size_t(t)])
           << ";\n";
         s << "#pragma unroll\n    for (int i = 0; i != VPL; ++i) {\n";
-        s << "        if (lane + (idx_t)i * TEAM < nvec) {\n";
+        s << "        const idx_t vv = lane + (idx_t)i * TEAM;\n";
+        s << "        if (" << in_row << ") {\n";
         s << "#pragma unroll\n            for (int j = 0; j != V; ++j) acc" << T << " = comb" << T << "(acc"
           << T << ", " << call(t, "i", "j") << ");\n";
         s << "        }\n    }\n";
@@ -1413,7 +1419,7 @@ cg_kernel_t gen_row_chain(cg_chain_t const& c, int max_vec)
     }
     s << "#pragma unroll\n    for (int i = 0; i != VPL; ++i) {\n";
     s << "        const idx_t vv = lane + (idx_t)i * TEAM;\n";
-    s << "        if (vv < nvec) {\n";
+    s << "        if (" << in_row << ") {\n";
     s << "            vec_t<" << storage_type(od) << ", V> o;\n";
     s << "#pragma unroll\n            for (int j = 0; j != V; ++j) o.v[j] = "
       << (od == dtype_t::f16 ? "(f16)(" : "(") << call(NS - 1, "i", "j") << ");\n";
