@@ -740,6 +740,15 @@ int apply_graph_t::fuse_row_chain(int v)
         c.stages.push_back(std::move(st));
     }
     if (c.exts.size() > 8) return 0;
+    // the intermediate results lie apart from everything the chain touches
+    for (int m : members) {
+        if (m == v) continue;
+        mem_t const& S = nodes_[size_t(m)].mems[0];
+        if (overlaps(S, P)) return 0;
+        for (mem_t const& x : ext_mems) {
+            if (overlaps(S, x)) return 0;
+        }
+    }
     // nobody between the first member and v may rewrite what the chain reads (it is read at
     // v's place now)
     for (int w = members.front() + 1; w < v; ++w) {

@@ -212,3 +212,92 @@ def test_chain_switched_off_by_the_environment(km, monkeypatch):
     g.add_dummy((l, sizes[2]), [c])
     g.add_memory_dependencies()
     assert g.optimize() == 0
+
+
+def chain_case(kind, lead, n, xdt):
+    """(nodes, buffers): nodes as (einsummable, out buffer, [input buffers]); buffers as
+    name -> (dtype, element count, is a statistic that is deleted)."""
+    R = len(lead) + 1
+    full, rows = list(range(R)), list(range(R - 1))
+    nrows = int(np.prod(lead))
+    x = "hole|%s@0" % xdt
+    up = x if xdt == "f32" else "to_f32[%s]" % x
+    down = (lambda t: t) if xdt == "f32" else (lambda t: "to_f16[%s]" % t)
+    bufs = {"X": (xdt, nrows * n, False), "Y": (xdt, nrows * n, False)}
+    nodes = []
+    if kind == "layernorm":
+        # mean, sum of squared deviations, (var + eps)^-1/2, (x - mean) * rstd * w + b
+        bufs.update(mean=("f32", nrows, True), dev=("f32", nrows, True), rstd=("f32", nrows, True),
+                    W=(xdt, n, False), B=(xdt, n, False))
+        centred = "+[%s,*[constant{f32|-1},hole|f32@1]]" % up
+        nodes.append((E(lead + [n], [full], R - 1, "*[constant{f32|%r},%s]" % (1.0 / n, up), "+"),
+                      "mean", ["X"]))
+        nodes.append((E(lead + [n], [full, rows], R - 1, "power{2}[%s]" % centred, "+"),
+                      "dev", ["X", "mean"]))
+        nodes.append((E(lead, [rows], R - 1,
+                        "power{-0.5}[+[*[constant{f32|%r},hole|f32@0],constant{f32|1e-05}]]" % (1.0 / n)),
+                      "rstd", ["dev"]))
+        w = "hole|%s@3" % xdt if xdt == "f32" else "to_f32[hole|%s@3]" % xdt
+        b = "hole|%s@4" % xdt if xdt == "f32" else "to_f32[hole|%s@4]" % xdt
+        nodes.append((E(lead + [n], [full, rows, rows, [R - 1], [R - 1]], R,
+                        down("+[*[*[%s,hole|f32@2],%s],%s]" % (centred, w, b))),
+                      "Y", ["X", "mean", "rstd", "W", "B"]))
+    elif kind == "minmax":
+        # (x - min) / (max - min + 1)
+        bufs.update(lo=("f32", nrows, True), hi=("f32", nrows, True))
+        nodes.append((E(lead + [n], [full], R - 1, up, "v"), "lo", ["X"]))
+        nodes.append((E(lead + [n], [full], R - 1, up, "^"), "hi", ["X"]))
+        span = "power{-1}[+[+[hole|f32@2,*[constant{f32|-1},hole|f32@1]],constant{f32|1}]]"
+        nodes.append((E(lead + [n], [full, rows, rows], R,
+                        down("*[+[%s,*[constant{f32|-1},hole|f32@1]],%s]" % (up, span))),
+                      "Y", ["X", "lo", "hi"]))
+    else:
+        # statistics in f16, as C4 has them: max, sum of exp(x - max), quotient
+        assert xdt == "f16"
+        bufs.update(m=("f16", nrows, True), l=("f16", nrows, True))
+        sub = "exp[+[hole|f16@0,*[constant{f16|-1},hole|f16@1]]]"
+        nodes.append((E(lead + [n], [full], R - 1, "hole|f16@0", "^"), "m", ["X"]))
+        nodes.append((E(lead + [n], [full, rows], R - 1, sub, "+"), "l", ["X", "m"]))
+        nodes.append((E(lead + [n], [full, rows, rows], R, "*[%s,power{-1}[hole|f16@2]]" % sub),
+                      "Y", ["X", "m", "l"]))
+    return nodes, bufs
+
+
+@pytest.mark.parametrize("kind,lead,n,xdt", [
+    ("layernorm", [7, 9], 768, "f16"),
+    ("layernorm", [33], 4096, "f32"),
+    ("layernorm", [2, 3, 4], 1000, "f16"),
+    ("minmax", [5, 5], 2048, "f16"),
+    ("minmax", [64], 333, "f32"),
+    ("f16stats", [8, 16], 2048, "f16"),
+    ("f16stats", [3], 16384, "f16"),         # eight vectors per lane
+])
+def test_other_chains_keep_every_bit(km, kind, lead, n, xdt):
+    nodes, bufs = chain_case(kind, lead, n, xdt)
+    names = list(bufs)
+    esz = {"f16": 2, "f32": 4}
+    sizes = [bufs[k][1] * esz[bufs[k][0]] for k in names]
+    offs, total = layout(sizes)
+    mem = {k: (o, s) for k, o, s in zip(names, offs, sizes)}
+
+    def build(g):
+        last_reader = {}
+        for e, out, ins in nodes:
+            i = g.add_einsummable(e, [mem[out]] + [mem[k] for k in ins])
+            for k in ins:
+                last_reader.setdefault(k, []).append(i)
+        for k in names:
+            if bufs[k][2]:
+                g.add_dummy(mem[k], last_reader[k])
+
+    r = rng(len(kind) * 100003 + n)
+    init = np.zeros(total, np.uint8)
+    for k in names:
+        if not bufs[k][2] and k != "Y":
+            lo, nb = mem[k]
+            init[lo:lo + nb] = normal(r, bufs[k][1], NP[DT[bufs[k][0]]], 1.5).view(np.uint8)
+    plain, fused, graphs, absorbed = run_both(km, build, total, init)
+    assert absorbed == len(nodes) - 1 and graphs[1].launches() == 1, (absorbed, graphs[1].launches())
+    lo, nb = mem["Y"]
+    assert np.array_equal(plain[lo:lo + nb], fused[lo:lo + nb])
+    assert np.isfinite(fused[lo:lo + nb].view(NP[DT[xdt]]).astype(np.float64)).all()
