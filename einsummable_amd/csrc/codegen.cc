@@ -224,6 +224,10 @@ __device__ __forceinline__ float  cvt_in(f16 v) { return (float)v; }
 __device__ __forceinline__ float  cvt_in(float v) { return v; }
 __device__ __forceinline__ double cvt_in(double v) { return v; }
 __device__ __forceinline__ c64    cvt_in(c64 v) { return v; }
+// a complex number kept as two f16
+struct h2 { f16 re, im; };
+__device__ __forceinline__ c64 cvt_in(h2 v) { return c64{(float)v.re, (float)v.im}; }
+__device__ __forceinline__ h2  narrow_c64(c64 v) { return h2{(f16)v.re, (f16)v.im}; }
 __device__ __forceinline__ float  lane_xor(float v, int m) { return __shfl_xor(v, m); }
 __device__ __forceinline__ double lane_xor(double v, int m) { return __shfl_xor(v, m); }
 __device__ __forceinline__ c64    lane_xor(c64 v, int m)
@@ -339,6 +343,18 @@ struct gen_t {
 
     std::string P(int i) const { return "a.p[" + std::to_string(i) + "]"; }
 
+    // how operand `op` (0 the output, 1 + k input k) lies in memory
+    std::string storage(int op) const
+    {
+        if (e.stored_as_half_pairs(op)) return "h2";
+        return storage_type(op == 0 ? e.out_dtype() : e.inn_dtype(op - 1));
+    }
+    int storage_size(int op) const
+    {
+        if (e.stored_as_half_pairs(op)) return 4;
+        return int(dtype_size(op == 0 ? e.out_dtype() : e.inn_dtype(op - 1)));
+    }
+
     void header()
     {
         src << PRELUDE;
@@ -356,9 +372,9 @@ struct gen_t {
     // `with_ws`: a pointer to partial results (in the accumulator type) follows the inputs
     void args_struct(bool with_ws = false)
     {
-        src << "struct args_t {\n    " << storage_type(e.out_dtype()) << "* out;\n";
+        src << "struct args_t {\n    " << storage(0) << "* out;\n";
         for (int i = 0; i != L.NI; ++i) {
-            src << "    const " << storage_type(e.inn_dtype(i)) << "* in" << i << ";\n";
+            src << "    const " << storage(1 + i) << "* in" << i << ";\n";
         }
         if (with_ws) src << "    " << compute_type(e.out_dtype()) << "* ws;\n";
         src << "    idx_t p[" << std::max(n_params, 1) << "];\n};\n";
@@ -366,6 +382,7 @@ struct gen_t {
 
     std::string store_cast(std::string const& v) const
     {
+        if (e.stored_as_half_pairs(0)) return "narrow_c64(" + v + ")";
         if (e.out_dtype() == dtype_t::f16) return "(f16)(" + v + ")";
         return v;
     }
@@ -392,9 +409,10 @@ std::string entry_name(einsummable_t const& e, const char* kind)
     }
     uint32_t h = 2166136261u;
     for (char c : e.join.str()) h = (h ^ uint8_t(c)) * 16777619u;
+    for (char c : e.half_complex) h = (h ^ uint8_t(c + 1)) * 16777619u;
     char buf[16];
     std::snprintf(buf, sizeof(buf), "_%08x", h);
-    return s + buf;
+    return s + buf + (e.any_half_pairs() ? "_h2" : "");
 }
 
 // Tuning aids: ES_KM_EW_UNROLL (vectors per thread of the elementwise kernels) and
@@ -467,10 +485,10 @@ cg_kernel_t gen_elementwise(einsummable_t const& e, int max_vec)
     // f16 -> f32 conversion ran at 3.1 TB/s that way and runs at 5.0 TB/s this way, the
     // reverse went from 4.4 to 5.0.
     // (An input without the innermost mode is one scalar per vector and has no say in this.)
-    int widest = int(dtype_size(e.out_dtype()));
+    int widest = g.storage_size(0);
     for (int k = 0; k != int(e.inns.size()); ++k) {
         if (acc[k] == access_t::bcast) continue;
-        widest = std::max(widest, int(dtype_size(e.inn_dtype(k))));
+        widest = std::max(widest, g.storage_size(1 + k));
     }
     int const vcap = std::min(max_vec, 16 / widest);
     int V;
@@ -515,10 +533,10 @@ cg_kernel_t gen_elementwise(einsummable_t const& e, int max_vec)
     // result there for the node that reads it next (C2: the row sum after exp(x - m) reads at
     // 6.0 instead of 5.4 TB/s, the producer is as fast either way); beyond that the cache
     // holds nothing useful at the end and plain stores only cost bandwidth.
-    uint64_t const out_bytes = n_out * dtype_size(e.out_dtype());
+    uint64_t const out_bytes = n_out * uint64_t(g.storage_size(0));
     uint64_t footprint = out_bytes;
     for (int k = 0; k != int(e.inns.size()); ++k) {
-        footprint += e.inn_nelem(k) * dtype_size(e.inn_dtype(k));
+        footprint += e.inn_nelem(k) * uint64_t(g.storage_size(1 + k));
     }
     bool const stream_out = out_bytes >= (64ull << 20) && footprint > (288ull << 20);
     // With a result beyond the cache's size such a node reads non-temporally too.  A line
@@ -567,7 +585,7 @@ cg_kernel_t gen_elementwise(einsummable_t const& e, int max_vec)
     s << "extern \"C\" __global__ __launch_bounds__(256) void " << g.k.entry << "(args_t a)\n{\n";
     s << "    const idx_t n_vec = " << g.P(p_nvec) << ";\n";
     for (int k = 0; k != L.NI; ++k) {
-        std::string T = storage_type(e.inn_dtype(k));
+        std::string T = g.storage(1 + k);
         if (acc[k] == access_t::bcast) {
             s << "    " << T << " s" << k << "[U];\n";
         } else {
@@ -613,7 +631,7 @@ cg_kernel_t gen_elementwise(einsummable_t const& e, int max_vec)
         if (R >= 2) s << "            const idx_t d0 = rem;\n";
     }
     for (int k = 0; k != L.NI; ++k) {
-        std::string T = storage_type(e.inn_dtype(k));
+        std::string T = g.storage(1 + k);
         if (acc[k] == access_t::straight) {
             s << "            r" << k << "[u] = ldv<" << NT_LD << ">(reinterpret_cast<const vec_t<" << T
               << ", V>*>(a.in" << k << " + vid[u] * V));\n";
@@ -641,7 +659,7 @@ cg_kernel_t gen_elementwise(einsummable_t const& e, int max_vec)
     }
     s << "        }\n    }\n";
     s << "#pragma unroll\n    for (int u = 0; u != U; ++u) {\n        if (live[u]) {\n";
-    s << "            vec_t<" << storage_type(e.out_dtype()) << ", V> res;\n";
+    s << "            vec_t<" << g.storage(0) << ", V> res;\n";
     s << "#pragma unroll\n            for (int j = 0; j != V; ++j) {\n";
     s << "                res.v[j] = " << g.store_cast([&] {
         std::string call = "join_fn(";
@@ -656,7 +674,7 @@ cg_kernel_t gen_elementwise(einsummable_t const& e, int max_vec)
         return call + ")";
     }()) << ";\n";
     s << "            }\n";
-    s << "            stv<" << NT_ST << ">(reinterpret_cast<vec_t<" << storage_type(e.out_dtype())
+    s << "            stv<" << NT_ST << ">(reinterpret_cast<vec_t<" << g.storage(0)
       << ", V>*>(a.out + vid[u] * V), res);\n";
     s << "        }\n    }\n";
     if (tail) {
@@ -676,10 +694,10 @@ cg_kernel_t gen_elementwise(einsummable_t const& e, int max_vec)
     uint64_t per_block = 256ull * uint64_t(U);
     g.k.grid = std::max<uint64_t>(1, (n_vec + per_block - 1) / per_block);
     g.k.block = 256;
-    g.k.out_inn_align.push_back(V * int(dtype_size(e.out_dtype())));
+    g.k.out_inn_align.push_back(V * g.storage_size(0));
     for (int k = 0; k != L.NI; ++k) {
         bool wide = acc[k] == access_t::straight || acc[k] == access_t::vec;
-        g.k.out_inn_align.push_back((wide ? V : 1) * int(dtype_size(e.inn_dtype(k))));
+        g.k.out_inn_align.push_back((wide ? V : 1) * g.storage_size(1 + k));
     }
     return std::move(g.k);
 }
@@ -1444,7 +1462,14 @@ cg_kernel_t generate_kernel(einsummable_t const& e, int max_vec)
     if (e.join_shape.size() > 12 || e.inns.size() > 8) {
         throw ir_error("generate_kernel: too many modes or inputs");
     }
+    for (int op = 0; op <= int(e.inns.size()); ++op) {
+        if (e.stored_as_half_pairs(op) &&
+            (op == 0 ? e.out_dtype() : e.inn_dtype(op - 1)) != dtype_t::c64) {
+            throw ir_error("generate_kernel: only complex tensors are kept as f16 pairs");
+        }
+    }
     if (!e.has_aggregation()) return gen_elementwise(e, max_vec);
+    if (e.any_half_pairs()) throw ir_error("generate_kernel: f16 pairs in a reduction");
     if (e.out_dtype() == dtype_t::c64 &&
         (e.castable.value() == castable_t::min || e.castable.value() == castable_t::max)) {
         throw ir_error("generate_kernel: min/max aggregation of complex values");

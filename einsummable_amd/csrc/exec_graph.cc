@@ -367,8 +367,74 @@ std::vector<int> expand(std::vector<int> const& inn, std::vector<std::vector<int
 // do not line up.  v reads input k position by position over its join modes; u has no
 // aggregation.  The two may cut the same elements into modes differently ([32, 4194304]
 // against [65536, 2048]): both are rewritten over the common pieces first.
+// exactly to_<to>[hole|<from>@0] over one straight input
+bool is_plain_conversion(einsummable_t const& e, dtype_t from, dtype_t to)
+{
+    node_t const& r = e.join.root;
+    return !e.has_aggregation() && e.inns.size() == 1 && is_iota(e.inns[0], int(e.join_shape.size())) &&
+           !e.any_half_pairs() && r.kind == op_kind::convert && r.dtype == to && r.children.size() == 1 &&
+           r.children[0].kind == op_kind::hole && r.children[0].arg == 0 && r.children[0].dtype == from;
+}
+
+// Conversions around a complex view.  A complex node that reads, as c64, the f32 tensor a
+// conversion from f16 has just written takes the f16 tensor itself, pairs of f16 widened on
+// the load (u the conversion, v the complex node); a conversion to f16 that reads, as f32,
+// what a complex node wrote becomes that node with its result rounded to pairs of f16 on
+// the store (u the complex node, v the conversion).  Rotary embeddings are spelled that
+// way: to_f32, the product with the frequencies on the buffer seen as complex, to_f16.
+std::optional<einsummable_t> merged_across_a_complex_view(einsummable_t const& u,
+                                                         einsummable_t const& v, int k)
+{
+    int const rank_v = int(v.join_shape.size());
+    if (u.out_dtype() == dtype_t::f32 && v.inn_dtype(k) == dtype_t::c64) {
+        if (!is_plain_conversion(u, dtype_t::f16, dtype_t::f32) || v.has_aggregation() ||
+            u.out_nelem() != 2 * v.inn_nelem(k) || !is_iota(v.inns[size_t(k)], rank_v) ||
+            v.stored_as_half_pairs(1 + k)) {
+            return std::nullopt;
+        }
+        scalarop_t identity;
+        identity.root.kind = op_kind::hole;
+        identity.root.dtype = dtype_t::c64;
+        identity.root.arg = 0;
+        identity.hole_dtypes = {dtype_t::c64};
+        std::vector<std::vector<int>> inns{v.inns[size_t(k)]};
+        std::vector<char>             half(v.inns.size() + 1, 0);
+        half[0] = v.stored_as_half_pairs(0);
+        half[1] = 1;
+        for (int i = 0, at = 2; i != int(v.inns.size()); ++i) {
+            if (i == k) continue;
+            inns.push_back(v.inns[size_t(i)]);
+            half[size_t(at++)] = v.stored_as_half_pairs(1 + i);
+        }
+        try {
+            einsummable_t r = einsummable_t::make(v.join_shape, inns, v.out_rank,
+                                                  scalarop_t::compose(v.join, k, identity), v.castable);
+            r.half_complex = half;
+            return r;
+        } catch (ir_error const&) {
+            return std::nullopt;
+        }
+    }
+    if (u.out_dtype() == dtype_t::c64 && v.inn_dtype(k) == dtype_t::f32) {
+        if (!is_plain_conversion(v, dtype_t::f32, dtype_t::f16) || u.has_aggregation() ||
+            v.out_nelem() != 2 * u.out_nelem() || u.stored_as_half_pairs(0)) {
+            return std::nullopt;
+        }
+        einsummable_t r = u;
+        r.half_complex.resize(u.inns.size() + 1, 0);
+        r.half_complex[0] = 1;
+        return r;
+    }
+    return std::nullopt;
+}
+
 std::optional<einsummable_t> merged(einsummable_t const& u, einsummable_t const& v, int k)
 {
+    if ((u.out_dtype() == dtype_t::f32 && v.inn_dtype(k) == dtype_t::c64) ||
+        (u.out_dtype() == dtype_t::c64 && v.inn_dtype(k) == dtype_t::f32)) {
+        return merged_across_a_complex_view(u, v, k);
+    }
+    if (u.any_half_pairs() || v.any_half_pairs()) return std::nullopt;
     if (u.out_dtype() != v.inn_dtype(k) || u.out_nelem() != v.inn_nelem(k)) return std::nullopt;
     if (u.inns.size() + v.inns.size() - 1 > 6) return std::nullopt;
     std::vector<uint64_t>         shape;
@@ -588,7 +654,10 @@ int apply_graph_t::fuse_row_chain(int v)
 {
     int const n = int(nodes_.size());
     node_t&   nv = nodes_[size_t(v)];
-    if (nv.kind != kind_t::einsummable || nv.e.has_aggregation() || nv.e.join.has_variables()) return 0;
+    if (nv.kind != kind_t::einsummable || nv.e.has_aggregation() || nv.e.join.has_variables() ||
+        nv.e.any_half_pairs()) {
+        return 0;
+    }
     int const R = int(nv.e.join_shape.size());
     if (R < 2) return 0;
     int const O = R - 1;
@@ -610,7 +679,7 @@ int apply_graph_t::fuse_row_chain(int v)
         return -1;
     };
     auto stage_kind = [&](einsummable_t const& e) {  // 1 reduction over the row, 2 pointwise on rows
-        if (e.join.has_variables()) return 0;
+        if (e.join.has_variables() || e.any_half_pairs()) return 0;
         if (e.has_aggregation()) return e.join_shape == shape && e.out_rank == O ? 1 : 0;
         return e.join_shape == rows ? 2 : 0;
     };

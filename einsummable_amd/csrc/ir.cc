@@ -893,7 +893,9 @@ einsummable_t einsummable_t::merge_adjacent_dims() const
     std::vector<std::vector<int>> new_inns;
     for (auto const& inn : inns) new_inns.push_back(squash(inn));
     int new_out_rank = int(squash(terms.back()).size());
-    return make(shape, new_inns, new_out_rank, join, castable);
+    einsummable_t r = make(shape, new_inns, new_out_rank, join, castable);
+    r.half_complex = half_complex;
+    return r;
 }
 
 std::string einsummable_t::str() const
@@ -923,6 +925,12 @@ std::string einsummable_t::key() const
         for (int m : inns[k]) s += std::to_string(m) + ".";
     }
     s += "->" + std::to_string(out_rank) + " | " + join.str();
+    if (any_half_pairs()) {
+        s += " | f16 pairs:";
+        for (size_t i = 0; i != half_complex.size(); ++i) {
+            if (half_complex[i]) s += i ? " in" + std::to_string(i - 1) : " out";
+        }
+    }
     return s;
 }
 

@@ -120,6 +120,24 @@ struct einsummable_t {
     int                           out_rank = 0;
     scalarop_t                    join;
     std::optional<castable_t>     castable;
+    // Not part of the reference's einsummable: [0] the output, [1 + k] input k -- a c64 tensor
+    // that lies in memory as pairs of f16 (real, imaginary) and is widened on the load or
+    // rounded on the store.  Empty: none.  Set by the exec graph's optimisation pass where a
+    // conversion node stood between an f16 tensor and its view as complex numbers (rotary
+    // embeddings: to_f32, the c64 product on the reinterpreted buffer, to_f16); only the
+    // generated elementwise kernels take such an einsummable.
+    std::vector<char>             half_complex;
+    bool stored_as_half_pairs(int operand) const
+    {
+        return size_t(operand) < half_complex.size() && half_complex[size_t(operand)] != 0;
+    }
+    bool any_half_pairs() const
+    {
+        for (char c : half_complex) {
+            if (c) return true;
+        }
+        return false;
+    }
 
     // Runs the checks and the aggregation-mode renumbering of the reference constructor
     // (einsummable.cc:32-93).  Throws ir_error when invalid.

@@ -151,7 +151,10 @@ std::optional<uint64_t> kernel_manager_t::build(einsummable_t const& e_)
 
 std::shared_ptr<plan_t> kernel_manager_t::make_plan(einsummable_t const& e, bool defer) const
 {
-    std::shared_ptr<plan_t> p = plan_contraction(e, device_);
+    // (complex tensors kept as f16 pairs: the generated elementwise kernels only)
+    std::shared_ptr<plan_t> p = e.any_half_pairs() ? plan_codegen(e, device_, defer)
+                                                   : plan_contraction(e, device_);
+    if (!p && e.any_half_pairs()) return nullptr;
     if (!p) p = plan_complex_contraction(e, device_);
     if (!p) p = plan_transpose(e, device_);
     if (!p) p = plan_staged_elementwise(e, device_, defer);

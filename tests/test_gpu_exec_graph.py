@@ -335,8 +335,10 @@ def test_optimized_layer_keeps_every_stored_bit(km, shape, n_streams):
     # (taken in by the row sum and by the division), the division; silu; the first residual
     # (taken in by the second norm and by the second residual).  Then three chains over
     # rows: each norm's sum of squares and its (mean + eps)^-1/2 go into x * rstd * w, the
-    # softmax's row max and row sum into the quotient.
-    assert fused.absorbed == 13 + 17 + 6, fused.absorbed
+    # softmax's row max and row sum into the quotient.  And the conversions around the two
+    # rotary products (to_f32 in front, to_f16 behind) go into the products, which read and
+    # write pairs of f16.
+    assert fused.absorbed == 13 + 17 + 6 + 4, fused.absorbed
     assert fused.graph.launches() == plain.graph.launches() - fused.absorbed
     for k, v in vals.items():
         plain.set_input(k, v)

@@ -156,7 +156,7 @@ def test_llama_layer_from_wire_optimized_keeps_the_result(km):
         off += (nbytes + 255) // 256 * 256
     g = ea.ApplyGraph(km)
     g.load_memgraph(mp.to_wire(layer_memgraph(lg, ranges, with_dels=True)))
-    assert g.optimize() == 36          # as when the runner adds the del nodes itself
+    assert g.optimize() == 40          # as when the runner adds the del nodes itself
     g.finalize(2)
     arena = torch.zeros(g.arena_bytes(), dtype=torch.uint8, device="cuda")
     for k, v in vals.items():

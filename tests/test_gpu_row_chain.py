@@ -301,3 +301,37 @@ def test_other_chains_keep_every_bit(km, kind, lead, n, xdt):
     lo, nb = mem["Y"]
     assert np.array_equal(plain[lo:lo + nb], fused[lo:lo + nb])
     assert np.isfinite(fused[lo:lo + nb].view(NP[DT[xdt]]).astype(np.float64)).all()
+
+
+@pytest.mark.parametrize("seq,heads,half", [(2048, 32, 64), (77, 5, 24), (3, 1, 1)])
+def test_conversions_around_a_complex_view_are_absorbed(km, seq, heads, half):
+    """Rotary embeddings as the reference's graph spells them: to_f32, the product with the
+    frequencies on the buffer seen as complex numbers, to_f16.  Optimised, the complex node
+    reads and writes pairs of f16 itself: one launch, the same bits."""
+    n = seq * heads * half * 2                       # f16 elements
+    up = E([n], [[0]], 1, "to_f32[hole|f16@0]")
+    rot = E([1, seq, heads, half], [[0, 1, 2, 3], [1, 3]], 4, "*[hole|c64@0,hole|c64@1]")
+    down = E([n], [[0]], 1, "to_f16[hole|f32@0]")
+    sizes = [n * 2, seq * half * 8, n * 4, n * 4, n * 2]
+    (X, F, A, B, Y), total = layout(sizes)
+
+    def build(g):
+        a = g.add_einsummable(up, [(A, sizes[2]), (X, sizes[0])])
+        b = g.add_einsummable(rot, [(B, sizes[3]), (A, sizes[2]), (F, sizes[1])])
+        c = g.add_einsummable(down, [(Y, sizes[4]), (B, sizes[3])])
+        g.add_dummy((A, sizes[2]), [b])
+        g.add_dummy((B, sizes[3]), [c])
+
+    r = rng(seq)
+    init = np.zeros(total, np.uint8)
+    init[X:X + sizes[0]] = normal(r, n, np.float16, 1.0).view(np.uint8)
+    ang = r.uniform(0, 6.28, seq * half)
+    init[F:F + sizes[1]] = (np.cos(ang) + 1j * np.sin(ang)).astype(np.complex64).view(np.uint8)
+    plain, fused, graphs, absorbed = run_both(km, build, total, init)
+    assert absorbed == 2 and graphs[1].launches() == 1
+    assert "f16 pairs: out in0" in graphs[1].describe(2)
+    assert np.array_equal(plain[Y:Y + sizes[4]], fused[Y:Y + sizes[4]])
+    got = fused[Y:Y + sizes[4]].view(np.float16).astype(np.float32).reshape(seq, heads, half, 2)
+    x = init[X:X + sizes[0]].view(np.float16).astype(np.float32).reshape(seq, heads, half, 2)
+    want = (x[..., 0] + 1j * x[..., 1]) * (np.cos(ang) + 1j * np.sin(ang)).reshape(seq, 1, half)
+    assert np.allclose(got[..., 0], want.real, atol=4e-3) and np.allclose(got[..., 1], want.imag, atol=4e-3)
