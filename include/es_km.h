@@ -239,6 +239,9 @@ int es_km_graph_add_memory_dependencies(es_km_graph_t* g);
  * intermediate result deleted afterwards (softmax: row max, sum of exp(x - max), the
  * quotient) -- becomes one launch that reads each row once and writes it once; the last
  * node's output keeps its bits (ES_KM_ROW_CHAINS=0 in the environment leaves chains alone).
+ * A conversion to f32 whose output a complex node reads as c64, and a conversion to f16 of
+ * what a complex node wrote (rotary embeddings: to_f32, product on the buffer seen as c64,
+ * to_f16), go into the complex node, which then reads and writes pairs of f16.
  * Node ids stay valid: an absorbed node becomes a dummy.  *n_absorbed
  * (may be null) receives how many were absorbed.  No counterpart in the reference, whose
  * engine launches the nodes as the memgraph lists them. */
