@@ -407,6 +407,50 @@ def test_exec_graph_optimize_makes_one_launch_of_a_chain_over_rows():
     assert g.describe(c).startswith("chain 262144:32768 0:32768 65536:8192 131072:1024 | 2 stages")
 
 
+def test_exec_graph_optimize_absorbs_conversions_around_a_complex_view():
+    """to_f32, a complex product on the buffer seen as c64, to_f16: the product takes the f16
+    tensor in and writes the f16 tensor out."""
+    import einsummable_amd as ea
+
+    E = ea.Einsummable
+    seq, heads, half = 16, 2, 8
+    n = seq * heads * half * 2
+    m = lambda slot, nbytes: (slot * 8192, nbytes)
+    up = E([n], [[0]], 1, "to_f32[hole|f16@0]")
+    rot = E([1, seq, heads, half], [[0, 1, 2, 3], [1, 3]], 4, "*[hole|c64@0,hole|c64@1]")
+    down = E([n], [[0]], 1, "to_f16[hole|f32@0]")
+    X, F, A, B, Y = m(0, 2 * n), m(1, 8 * seq * half), m(2, 4 * n), m(3, 4 * n), m(4, 2 * n)
+
+    def graph(del_a=True, del_b=True, first=up):
+        g = ea.ApplyGraph(None)
+        a = g.add_einsummable(first, [A, X] if first is up else [A, (X[0], 4 * n)])
+        b = g.add_einsummable(rot, [B, A, F])
+        c = g.add_einsummable(down, [Y, B])
+        if del_a:
+            g.add_dummy(A, [b])
+        if del_b:
+            g.add_dummy(B, [c])
+        g.add_memory_dependencies()
+        return g, (a, b, c)
+
+    g, (a, b, c) = graph()
+    assert g.optimize() == 2
+    assert g.describe(a).startswith("dummy") and g.describe(b).startswith("dummy")
+    assert g.describe(c) == ("einsummable 32768:1024 0:1024 8192:1024 | [1,16,2,8]: 0.1.2.3.,1.3.->4 | "
+                             "*[to_c64[hole|c64@0],hole|c64@1] | f16 pairs: out in0")
+    g.finalize(1)
+    assert g.launches() == 1
+    # one side only
+    g, (a, b, c) = graph(del_b=False)
+    assert g.optimize() == 1 and g.describe(b).endswith("| f16 pairs: in0")
+    g, (a, b, c) = graph(del_a=False)
+    assert g.optimize() == 1 and g.describe(c).endswith("| f16 pairs: out")
+    # a producer that is more than the conversion keeps its node
+    scaled = E([n], [[0]], 1, "*[constant{f32|2},hole|f32@0]")
+    g, (a, b, c) = graph(first=scaled, del_b=False)
+    assert g.optimize() == 0
+
+
 def test_exec_graph_optimize_leaves_what_it_cannot_prove():
     import einsummable_amd as ea
 
