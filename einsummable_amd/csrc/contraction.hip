@@ -188,6 +188,63 @@ struct contraction_plan_t : plan_t {
         }
     }
 
+    // Products of this shape on other buffers ride along as batch entries of one launch of
+    // the persistent 128 x 256 kernel when one of them has at most a tile per compute unit (a
+    // LLaMA projection of 2048 tokens): set-up, first loads and the last epilogue are then
+    // paid once instead of once per product.  What that buys is small -- the q, k and v
+    // projections 176 us as one launch against 188 as three: under the board's power limit
+    // the time saved is partly given back as clock -- and with several rounds of tiles per
+    // product it buys nothing (w1 and w3: 362 against 358 us), so those stay as they are.
+    int max_group() const override
+    {
+        const char* env = std::getenv("ES_KM_GEMM_GROUPS");  // tuning and tests
+        bool const  off = env && env[0] == '0';
+        bool const fits = dtype == dtype_t::f16 && args.persistent == 2 && args.batch == 1 &&
+                          args.splits <= 1 && workspace_bytes == 0 &&
+                          uint64_t(args.tiles_m) * args.tiles_n <= args.workgroups;
+        return fits && !off ? 8 : 1;
+    }
+
+    void run_group(hipStream_t stream, int runs, void* const* outs,
+                   void const* const* inns) const override
+    {
+        if (runs < 1 || runs > max_group()) {
+            throw km_error(km_status::invalid, "contraction: too many runs for one launch");
+        }
+        gemm_args_t a = args;
+        a.ws = nullptr;
+        a.A = swapped ? inns[1] : inns[0];
+        a.B = swapped ? inns[0] : inns[1];
+        a.C = outs[0];
+        auto mis = [](void const* p) { return reinterpret_cast<uintptr_t>(p) % 16 != 0; };
+        bool aligned = true;
+        for (int g = 0; g != runs; ++g) {
+            void const* const x = swapped ? inns[2 * g + 1] : inns[2 * g];
+            void const* const y = swapped ? inns[2 * g] : inns[2 * g + 1];
+            aligned = aligned && !mis(x) && !mis(y) && !mis(outs[g]);
+            a.group_off[0][g] = (static_cast<char const*>(x) - static_cast<char const*>(a.A)) / 2;
+            a.group_off[1][g] = (static_cast<char const*>(y) - static_cast<char const*>(a.B)) / 2;
+            a.group_off[2][g] = (static_cast<char const*>(outs[g]) - static_cast<char const*>(a.C)) / 2;
+        }
+        if (runs == 1 || !aligned || !gemm::pc::gemm_pc_eligible(a)) {
+            // what one launch cannot take runs one by one
+            for (int g = 0; g != runs; ++g) run(stream, outs[g], inns + 2 * g, nullptr, 0);
+            return;
+        }
+        a.grouped = 1;
+        a.batch = uint32_t(runs);
+        a.gb.n = 1;
+        a.gb.size[0] = uint32_t(runs);
+        a.gb.sx[0] = a.gb.sy[0] = a.gb.sz[0] = 0;
+        a.xcd_total = uint32_t(uint64_t(a.tiles_m) * a.tiles_n * uint64_t(runs));
+        launch(a, stream);
+        hipError_t err = hipGetLastError();
+        if (err != hipSuccess) {
+            throw km_error(km_status::device,
+                           std::string("contraction launch: ") + hipGetErrorString(err));
+        }
+    }
+
     void launch(gemm_args_t const& a, hipStream_t stream) const
     {
         switch (dtype) {

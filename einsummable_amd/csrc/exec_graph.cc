@@ -1037,6 +1037,38 @@ void apply_graph_t::finalize(int n_streams)
         v = end;
     }
 
+    // Runs of sibling products.  Einsummables of one key that follow each other in launch
+    // order (dummies aside) on one stream, none depending on another -- the q, k and v
+    // projections of one input, w1 and w3 -- go out as one launch when their kernel takes
+    // several runs at once (plan_t::max_group): at the first one's place, like the touches.
+    for (int v = 0; km_ && v < n; ++v) {
+        node_t& head = nodes_[v];
+        if (head.kind != kind_t::einsummable || head.batch_head >= 0) continue;
+        plan_t const* const plan = km_->plan_of(head.e);
+        int const           cap = plan ? plan->max_group() : 1;
+        if (cap < 2) continue;
+        std::string const key = head.e.merge_adjacent_dims().key();
+        std::vector<int>  members{v};
+        for (int w = v + 1; w < n && int(members.size()) < cap; ++w) {
+            node_t const& x = nodes_[w];
+            if (x.kind == kind_t::dummy) continue;
+            if (x.kind != kind_t::einsummable || x.batch_head >= 0 || x.stream != head.stream ||
+                x.e.merge_adjacent_dims().key() != key) {
+                break;
+            }
+            // independent of the members before it: what it waits for lies before the head
+            bool early = true;
+            for (int d : real_deps[size_t(w)]) early = early && d < v;
+            if (!early) break;
+            members.push_back(w);
+        }
+        if (members.size() < 2) continue;
+        for (int m : members) {
+            nodes_[m].batch_head = v;
+            head.batch.push_back(m);
+        }
+    }
+
     if (km_) {
         check(hipSetDevice(km_->device()), "hipSetDevice");
         streams_.assign(size_t(n_streams), nullptr);  // slot 0 is the caller's stream
@@ -1229,16 +1261,28 @@ void apply_graph_t::run(hipStream_t main, void* arena_) const
             if (n.batch_head != v) continue;  // launched with its head
             std::vector<touch_t>     touches;
             std::vector<void const*> inns;
+            std::vector<void*>       outs;
             for (int m : n.batch) {
                 node_t const& nm = nodes_[size_t(m)];
                 for (int d : nm.waits) {
                     check(hipStreamWaitEvent(st, events_[size_t(event_of_[size_t(d)])], 0),
                           "hipStreamWaitEvent");
                 }
-                touches.push_back(nm.touch);
-                inns.push_back(arena + nm.mems[1].offset);
+                if (n.kind == kind_t::einsummable) {
+                    outs.push_back(arena + nm.mems[0].offset);
+                    for (size_t i = 1; i != nm.mems.size(); ++i) inns.push_back(arena + nm.mems[i].offset);
+                } else {
+                    touches.push_back(nm.touch);
+                    inns.push_back(arena + nm.mems[1].offset);
+                }
             }
-            km_->touch_batch(touches, st, arena + n.mems[0].offset, inns);
+            if (n.kind == kind_t::einsummable) {
+                plan_t const* const plan = km_->plan_of(n.e);
+                if (!plan) throw km_error(km_status::not_built, "apply graph: einsummable not built");
+                plan->run_group(st, int(outs.size()), outs.data(), inns.data());
+            } else {
+                km_->touch_batch(touches, st, arena + n.mems[0].offset, inns);
+            }
             for (int m : n.batch) {
                 if (nodes_[size_t(m)].record) {
                     check(hipEventRecord(events_[size_t(event_of_[size_t(m)])], st),

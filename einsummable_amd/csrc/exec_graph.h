@@ -176,7 +176,9 @@ private:
         // Touches of one group that follow each other in launch order and write the same
         // output run as one launch (kernel_manager_t::touch_batch), at the first one's
         // place: `batch_head` is that node's id (-1: launched on its own), and the head
-        // holds the ids of all of them.
+        // holds the ids of all of them.  Likewise independent einsummables of one key that
+        // follow each other, when their kernel takes several runs at once
+        // (plan_t::run_group: the q, k and v projections of a layer).
         int                batch_head = -1;
         std::vector<int>   batch;
         // chain over rows: its kernel (null without a kernel manager) and how many nodes it

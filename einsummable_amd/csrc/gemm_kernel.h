@@ -73,6 +73,11 @@ struct gemm_args_t {
     // every sum is multiplied by this before it is rounded to the output type (1 for a plain
     // product); split-K partial tiles stay unscaled, the fold applies it
     double      alpha;
+    // Several products of one plan in one launch (gemm_pc_kernel): batch entry g reads and
+    // writes at these element offsets from A, B and C instead of the batch strides -- the
+    // same operand for all (offset 0 throughout) or buffers that lie anywhere
+    uint32_t    grouped;
+    int64_t     group_off[3][8];  // [A, B, C][entry]
 };
 
 __device__ __forceinline__ void group_offsets(group_t const& g, uint32_t i, int64_t& ox,

@@ -20,6 +20,8 @@
 #pragma once
 #include "gemm_w4_kernel.h"
 
+#include <cstddef>
+
 namespace es
 {
 namespace gemm
@@ -27,6 +29,17 @@ namespace gemm
 namespace pc
 {
 using namespace w4;
+
+// The offsets of a grouped launch, read through the kernel-argument pointer (the arguments
+// are the kernel's first parameter): a run-time index into the by-value struct would have the
+// compiler copy the whole block into private memory first.
+__device__ __forceinline__ int64_t const __attribute__((address_space(4))) * group_table()
+{
+    typedef char const __attribute__((address_space(4))) const_byte_t;
+    typedef int64_t const __attribute__((address_space(4))) const_off_t;
+    return (const_off_t*)((const_byte_t*)__builtin_amdgcn_kernarg_segment_ptr() +
+                          offsetof(gemm_args_t, group_off));
+}
 
 // Fragment read i of R goes behind matrix instruction i (N - 1) / R of a k-step's N: the index of
 // the read behind instruction q, or -1
@@ -262,7 +275,12 @@ __global__ __launch_bounds__(512) void gemm_pc_kernel(gemm_args_t a, uint32_t to
     auto seek_tile = [&](uint32_t L) ES_INLINE {
         tile_t const t = locate(L);
         int64_t      boa, bob;
-        group_offsets(a.gb, t.bz, boa, bob);
+        if (a.grouped) {
+            boa = group_table()[t.bz];
+            bob = group_table()[8 + t.bz];
+        } else {
+            group_offsets(a.gb, t.bz, boa, bob);
+        }
         A_tile = uniform(static_cast<T const*>(a.A) + boa);
         B_tile = uniform(static_cast<T const*>(a.B) + bob);
         uint32_t const lane_a = load_chunk * VL * uint32_t(a.gk.sx[0]) * uint32_t(sizeof(T));
@@ -367,7 +385,9 @@ __global__ __launch_bounds__(512) void gemm_pc_kernel(gemm_args_t a, uint32_t to
         st_c = st_c + 1 == NS ? 0 : st_c + 1;
         tile_t const   t = locate(blockIdx.x + it * G);
         int64_t        boc;
-        if (a.gb.n == 1) {
+        if (a.grouped) {
+            boc = group_table()[16 + t.bz];
+        } else if (a.gb.n == 1) {
             boc = int64_t(t.bz) * a.gb.sz[0];
         } else {
             boc = 0;

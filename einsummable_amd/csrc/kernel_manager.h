@@ -40,6 +40,15 @@ struct plan_t {
     uint64_t    workspace_bytes = 0;
     int         n_inns = 0;
     std::string description;
+    // How many runs of this plan on different buffers one launch can take (1: none), and
+    // that launch: outs[g], and inns[g * n_inns + k] for run g.  Same results as the runs
+    // one after the other.
+    virtual int  max_group() const { return 1; }
+    virtual void run_group(hipStream_t, int /*runs*/, void* const* /*outs*/,
+                           void const* const* /*inns*/) const
+    {
+        throw km_error(km_status::invalid, "this kernel does not take several runs at once");
+    }
     // Plans whose generated kernels were planned without being compiled (plan_codegen with
     // `defer`) add themselves: finish_codegen_plans compiles and loads them together.
     virtual void deferred(std::vector<plan_t*>&) {}

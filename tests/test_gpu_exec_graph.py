@@ -339,7 +339,8 @@ def test_optimized_layer_keeps_every_stored_bit(km, shape, n_streams):
     # rotary products (to_f32 in front, to_f16 behind) go into the products, which read and
     # write pairs of f16.
     assert fused.absorbed == 13 + 17 + 6 + 4, fused.absorbed
-    assert fused.graph.launches() == plain.graph.launches() - fused.absorbed
+    # (sibling projections that now follow each other may share a launch on top of that)
+    assert fused.graph.launches() <= plain.graph.launches() - fused.absorbed
     for k, v in vals.items():
         plain.set_input(k, v)
         fused.set_input(k, v)
@@ -500,3 +501,39 @@ def test_exec_graph_errors(km):
     g.finalize(2)
     with pytest.raises(ea.KmError):
         g.add_einsummable(e, [(0, 64), (64, 64)], deps=[a])      # immutable after finalize
+
+
+@pytest.mark.parametrize("m,n,k,runs", [(2048, 4096, 4096, 3), (2048, 11008, 4096, 2), (384, 512, 256, 5),
+                                         (1000, 3000, 4096, 2)])
+def test_sibling_products_in_one_launch(km, monkeypatch, m, n, k, runs):
+    """Independent products of one shape that follow each other (q, k and v of one input; w1
+    and w3) go out as one launch of the persistent kernel: the same bits as one by one."""
+    import torch
+
+    e = E.from_str("ij,kj->ik", dict(i=m, j=k, k=n), "*[hole|f16@0,hole|f16@1]", "+")
+    r = rng(m + runs)
+    x = normal(r, m * k, np.float16, 0.5)
+    ws = [normal(r, n * k, np.float16, 0.5) for _ in range(runs)]
+    sizes = [m * k * 2] + [n * k * 2] * runs + [m * n * 2] * runs
+    offs = np.concatenate([[0], np.cumsum([(s + 255) // 256 * 256 + 256 for s in sizes])]).astype(np.int64)
+    mem = lambda i: (int(offs[i]), sizes[i])
+    results = []
+    for grouped in (False, True):
+        monkeypatch.setenv("ES_KM_GEMM_GROUPS", "1" if grouped else "0")
+        g = ea.ApplyGraph(km)
+        ids = [g.add_einsummable(e, [mem(1 + runs + j), mem(0), mem(1 + j)]) for j in range(runs)]
+        g.add_memory_dependencies()
+        g.finalize(1)
+        if "waves=4+4 persistent" in km.describe(e) and (m // 128) * (n // 256) <= 256:
+            assert g.launches() == (1 if grouped else runs)
+        arena = torch.zeros(int(offs[-1]), dtype=torch.uint8, device="cuda")
+        arena[offs[0]:offs[0] + sizes[0]] = torch.from_numpy(x.view(np.uint8)).cuda()
+        for j, w in enumerate(ws):
+            arena[offs[1 + j]:offs[1 + j] + sizes[1 + j]] = torch.from_numpy(w.view(np.uint8)).cuda()
+        g.run(stream_handle(), arena.data_ptr())
+        torch.cuda.synchronize()
+        results.append(arena.cpu().numpy())
+    assert np.array_equal(results[0], results[1])
+    got = results[1][offs[1 + runs]:offs[1 + runs] + sizes[1 + runs]].view(np.float16).astype(np.float32)
+    want = x.astype(np.float32).reshape(m, k) @ ws[0].astype(np.float32).reshape(n, k).T
+    assert np.allclose(got.reshape(m, n), want, rtol=1e-2, atol=0.05 * np.sqrt(k) * 0.25)
