@@ -1075,6 +1075,10 @@ t0 = time.perf_counter()
 if mode == "graph":
     # the exec graph builds its distinct einsummables together (es_km_graph_finalize)
     ArenaRunner(km, g, n_streams=1)
+elif mode == "optimized":
+    # the same through the optimisation pass: merged einsummables and chains over rows are
+    # planned by the pass and compiled at finalize, as one program each
+    ArenaRunner(km, g, n_streams=1, optimize=True)
 else:
     for node in g.nodes:
         if node["kind"] == "einsummable":
@@ -1096,8 +1100,9 @@ def run_build_latency():
     root = os.path.dirname(os.path.abspath(__file__))
     out = {}
     runs = [("first_process_empty_cache", "graph", 0), ("second_process_cache_on_disk", "graph", 0),
-            ("one_build_call_after_the_other_empty_cache", "serial", 1)]
-    caches = [tempfile.mkdtemp(prefix="es_km_cache_") for _ in range(2)]
+            ("one_build_call_after_the_other_empty_cache", "serial", 1),
+            ("optimized_graph_first_process_empty_cache", "optimized", 2)]
+    caches = [tempfile.mkdtemp(prefix="es_km_cache_") for _ in range(3)]
     try:
         for label, mode, which in runs:
             env = dict(os.environ, ES_KM_CACHE_DIR=caches[which])

@@ -1871,7 +1871,7 @@ std::shared_ptr<plan_t> plan_codegen(einsummable_t const& e, int device, bool de
     return p;
 }
 
-std::shared_ptr<plan_t> plan_row_chain(cg_chain_t const& c, int device)
+std::shared_ptr<plan_t> plan_row_chain(cg_chain_t const& c, int device, bool defer)
 {
     auto p = std::make_shared<codegen_plan_t>();
     p->wide.k = generate_row_chain(c);  // throws ir_error when the chain has no kernel
@@ -1885,7 +1885,9 @@ std::shared_ptr<plan_t> plan_row_chain(cg_chain_t const& c, int device)
         p->has_narrow = false;  // rows too long for one element per lane and step
     }
     p->n_inns = p->wide.k.n_inns;
-    if (device >= 0) {
+    if (device >= 0 && defer) {
+        p->waiting = true;
+    } else if (device >= 0) {
         load_kernel(p->wide, device, {});
         if (p->has_narrow) load_kernel(p->narrow, device, {});
     }
@@ -1908,6 +1910,7 @@ void finish_codegen_plans(std::vector<plan_t*> const& plans, int device)
         std::set<std::string> seen;
         for (codegen_plan_t* p : ps) {
             for (variant_t* v : {&p->wide, &p->narrow}) {
+                if (v == &p->narrow && !p->has_narrow) continue;
                 if (seen.count(v->k.source) || module_loaded(device, v->k.source)) continue;
                 seen.insert(v->k.source);
                 fresh.push_back(v);
@@ -1956,7 +1959,7 @@ void finish_codegen_plans(std::vector<plan_t*> const& plans, int device)
     }
     for (codegen_plan_t* p : ps) {
         load_kernel(p->wide, device, {});
-        load_kernel(p->narrow, device, {});
+        if (p->has_narrow) load_kernel(p->narrow, device, {});
         p->waiting = false;
     }
 }

@@ -583,7 +583,8 @@ bool apply_graph_t::absorb_into_readers(int u)
             }
             if (km_) {
                 try {
-                    if (!km_->build(m.value())) return false;
+                    // (compiled at finalize, with the graph's other kernels)
+                    if (!km_->buildable(m.value())) return false;
                 } catch (km_error const&) {
                     return false;
                 } catch (ir_error const&) {
@@ -831,7 +832,8 @@ int apply_graph_t::fuse_row_chain(int v)
     std::shared_ptr<plan_t> plan;
     try {
         if (km_) check(hipSetDevice(km_->device()), "hipSetDevice");
-        plan = plan_row_chain(c, km_ ? km_->device() : -1);
+        // (compiled at finalize, all chains of the graph as one program)
+        plan = plan_row_chain(c, km_ ? km_->device() : -1, true);
     } catch (ir_error const&) {
         return 0;
     } catch (km_error const&) {
@@ -921,6 +923,15 @@ void apply_graph_t::finalize(int n_streams)
                 throw km_error(km_status::invalid, "apply graph: no kernel for an einsummable "
                                                    "(build returned unsupported)");
             }
+        }
+        // ... and so are the chains over rows that optimize() made
+        std::vector<plan_t*> waiting;
+        for (node_t const& nd : nodes_) {
+            if (nd.kind == kind_t::chain && nd.chain_plan) nd.chain_plan->deferred(waiting);
+        }
+        if (!waiting.empty()) {
+            check(hipSetDevice(km_->device()), "hipSetDevice");
+            finish_codegen_plans(waiting, km_->device());
         }
     }
 

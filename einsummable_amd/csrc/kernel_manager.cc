@@ -143,10 +143,32 @@ std::optional<uint64_t> kernel_manager_t::build(einsummable_t const& e_)
     auto          it = plans_.find(key);
     if (it != plans_.end()) return it->second->workspace_bytes;
 
-    std::shared_ptr<plan_t> p = make_plan(e);
+    std::shared_ptr<plan_t> p;
+    auto                    planned = planned_.find(key);
+    if (planned != planned_.end()) {
+        p = std::move(planned->second);
+        planned_.erase(planned);
+        std::vector<plan_t*> waiting;
+        p->deferred(waiting);
+        finish_codegen_plans(waiting, device_);
+    } else {
+        p = make_plan(e);
+    }
     if (!p) return std::nullopt;
     plans_.emplace(key, p);
     return p->workspace_bytes;
+}
+
+bool kernel_manager_t::buildable(einsummable_t const& e_)
+{
+    if (e_.join.has_variables()) return false;
+    einsummable_t     e = e_.merge_adjacent_dims();
+    std::string const key = e.key();
+    if (plans_.count(key) || planned_.count(key)) return true;
+    std::shared_ptr<plan_t> p = make_plan(e, true);
+    if (!p) return false;
+    planned_.emplace(key, std::move(p));
+    return true;
 }
 
 std::shared_ptr<plan_t> kernel_manager_t::make_plan(einsummable_t const& e, bool defer) const
@@ -175,7 +197,13 @@ std::vector<std::optional<uint64_t>> kernel_manager_t::build_many(
         keys[i] = merged.key();
         if (plans_.count(keys[i]) || seen.count(keys[i])) continue;
         seen.emplace(keys[i], fresh.size());
-        fresh.emplace_back(keys[i], make_plan(merged, true));
+        auto planned = planned_.find(keys[i]);
+        if (planned != planned_.end()) {
+            fresh.emplace_back(keys[i], std::move(planned->second));
+            planned_.erase(planned);
+        } else {
+            fresh.emplace_back(keys[i], make_plan(merged, true));
+        }
     }
     std::vector<plan_t*> waiting;
     for (auto const& kp : fresh) {

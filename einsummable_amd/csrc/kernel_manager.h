@@ -67,6 +67,10 @@ public:
     // error contract as build() called for each in turn; like build(), not to be called
     // concurrently.
     std::vector<std::optional<uint64_t>> build_many(std::vector<einsummable_t> const& es);
+    // Whether build() would succeed, without compiling anything: the plan is made (a generated
+    // kernel as source only) and kept for the build() or build_many() that follows, which
+    // compiles it -- build_many() with all the others as one program.
+    bool                    buildable(einsummable_t const& e);
     uint64_t                workspace_size(einsummable_t const& e) const;
     std::string             describe(einsummable_t const& e) const;
 
@@ -107,6 +111,7 @@ private:
 
     int                                                      device_;
     std::unordered_map<std::string, std::shared_ptr<plan_t>> plans_;      // by merged key
+    std::unordered_map<std::string, std::shared_ptr<plan_t>> planned_;    // by buildable(): not compiled yet
     std::unordered_map<std::string, std::shared_ptr<plan_t>> raw_plans_;  // by caller key
 };
 
@@ -118,10 +123,11 @@ std::shared_ptr<plan_t> plan_transpose(einsummable_t const& e, int device);
 // `defer`: generate the kernels' source only; finish_codegen_plans compiles and loads
 std::shared_ptr<plan_t> plan_codegen(einsummable_t const& e, int device, bool defer = false);
 // The kernel of a chain of nodes over rows (codegen.h: cg_chain_t), compiled and loaded on
-// `device` (a negative device: generated only, for inspection).  run() takes the last node's
+// `device` (a negative device: generated only, for inspection; `defer`: compiled and loaded by
+// finish_codegen_plans, with the other kernels of its list).  run() takes the last node's
 // output and the chain's inputs.  Throws ir_error when the chain has no such kernel.
 struct cg_chain_t;
-std::shared_ptr<plan_t> plan_row_chain(cg_chain_t const& c, int device);
+std::shared_ptr<plan_t> plan_row_chain(cg_chain_t const& c, int device, bool defer = false);
 // Compiles the generated kernels of all these plans as ONE runtime-compiled program (the
 // compiler's fixed cost per program is most of the time of a small kernel, and it compiles
 // one program at a time whatever the number of calling threads: the 25 distinct generated
