@@ -488,6 +488,9 @@ cg_kernel_t gen_elementwise(einsummable_t const& e, int max_vec)
     int widest = g.storage_size(0);
     for (int k = 0; k != int(e.inns.size()); ++k) {
         if (acc[k] == access_t::bcast) continue;
+        // (a small input that every row reads again comes from the caches whatever its
+        // access width: the rotary product's frequencies beside its f16 pairs)
+        if (e.any_half_pairs() && e.inn_nelem(k) * 8 <= n_out) continue;
         widest = std::max(widest, g.storage_size(1 + k));
     }
     int const vcap = std::min(max_vec, 16 / widest);
