@@ -747,6 +747,24 @@ int64_t es_km_graph_node_describe(es_km_graph_t* g, int id, char* out, uint64_t 
     return int64_t(s.size());
 }
 
+int64_t es_km_graph_node_source(es_km_graph_t* g, int id, int compile, char* out, uint64_t cap)
+{
+    if (!g || id < 0 || id >= g->graph->n_nodes()) return ES_KM_ERR_INVALID;
+    int64_t   length = 0;
+    int const rc = guarded(g->owner, [&]() -> int {
+        std::string const s = g->graph->generated_source(id);
+        if (compile && !s.empty()) es::compile_hip_source(s, "es_generated.hip", "gfx950");
+        if (out && cap) {
+            uint64_t const n = std::min<uint64_t>(cap - 1, s.size());
+            std::memcpy(out, s.data(), n);
+            out[n] = 0;
+        }
+        length = int64_t(s.size());
+        return ES_KM_OK;
+    });
+    return rc < 0 ? rc : length;
+}
+
 int es_km_graph_launches(es_km_graph_t* g)
 {
     return g ? g->graph->n_launches() : ES_KM_ERR_INVALID;

@@ -1744,6 +1744,7 @@ struct codegen_plan_t : plan_t {
 
     explicit codegen_plan_t(einsummable_t const& e_) : e(e_) {}
     codegen_plan_t() = default;  // a chain of einsummables
+    std::string source() const override { return wide.k.source; }
     bool has_narrow = true;
     bool waiting = false;  // the variants' kernels are not loaded yet
     void deferred(std::vector<plan_t*>& out) override

@@ -238,6 +238,20 @@ std::string apply_graph_t::describe(int id) const
     return s;
 }
 
+std::string apply_graph_t::generated_source(int id) const
+{
+    node_t const& n = nodes_[size_t(id)];
+    if (n.kind == kind_t::chain) return n.chain_plan ? n.chain_plan->source() : std::string();
+    if (n.kind != kind_t::einsummable) return std::string();
+    einsummable_t const e = n.e.merge_adjacent_dims();
+    if (e.is_contraction() || e.join.has_variables()) return std::string();
+    try {
+        return generate_kernel(e).source;
+    } catch (ir_error const&) {
+        return std::string();
+    }
+}
+
 uint64_t apply_graph_t::arena_bytes() const
 {
     uint64_t need = 0;

@@ -137,6 +137,10 @@ public:
     // "<kind> <range>..." -- the output first, "offset:size" each -- and for an einsummable
     // its key (shape, castable, modes, join text) after " | "; for inspection and tests
     std::string describe(int id) const;
+    // The HIP source of the kernel the code generator makes for node `id` -- an einsummable
+    // it would take (what optimize() merged included) or a chain over rows -- empty for any
+    // other node.  Works without a kernel manager and before finalize: an aid for tests.
+    std::string generated_source(int id) const;
 
     int n_nodes() const { return int(nodes_.size()); }
     // smallest arena that holds every range a node touches

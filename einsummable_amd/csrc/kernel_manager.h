@@ -43,6 +43,8 @@ struct plan_t {
     // How many runs of this plan on different buffers one launch can take (1: none), and
     // that launch: outs[g], and inns[g * n_inns + k] for run g.  Same results as the runs
     // one after the other.
+    // the HIP source of a generated kernel (its vector variant), empty for the others
+    virtual std::string source() const { return std::string(); }
     virtual int  max_group() const { return 1; }
     virtual void run_group(hipStream_t, int /*runs*/, void* const* /*outs*/,
                            void const* const* /*inns*/) const

@@ -38,6 +38,7 @@ EXPORTS = [
     "es_km_graph_add_memory_dependencies",
     "es_km_graph_optimize",
     "es_km_graph_node_describe",
+    "es_km_graph_node_source",
     "es_km_graph_finalize",
     "es_km_graph_run",
     "es_km_graph_node_info",
@@ -200,6 +201,8 @@ def load_library():
     lib.es_km_graph_optimize.argtypes = [V, ctypes.POINTER(ctypes.c_int)]
     lib.es_km_graph_node_describe.restype = ctypes.c_int64
     lib.es_km_graph_node_describe.argtypes = [V, I, ctypes.c_char_p, U64]
+    lib.es_km_graph_node_source.restype = ctypes.c_int64
+    lib.es_km_graph_node_source.argtypes = [V, I, I, ctypes.c_char_p, U64]
     lib.es_km_graph_finalize.argtypes = [V, I]
     lib.es_km_graph_run.argtypes = [V, V, V]
     lib.es_km_graph_node_info.argtypes = [V, I, V, V, V, I, V]
@@ -647,6 +650,14 @@ class ApplyGraph:
         n = self._lib.es_km_graph_node_describe(self._g, int(node), buf, len(buf))
         if n < 0:
             raise KmError(int(n), "no such node")
+        return buf.value.decode()
+
+    def node_source(self, node, compile=False):
+        """HIP source of the generated kernel of a node ("" when it has none); `compile`
+        also compiles it for gfx950, which needs no device."""
+        buf = ctypes.create_string_buffer(1 << 17)
+        n = self._lib.es_km_graph_node_source(self._g, int(node), int(compile), buf, len(buf))
+        self._check(n)
         return buf.value.decode()
 
     def cross_stream_waits(self):

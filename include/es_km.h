@@ -265,6 +265,13 @@ int es_km_graph_cross_stream_waits(es_km_graph_t* g);
  * scalarop's operator<<, src/einsummable/scalarop.cc:2881-3011).  Writes at most cap-1
  * characters and a terminator; returns the full length, negative for a bad id. */
 int64_t es_km_graph_node_describe(es_km_graph_t* g, int id, char* out, uint64_t cap);
+/* Test aid, like es_km_codegen_source: the HIP source of the generated kernel of a node (an
+ * elementwise or reduction einsummable, what es_km_graph_optimize merged included, or a chain
+ * over rows), empty for any other node; with `compile` it is also compiled for gfx950 (no
+ * device needed).  Returns the full length, negative on an error (a failed compile:
+ * ES_KM_ERR_DEVICE, text in es_km_last_error of the graph's manager, or of NULL).  No
+ * counterpart in the reference. */
+int64_t es_km_graph_node_source(es_km_graph_t* g, int id, int compile, char* out, uint64_t cap);
 /* After finalize: launches one run makes.  Touches of one group that follow each other in
  * insertion order and write the same output range count once: they run as one
  * es_km_touch_batch launch, with the bytes of one launch per touch

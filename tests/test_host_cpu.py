@@ -388,6 +388,10 @@ def test_exec_graph_optimize_makes_one_launch_of_a_chain_over_rows():
     assert g.optimize() == 2
     assert g.describe(a).startswith("dummy") and g.describe(b).startswith("dummy")
     assert g.describe(c).startswith("chain 262144:32768 0:32768 65536:8192 | 3 stages, the last [4,64,64]:")
+    # the chain's kernel: three joins, the statistics never stored, and it compiles for gfx950
+    src = g.node_source(c, compile=True)
+    assert all(("join_fn%d(" % t) in src for t in range(3)) and "es_rowchain__3stages_2inputs__f16" in src
+    assert src.count("a.out") == 1 and "__expf" in src
     g.finalize(1)
     assert g.launches() == 1
     assert g.node_mems(c)[0] == "chain"
@@ -438,6 +442,8 @@ def test_exec_graph_optimize_absorbs_conversions_around_a_complex_view():
     assert g.describe(a).startswith("dummy") and g.describe(b).startswith("dummy")
     assert g.describe(c) == ("einsummable 32768:1024 0:1024 8192:1024 | [1,16,2,8]: 0.1.2.3.,1.3.->4 | "
                              "*[to_c64[hole|c64@0],hole|c64@1] | f16 pairs: out in0")
+    src = g.node_source(c, compile=True)        # pairs of f16 in and out, and it compiles
+    assert "const h2* in0;" in src and "h2* out;" in src and "narrow_c64(" in src
     g.finalize(1)
     assert g.launches() == 1
     # one side only
