@@ -411,6 +411,46 @@ def test_exec_graph_optimize_makes_one_launch_of_a_chain_over_rows():
     assert g.describe(c).startswith("chain 262144:32768 0:32768 65536:8192 131072:1024 | 2 stages")
 
 
+def test_exec_graph_optimize_declines_chains_it_cannot_run_as_one_kernel():
+    import einsummable_amd as ea
+
+    E = ea.Einsummable
+    m = lambda slot, nbytes: (slot * (1 << 20), nbytes)
+
+    def softmax(rows, n, x_modes=None, align=0, out_on=None):
+        """max, sum of exp(x - max), quotient over [rows, n] f32; returns (graph, absorbed)"""
+        g = ea.ApplyGraph(None)
+        xm = x_modes or [0, 1]
+        shape = [rows, n]
+        sub = "+[hole|f32@0,*[constant{f32|-1},hole|f32@1]]"
+        rmax = E(shape, [xm], 1, "hole|f32@0", "^")
+        rsum = E(shape, [xm, [0]], 1, "exp[" + sub + "]", "+")
+        norm = E(shape, [xm, [0], [0]], 2, "*[exp[" + sub + "],power{-1}[hole|f32@2]]")
+        X = (m(0, 4 * rows * n)[0] + align, 4 * rows * n)
+        mx, l = m(1, 4 * rows), m(2, 4 * rows)
+        P = m(3, 4 * rows * n) if out_on is None else out_on(X, mx)
+        a = g.add_einsummable(rmax, [mx, X])
+        b = g.add_einsummable(rsum, [l, X, mx])
+        c = g.add_einsummable(norm, [P, X, mx, l])
+        g.add_dummy(mx, [b, c])
+        g.add_dummy(l, [c])
+        g.add_memory_dependencies()
+        return g, g.optimize()
+
+    assert softmax(64, 512)[1] == 2
+    # rows too long for a team's registers (more than eight vectors per lane)
+    assert softmax(4, 1 << 15)[1] == 0
+    # the tensor read across its rows (modes permuted): the statistics need a gather
+    assert softmax(64, 64, x_modes=[1, 0])[1] == 0
+    # buffers off the 16-byte grid
+    assert softmax(64, 512, align=4)[1] == 0
+    # the output on half of the input: neither apart from it nor exactly on it
+    assert softmax(64, 512, out_on=lambda X, mx: (X[0] + X[1] // 2, X[1]))[1] == 0
+    # the output exactly on the input is fine (every row is read before it is written)
+    g, n = softmax(64, 512, out_on=lambda X, mx: X)
+    assert n == 2 and g.describe(2).startswith("chain 0:131072 0:131072 |")
+
+
 def test_exec_graph_optimize_absorbs_conversions_around_a_complex_view():
     """to_f32, a complex product on the buffer seen as c64, to_f16: the product takes the f16
     tensor in and writes the f16 tensor out."""
